@@ -1,0 +1,108 @@
+/*
+ * C ABI of librode_hip.so -- RoDe row-decomposition preprocessing, SpMM and
+ * SDDMM for AMD MI355X (gfx950).
+ *
+ * Plain pointers and sizes only.  Every pointer named d_* is DEVICE memory
+ * owned by the caller; nothing here allocates or frees, and nothing
+ * synchronises with the host: all work is queued on the streams passed in
+ * (a `void*` stream is a hipStream_t; NULL is HIP's default stream).
+ * Return value: 0 on success, otherwise a hipError_t value
+ * (rode_hip_error_string() turns it into text).
+ *
+ * Layout and alignment contract (same as the reference kernels, which use
+ * 128-bit accesses throughout, e.g. RoDe_SpMM/RoDeSpmm.cu:89,247-248 and
+ * RoDe_SDDMM/RoDeSddmm.cu:75,80,88): all arrays row-major and 16-byte aligned.
+ */
+#ifndef RODE_HIP_H_
+#define RODE_HIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Library version, (major << 16) | minor. */
+int rode_hip_version(void);
+
+/* Text for a code returned by the functions below. */
+const char* rode_hip_error_string(int code);
+
+/*
+ * Scratch bytes rode_hip_preprocess() needs for a matrix of M rows
+ * (replaces the cudaMalloc/cudaFree of CUB temp storage inside the reference's
+ * GPU preprocess, Preprocess_opt/_preprocess.cu:325-335).
+ */
+size_t rode_hip_preprocess_workspace_bytes(int M);
+
+/*
+ * Row decomposition on the GPU.
+ * Replaces RoDe_preprocess (GPU), Preprocess_opt/_preprocess.cu:323-339, and
+ * produces the arrays of the CPU routine RoDe_SDDMM/main.cu:114-163 bit for
+ * bit, sentinel d_st_off[n_blk] = row_ptr[M] included.
+ *   seg_length, k_block, vec_len : decomposition parameters, order of
+ *                                  _preprocess.cu:323 (512,32,4 or 32,32,4 in the reference)
+ *   d_row_ptr        int[M+1]    CSR row pointer
+ *   d_block_r_ind    int[cap]    out: row of every block segment
+ *   d_st_off         int[cap+1]  out: first nonzero of every block segment, then the sentinel
+ *   d_residue_r_ind  int[>=M]    out: rows that own a residue
+ *   d_n_blk, d_n_res int[1] each out: segment / residue counts
+ *   capacity_blocks  cap above; must be >= (nnz + (vec_len-1)*M)/seg_length + M
+ *                    (the reference sizes it nnz/seg + M, _preprocess.cu:426)
+ *   d_workspace      rode_hip_preprocess_workspace_bytes(M) bytes, 8-byte aligned
+ */
+int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const int* d_row_ptr,
+                        int* d_block_r_ind, int* d_st_off, int* d_residue_r_ind, int* d_n_blk, int* d_n_res,
+                        int capacity_blocks, void* d_workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * SpMM  C[M x n] += A_csr[M x k] * B[k x n]  (fp32 values, fp32 or fp16 dense B,
+ * fp32 accumulate and output).
+ * Replaces RoDeSpmm_n32 / RoDeSpmm_n128 (fp32), RoDe_SpMM/RoDeSpmm.h:4-8,
+ * RoDeSpmm.cu:511-519: the block-segment kernel runs on stream1 over m1
+ * segments, the residue kernel on stream2 over m2 rows.  As in the reference
+ * C must be zero on entry: segments and tails of long rows are added with
+ * atomics, short rows are stored, rows without nonzeros are not touched.
+ * n must be a multiple of 32 (the reference tiles are 32 / 64 wide and
+ * unguarded); the decomposition must have been made with k_block 32, vec_len 4.
+ */
+int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
+                      const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
+                      const int* d_row_seg_st_offsets, const float* d_B, float* d_C, void* stream1,
+                      void* stream2);
+
+/* Same with B stored as IEEE fp16 (no reference entry point; operand semantics of the
+ * unused helper VectorCompute<half4>::FMA, RoDe_SpMM/common_utils.h:183-230:
+ * widen to fp32, fp32 FMA). */
+int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
+                      const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
+                      const int* d_row_seg_st_offsets, const void* d_B_half, float* d_C, void* stream1,
+                      void* stream2);
+
+/*
+ * SDDMM  out[idx] = values[idx] * <lhs[row(idx),:], rhs[col(idx),:]>.
+ * Replaces RoDeSDDMM_n32 / RoDeSDDMM_n128, RoDe_SDDMM/RoDeSddmm.h:4-9,
+ * RoDeSddmm.cu:496-545.  k must be 32, 64 or 128 (the reference has 32 and
+ * 128).  Segments may have any length that the decomposition produced, so one
+ * entry point serves both reference parameter sets (512,32,4) and (32,32,4).
+ * Every out[idx], idx < nnz, is written exactly once; out needs no clearing.
+ * A launch is skipped only when its count is zero (the reference also skips it
+ * when the stream handle is NULL, RoDeSddmm.cu:503,509; here NULL is the
+ * default stream).
+ */
+int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_block,
+                       const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
+                       const int* d_column_indices, const float* d_values, const float* d_lhs_matrix,
+                       const float* d_rhs_matrix, float* d_out, void* stream1, void* stream2);
+
+/* Same with lhs / rhs stored as IEEE fp16, fp32 accumulate (no reference entry point). */
+int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_block,
+                       const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
+                       const int* d_column_indices, const float* d_values, const void* d_lhs_half,
+                       const void* d_rhs_half, float* d_out, void* stream1, void* stream2);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RODE_HIP_H_ */

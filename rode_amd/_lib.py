@@ -1,0 +1,50 @@
+"""Loader of ``librode_hip.so`` (the C ABI declared in ``include/rode_hip.h``).
+
+There is no fallback: if the library has not been built, or a call returns an
+error code, a ``RuntimeError`` is raised.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "librode_hip.so")
+WORKLOADS_PATH = os.path.join(_HERE, "lib", "librode_workloads.so")
+
+c_int, c_void_p, c_size_t = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+
+# name -> (restype, argtypes); must list every symbol include/rode_hip.h declares.
+SIGNATURES = {
+    "rode_hip_version": (c_int, []),
+    "rode_hip_error_string": (ctypes.c_char_p, [c_int]),
+    "rode_hip_preprocess_workspace_bytes": (c_size_t, [c_int]),
+    "rode_hip_preprocess": (c_int, [c_int] * 4 + [c_void_p] * 6 + [c_int, c_void_p, c_size_t, c_void_p]),
+    "rode_hip_spmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 10),
+    "rode_hip_spmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 10),
+    "rode_hip_sddmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 11),
+    "rode_hip_sddmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 11),
+}
+
+_lib = None
+
+
+def load():
+    """Return the ctypes handle of ``librode_hip.so`` (loaded once)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C rode_amd/csrc` "
+                "(or `python -c 'import __graft_entry__ as g; g.build()'`); there is no CPU fallback"
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def check(code, what):
+    if code != 0:
+        msg = load().rode_hip_error_string(code).decode()
+        raise RuntimeError(f"{what} failed: {msg} (hipError {code})")

@@ -1,0 +1,162 @@
+// extern "C" boundary of librode_hip.so plus the C++ entry points that keep the
+// reference's signatures.  No kernel code here.
+#include "../../include/rode_hip.h"
+#include "../../include/RoDePreprocess.h"
+#include "../../include/RoDeSddmm.h"
+#include "../../include/RoDeSpmm.h"
+#include "rode_internal.hpp"
+
+#include <cstdio>
+
+namespace {
+
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+} // namespace
+
+extern "C" {
+
+int rode_hip_version(void) { return (0 << 16) | 1; }
+
+const char* rode_hip_error_string(int code) { return hipGetErrorString(static_cast<hipError_t>(code)); }
+
+size_t rode_hip_preprocess_workspace_bytes(int M) { return rode::preprocess_workspace_bytes(M); }
+
+int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const int* d_row_ptr, int* d_block_r_ind,
+                        int* d_st_off, int* d_residue_r_ind, int* d_n_blk, int* d_n_res, int capacity_blocks,
+                        void* d_workspace, size_t workspace_bytes, void* stream)
+{
+    if (seg_length <= 0 || k_block <= 0 || vec_len <= 0 || M < 0 || capacity_blocks < 0) return hipErrorInvalidValue;
+    if (!d_row_ptr || !d_block_r_ind || !d_st_off || !d_residue_r_ind || !d_n_blk || !d_n_res || !d_workspace)
+        return hipErrorInvalidValue;
+    if (workspace_bytes < rode::preprocess_workspace_bytes(M) || (reinterpret_cast<uintptr_t>(d_workspace) & 7u))
+        return hipErrorInvalidValue;
+    return rode::preprocess_launch(seg_length, k_block, vec_len, M, d_row_ptr, d_block_r_ind, d_st_off,
+                                   d_residue_r_ind, d_n_blk, d_n_res, d_workspace, capacity_blocks, as_stream(stream));
+}
+
+int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
+                      const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
+                      const int* d_row_seg_st_offsets, const float* d_B, float* d_C, void* stream1, void* stream2)
+{
+    (void)k;
+    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
+    if (m1 == 0 && m2 == 0) return hipSuccess;
+    if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
+    return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
+                                    d_column_indices, d_values, d_B, d_C, as_stream(stream1), as_stream(stream2));
+}
+
+int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
+                      const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
+                      const int* d_row_seg_st_offsets, const void* d_B_half, float* d_C, void* stream1,
+                      void* stream2)
+{
+    (void)k;
+    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
+    if (m1 == 0 && m2 == 0) return hipSuccess;
+    if (!aligned16(d_B_half) || !aligned16(d_C)) return hipErrorInvalidValue;
+    return rode::spmm_launch<__half>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
+                                     d_column_indices, d_values, static_cast<const __half*>(d_B_half), d_C,
+                                     as_stream(stream1), as_stream(stream2));
+}
+
+int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,
+                       const int* d_st_offsets, const int* d_row_offsets, const int* d_column_indices,
+                       const float* d_values, const float* d_lhs_matrix, const float* d_rhs_matrix, float* d_out,
+                       void* stream1, void* stream2)
+{
+    (void)n;
+    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
+    if (m1 == 0 && m2 == 0) return hipSuccess;
+    if (!aligned16(d_lhs_matrix) || !aligned16(d_rhs_matrix)) return hipErrorInvalidValue;
+    return rode::sddmm_launch<float>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
+                                     d_row_offsets, d_column_indices, d_values, d_lhs_matrix, d_rhs_matrix, d_out,
+                                     as_stream(stream1), as_stream(stream2));
+}
+
+int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,
+                       const int* d_st_offsets, const int* d_row_offsets, const int* d_column_indices,
+                       const float* d_values, const void* d_lhs_half, const void* d_rhs_half, float* d_out,
+                       void* stream1, void* stream2)
+{
+    (void)n;
+    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
+    if (m1 == 0 && m2 == 0) return hipSuccess;
+    if (!aligned16(d_lhs_half) || !aligned16(d_rhs_half)) return hipErrorInvalidValue;
+    return rode::sddmm_launch<__half>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
+                                      d_row_offsets, d_column_indices, d_values,
+                                      static_cast<const __half*>(d_lhs_half), static_cast<const __half*>(d_rhs_half),
+                                      d_out, as_stream(stream1), as_stream(stream2));
+}
+
+} // extern "C"
+
+// ---- reference-signature C++ entry points ----------------------------------
+// The reference functions return void and check nothing (RoDeSpmm.cu:505-508,
+// RoDeSddmm.cu:503-512); a failure here is at least reported on stderr.
+namespace {
+void report(const char* fn, int code)
+{
+    if (code != 0) std::fprintf(stderr, "%s: %s\n", fn, rode_hip_error_string(code));
+}
+} // namespace
+
+void RoDeSpmm_n32(int m1, int m2, int k, int n, const float* values, const int* column_indices, const int* row_offsets,
+                  const int* row_indices1, const int* row_indices2, const int* row_seg_st_offsets, const float* B,
+                  float* C, hipStream_t stream1, hipStream_t stream2)
+{
+    report("RoDeSpmm_n32", rode_hip_spmm_f32(m1, m2, k, n, values, column_indices, row_offsets, row_indices1,
+                                             row_indices2, row_seg_st_offsets, B, C, stream1, stream2));
+}
+
+void RoDeSpmm_n128(int m1, int m2, int k, int n, const float* values, const int* column_indices, const int* row_offsets,
+                   const int* row_indices1, const int* row_indices2, const int* row_seg_st_offsets, const float* B,
+                   float* C, hipStream_t stream1, hipStream_t stream2)
+{
+    report("RoDeSpmm_n128", (n % 64) ? (int)hipErrorInvalidValue
+                                     : rode_hip_spmm_f32(m1, m2, k, n, values, column_indices, row_offsets,
+                                                         row_indices1, row_indices2, row_seg_st_offsets, B, C,
+                                                         stream1, stream2));
+}
+
+void RoDeSDDMM_n32(int m1, int m2, int n, int k, const int* row_indices_block, const int* row_indices_residue,
+                   const int* st_offsets, const int* row_offsets, const int* column_indices, const float* values,
+                   const float* lhs_matrix, const float* rhs_matrix, float* out, hipStream_t stream1,
+                   hipStream_t stream2)
+{
+    report("RoDeSDDMM_n32", k != 32 ? (int)hipErrorInvalidValue
+                                    : rode_hip_sddmm_f32(m1, m2, n, k, row_indices_block, row_indices_residue,
+                                                         st_offsets, row_offsets, column_indices, values, lhs_matrix,
+                                                         rhs_matrix, out, stream1, stream2));
+}
+
+void RoDeSDDMM_n128(int m1, int m2, int n, int k, const int* row_indices_block, const int* row_indices_residue,
+                    const int* st_offsets, const int* row_offsets, const int* column_indices, const float* values,
+                    const float* lhs_matrix, const float* rhs_matrix, float* out, hipStream_t stream1,
+                    hipStream_t stream2)
+{
+    report("RoDeSDDMM_n128", k != 128 ? (int)hipErrorInvalidValue
+                                      : rode_hip_sddmm_f32(m1, m2, n, k, row_indices_block, row_indices_residue,
+                                                           st_offsets, row_offsets, column_indices, values,
+                                                           lhs_matrix, rhs_matrix, out, stream1, stream2));
+}
+
+void RoDe_preprocess(int N_SEG, int blockX, int vecLen, int M, const int* row_ptr, int* block_r_ind, int* st_off,
+                     int* residue_r_ind, int* n_blk, int* n_res)
+{
+    void* ws = nullptr;
+    const size_t bytes = rode_hip_preprocess_workspace_bytes(M);
+    hipError_t e = hipMalloc(&ws, bytes);
+    if (e != hipSuccess) {
+        report("RoDe_preprocess", (int)e);
+        return;
+    }
+    // The signature carries no capacity: the caller's arrays are trusted to hold
+    // the result, as in the reference.
+    report("RoDe_preprocess", rode_hip_preprocess(N_SEG, blockX, vecLen, M, row_ptr, block_r_ind, st_off,
+                                                  residue_r_ind, n_blk, n_res, 0x7fffffff, ws, bytes, nullptr));
+    (void)hipFree(ws); // waits for the queued kernels
+}

@@ -1,0 +1,113 @@
+// Device-side helpers shared by the RoDe kernels (gfx950 / CDNA4, wave64 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+namespace rode {
+
+constexpr int kWave = 64;         // lanes per wavefront
+constexpr int kWavesPerWg = 4;    // every kernel here launches 256-thread workgroups
+constexpr int kWgThreads = kWave * kWavesPerWg;
+constexpr int kXcds = 8;          // MI355X: 8 XCDs, each with its own L2
+constexpr int kBlockItems = 32;   // k_block the kernels are written for (RoDeSpmm.cu:513, RoDeSddmm.cu:517)
+constexpr int kVecLen = 4;        // vec_len the kernels are written for (128-bit sparse loads)
+
+// Workgroups are dealt round-robin to the XCDs, so neighbouring blockIdx values
+// land on different L2s.  Remap so that a contiguous range of logical ids shares
+// one XCD (neighbouring sparse rows touch neighbouring dense rows).  The grid
+// must be a multiple of kXcds; ids past the item count are discarded by the
+// caller's bounds check.
+__device__ __forceinline__ int xcd_logical_block(int bid, int nblocks)
+{
+    const int per_xcd = nblocks / kXcds;
+    return (bid % kXcds) * per_xcd + bid / kXcds;
+}
+
+// ---- cross-lane exchanges ------------------------------------------------
+// xor 1 / xor 2 inside a quad: DPP quad_perm, full rate on the VALU.
+__device__ __forceinline__ float lane_xor1(float v)
+{
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1 /*[1,0,3,2]*/, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lane_xor2(float v)
+{
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E /*[2,3,0,1]*/, 0xF, 0xF, true));
+}
+// xor 4 / 8 / 16: ds_swizzle in bit-mask mode (and=0x1f, or=0, xor=mask); no LDS memory is touched.
+__device__ __forceinline__ float lane_xor4(float v)
+{
+    return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (4 << 10) | 0x1F));
+}
+__device__ __forceinline__ float lane_xor8(float v)
+{
+    return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (8 << 10) | 0x1F));
+}
+__device__ __forceinline__ float lane_xor16(float v)
+{
+    return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (16 << 10) | 0x1F));
+}
+// xor 32: swap the two 32-lane halves of the wave.
+__device__ __forceinline__ float lane_xor32(float v)
+{
+    return __shfl_xor(v, 32, kWave);
+}
+
+// Sum over the lanes l ^ m for every power of two m with LO <= m < HI.
+// Every lane ends up with the total of its group.
+template <int LO, int HI>
+__device__ __forceinline__ float butterfly_sum(float v)
+{
+    if (LO <= 1 && 1 < HI) v += lane_xor1(v);
+    if (LO <= 2 && 2 < HI) v += lane_xor2(v);
+    if (LO <= 4 && 4 < HI) v += lane_xor4(v);
+    if (LO <= 8 && 8 < HI) v += lane_xor8(v);
+    if (LO <= 16 && 16 < HI) v += lane_xor16(v);
+    if (LO <= 32 && 32 < HI) v += lane_xor32(v);
+    return v;
+}
+
+// ---- dense operand access --------------------------------------------------
+// One lane reads DenseVec<T>::kElems consecutive dense elements with a single
+// 128-bit load and widens them to fp32.
+template <typename T>
+struct DenseVec;
+
+template <>
+struct DenseVec<float> {
+    static constexpr int kElems = 4;
+    __device__ __forceinline__ static void load(const float* p, float (&out)[4])
+    {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    }
+};
+
+template <>
+struct DenseVec<__half> {
+    static constexpr int kElems = 8;
+    __device__ __forceinline__ static void load(const __half* p, float (&out)[8])
+    {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const __half2 h = *reinterpret_cast<const __half2*>(&w[i]);
+            const float2 f = __half22float2(h);
+            out[2 * i] = f.x;
+            out[2 * i + 1] = f.y;
+        }
+    }
+};
+
+// Make LDS writes of this wave visible to its other lanes.  A wave executes its
+// LDS instructions in order, so only the compiler has to be kept from moving
+// accesses across this point.
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+} // namespace rode

@@ -1,0 +1,25 @@
+// Launch functions behind the C ABI (one per kernel family).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stddef.h>
+
+namespace rode {
+
+size_t preprocess_workspace_bytes(int M);
+
+hipError_t preprocess_launch(int seg, int kblock, int veclen, int M, const int* row_ptr, int* block_r_ind,
+                             int* st_off, int* residue_r_ind, int* n_blk, int* n_res, void* workspace,
+                             int capacity_blocks, hipStream_t stream);
+
+template <typename T>
+hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
+                       const int* row_ptr, const int* col, const float* val, const T* B, float* C, hipStream_t s1,
+                       hipStream_t s2);
+
+template <typename T>
+hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int* residue_rows, const int* st_off,
+                        const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs,
+                        float* out, hipStream_t s1, hipStream_t s2);
+
+} // namespace rode

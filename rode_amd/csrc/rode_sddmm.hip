@@ -1,0 +1,213 @@
+// SDDMM over a row-decomposed CSR pattern:
+//     out[idx] = values[idx] * < lhs[row(idx), :], rhs[col(idx), :] >
+// Same work split and index arithmetic as the reference's SDDMMKernel4Block
+// (RoDe_SDDMM/RoDeSddmm.cu:15-203) and SDDMMKernel4Residue (:206-494); the
+// execution shape is written for 64-lane wavefronts:
+//
+//   * a "unit" is 32 consecutive nonzero slots handled by one 32-lane half of a
+//     wave: lane e of the half owns slot e (its column index, its value, its
+//     output), so sparse loads and the final store are fully coalesced;
+//   * inside a half, groups of LPR = K / (elements per 128-bit load) lanes read
+//     one dense rhs row per load instruction, LPR rows per group per unit;
+//   * the K-slices of four rows at a time are combined with a transpose-reduce
+//     (DPP quad_perm for xor 1/2, ds_swizzle for xor 4/8/16) that leaves the dot
+//     product of slot e in lane e;
+//   * block kernel: one wave walks one block segment, 64 slots per step, the
+//     lhs row slice stays in registers for the whole segment;
+//   * residue kernel: each half-wave takes one residue row (< 32 slots).
+#include "rode_device.hpp"
+#include "rode_internal.hpp"
+
+namespace rode {
+
+namespace {
+
+template <typename T, int K>
+struct SddmmShape {
+    static constexpr int kVec = DenseVec<T>::kElems;
+    static constexpr int kLpr = K / kVec;      // lanes that cover one dense row
+    static constexpr int kQuads = kLpr / 4;    // slot quads per lane group per unit
+    static_assert(K % kVec == 0 && kLpr >= 4 && kLpr <= 32 && (kLpr & (kLpr - 1)) == 0,
+                  "unsupported K for this dense type");
+};
+
+// Dot products of one 32-slot unit.  `my_col` is the column of this lane's
+// slot; `nslots` (half-uniform) is how many leading slots of the half need a
+// result.  Returns the dot product for this lane's slot (0 for slots that were
+// skipped).  FULL promises nslots == 32 and removes the per-quad tests.
+template <typename T, int K, bool FULL>
+__device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane, const float (&a)[SddmmShape<T, K>::kVec],
+                                            int my_col, int nslots, int* lds_cols, int lane)
+{
+    using S = SddmmShape<T, K>;
+    constexpr int VEC = S::kVec, LPR = S::kLpr;
+
+    lds_cols[lane] = my_col;
+    wave_lds_sync();
+
+    const int ls = lane % LPR;                    // lane inside its group
+    const int group_first = (lane & 31) - ls;     // first slot (within the half) of this group
+    const int* group_cols = lds_cols + (lane & 32) + group_first;
+    float result = 0.f;
+
+#pragma unroll
+    for (int q = 0; q < S::kQuads; ++q) {
+        if (FULL || group_first + 4 * q < nslots) {
+            const int4 c4 = *reinterpret_cast<const int4*>(group_cols + 4 * q);
+            const int c[4] = {c4.x, c4.y, c4.z, c4.w};
+            float p[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float b[VEC];
+                DenseVec<T>::load(rhs_lane + (size_t)c[j] * K, b);
+                float d = 0.f;
+#pragma unroll
+                for (int x = 0; x < VEC; ++x) d = fmaf(a[x], b[x], d);
+                p[j] = d;
+            }
+            // transpose-reduce: afterwards lane (ls & 3) == j holds slot j of the quad
+            const bool hi2 = ls & 2, hi1 = ls & 1;
+            const float k0 = hi2 ? p[2] : p[0], s0 = hi2 ? p[0] : p[2];
+            const float k1 = hi2 ? p[3] : p[1], s1 = hi2 ? p[1] : p[3];
+            const float q0 = k0 + lane_xor2(s0);
+            const float q1 = k1 + lane_xor2(s1);
+            float r = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
+            r = butterfly_sum<4, LPR>(r);
+            if ((ls >> 2) == q) result = r;
+        }
+    }
+    return result;
+}
+
+template <typename T, int K>
+__device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int row, int lane,
+                                               float (&a)[SddmmShape<T, K>::kVec])
+{
+    using S = SddmmShape<T, K>;
+    DenseVec<T>::load(lhs + (size_t)row * K + (lane % S::kLpr) * S::kVec, a);
+}
+
+// One wave per block segment.  Segment s covers the aligned slots
+// [base, base + cnt) with base = st_off[s] & ~3 and cnt = floor((len + mask) / 32) * 32
+// (RoDeSddmm.cu:35-54); the first `mask` slots belong to the previous row and are
+// computed but never stored (RoDeSddmm.cu:56-58, 197).
+template <typename T, int K>
+__global__ void __launch_bounds__(kWgThreads)
+sddmm_block_kernel(int m1, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                   const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
+                   const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
+{
+    using S = SddmmShape<T, K>;
+    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int seg = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
+    if (seg >= m1) return;
+
+    const int row = block_rows[seg];
+    const int start = st_off[seg];
+    const int end = min(row_ptr[row + 1], st_off[seg + 1]);
+    const int mask = start & (kVecLen - 1);
+    const int base = start - mask;
+    const int cnt = (end - start + mask) / kBlockItems * kBlockItems;
+
+    float a[S::kVec];
+    load_lhs_slice<T, K>(lhs, row, lane, a);
+    const T* rhs_lane = rhs + (lane % S::kLpr) * S::kVec;
+    int* lds_cols = lds + wave * kWave;
+
+    for (int off = 0; off < cnt; off += kWave) {
+        if (off + (lane & 32) < cnt) { // the upper half sits out a trailing 32-slot step
+            const int slot = off + lane;
+            const int c = col[base + slot];
+            const float v = val[base + slot];
+            const float d = sddmm_unit<T, K, true>(rhs_lane, a, c, 32, lds_cols, lane);
+            if (slot >= mask) out[base + slot] = v * d;
+        }
+    }
+}
+
+// One 32-lane half per residue row.  Tail selection follows RoDeSddmm.cu:237-243:
+// with N = len + (s & 3), rows with N >= 32 keep only their last N % 32 slots
+// starting at (s & ~3) + floor(N / 32) * 32; shorter rows are taken whole.
+template <typename T, int K>
+__global__ void __launch_bounds__(kWgThreads)
+sddmm_residue_kernel(int m2, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
+                     const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
+                     const T* __restrict__ rhs, float* __restrict__ out)
+{
+    using S = SddmmShape<T, K>;
+    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * 2 + (lane >> 5);
+
+    int row = 0, first = 0, cnt = 0;
+    if (item < m2) {
+        row = residue_rows[item];
+        const int s = row_ptr[row], e = row_ptr[row + 1];
+        const int pad = s & (kVecLen - 1);
+        const int N = e - s + pad;
+        if (N >= kBlockItems) {
+            first = (s - pad) + N / kBlockItems * kBlockItems;
+            cnt = N % kBlockItems;
+        } else {
+            first = s;
+            cnt = e - s;
+        }
+    }
+    if (cnt <= 0) return; // an empty, unaligned row is listed as a residue but owns no slot
+
+    const int slot = lane & 31;
+    const int idx = first + min(slot, cnt - 1);
+    const int c = col[idx];
+    const float v = val[idx];
+    float a[S::kVec];
+    load_lhs_slice<T, K>(lhs, row, lane, a);
+    const T* rhs_lane = rhs + (lane % S::kLpr) * S::kVec;
+    const float d = sddmm_unit<T, K, false>(rhs_lane, a, c, cnt, lds + wave * kWave, lane);
+    if (slot < cnt) out[idx] = v * d;
+}
+
+inline int grid_for_waves(long long nwaves)
+{
+    long long wgs = (nwaves + kWavesPerWg - 1) / kWavesPerWg;
+    wgs = (wgs + kXcds - 1) / kXcds * kXcds; // xcd_logical_block needs a multiple of kXcds
+    return (int)wgs;
+}
+
+template <typename T, int K>
+hipError_t launch(int m1, int m2, const int* block_rows, const int* residue_rows, const int* st_off,
+                  const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
+                  hipStream_t s1, hipStream_t s2)
+{
+    if (m1 > 0) {
+        sddmm_block_kernel<T, K><<<grid_for_waves(m1), kWgThreads, 0, s1>>>(m1, block_rows, st_off, row_ptr, col, val,
+                                                                            lhs, rhs, out);
+    }
+    if (m2 > 0) {
+        sddmm_residue_kernel<T, K><<<grid_for_waves(((long long)m2 + 1) / 2), kWgThreads, 0, s2>>>(
+            m2, residue_rows, row_ptr, col, val, lhs, rhs, out);
+    }
+    return hipGetLastError();
+}
+
+} // namespace
+
+template <typename T>
+hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int* residue_rows, const int* st_off,
+                        const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs,
+                        float* out, hipStream_t s1, hipStream_t s2)
+{
+    switch (k) {
+    case 32: return launch<T, 32>(m1, m2, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, s1, s2);
+    case 64: return launch<T, 64>(m1, m2, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, s1, s2);
+    case 128: return launch<T, 128>(m1, m2, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, s1, s2);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template hipError_t sddmm_launch<float>(int, int, int, const int*, const int*, const int*, const int*, const int*,
+                                        const float*, const float*, const float*, float*, hipStream_t, hipStream_t);
+template hipError_t sddmm_launch<__half>(int, int, int, const int*, const int*, const int*, const int*, const int*,
+                                         const float*, const __half*, const __half*, float*, hipStream_t, hipStream_t);
+
+} // namespace rode

@@ -1,0 +1,139 @@
+"""PyTorch-facing SDDMM op with the interface of the reference's
+``RoDe_SDDMM/rode_sddmm.py``: ``RoDeCSR`` (:12-191), ``rode_sddmm`` (:194-248),
+``torch_sddmm_reference`` (:251-304) and ``compare_results`` (:307-378).
+"""
+import torch
+
+from . import rode_sddmm_hip
+
+
+class RoDeCSR:
+    """CSR matrix plus its RoDe row decomposition (block segments + residues).
+
+    Attributes (same names as the reference class): ``m, n, k, nnz, device,
+    row_offsets_cpu, row_offsets, column_indices, values, block_indices,
+    residue_indices, st_offsets, m1, m2``.
+    """
+
+    # Decomposition parameters per hidden size k.  32 and 128 are the
+    # reference's table (rode_sddmm.py:35-38); 64 is an addition.  The kernels
+    # walk a segment in 64-slot steps whatever its length, so any seg_length that
+    # is a multiple of 32 is valid for any k.
+    CONFIGS = {
+        32: {"seg_length": 512, "k_block": 32, "vec_len": 4},
+        64: {"seg_length": 512, "k_block": 32, "vec_len": 4},
+        128: {"seg_length": 32, "k_block": 32, "vec_len": 4},
+    }
+
+    def __init__(self, row_offsets, column_indices, values, device, m, n, k=128, config=None):
+        if k not in self.CONFIGS:
+            raise ValueError(f"k must be one of {sorted(self.CONFIGS)}, got {k}")
+        self.m = m
+        self.n = n
+        self.k = k
+        self.nnz = values.numel()
+        self.device = torch.device(device)
+        self.config = dict(config) if config is not None else dict(self.CONFIGS[k])
+
+        self.row_offsets_cpu = row_offsets.to(dtype=torch.int32, device="cpu").contiguous()
+        self.column_indices = column_indices.to(dtype=torch.int32, device=self.device).contiguous()
+        self.values = values.to(dtype=torch.float32, device=self.device).contiguous()
+        self.row_offsets = self.row_offsets_cpu.to(device=self.device)
+        self._preprocess()
+
+    def _preprocess(self):
+        """Row decomposition on the GPU; the index arrays never visit the host."""
+        cfg = self.config
+        blk, st, res, m1, m2 = rode_sddmm_hip.preprocess_device(
+            self.row_offsets, self.nnz, cfg["seg_length"], cfg["k_block"], cfg["vec_len"])
+        self.block_indices = blk
+        self.st_offsets = st
+        self.residue_indices = res
+        self.m1 = m1
+        self.m2 = m2
+
+    @classmethod
+    def from_random(cls, m, n, nnz_per_row, device, k=128):
+        """Random pattern with about ``nnz_per_row`` entries per row (duplicates
+        removed, rows not padded), N(0,1) values -- rode_sddmm.py:100-144."""
+        nnz_raw = m * nnz_per_row
+        coords = torch.unique(torch.randint(0, m, (nnz_raw,)) * n + torch.randint(0, n, (nnz_raw,)))
+        rows = torch.div(coords, n, rounding_mode="floor")
+        cols = coords % n
+        vals = torch.randn(coords.numel(), dtype=torch.float32)
+        row_offsets = torch.zeros(m + 1, dtype=torch.int64)
+        row_offsets[1:] = torch.cumsum(torch.bincount(rows, minlength=m), 0)
+        return cls(row_offsets.to(torch.int32), cols.to(torch.int32), vals, device, m, n, k)
+
+    def to_torch_sparse_csr(self):
+        """``torch.sparse_csr`` copy without the explicit zeros that pad rows in the
+        reference's C++ generators (rode_sddmm.py:146-185)."""
+        keep = (self.values != 0).cpu()
+        ro = self.row_offsets_cpu.to(torch.int64)
+        rows = torch.repeat_interleave(torch.arange(self.m), ro[1:] - ro[:-1])
+        crow = torch.zeros(self.m + 1, dtype=torch.int64)
+        crow[1:] = torch.cumsum(torch.bincount(rows[keep], minlength=self.m), 0)
+        return torch.sparse_csr_tensor(
+            crow,
+            self.column_indices.cpu()[keep].to(torch.int64),
+            self.values.cpu()[keep],
+            size=(self.m, self.n),
+            device=self.device,
+        )
+
+    def __repr__(self):
+        return (f"RoDeCSR(m={self.m}, n={self.n}, nnz={self.nnz}, k={self.k}, "
+                f"m1={self.m1}, m2={self.m2}, device={self.device})")
+
+
+def rode_sddmm(sparse_matrix, lhs, rhs):
+    """out = S (.) (lhs @ rhs^T) sampled at the nonzeros of S; returns the (nnz,)
+    values in CSR order.  lhs is (m, k), rhs is (n, k); float32, or float16 with
+    fp32 accumulation."""
+    m, n, k = sparse_matrix.m, sparse_matrix.n, sparse_matrix.k
+    if tuple(lhs.shape) != (m, k):
+        raise ValueError(f"lhs_matrix shape must be ({m}, {k}), got {tuple(lhs.shape)}")
+    if tuple(rhs.shape) != (n, k):
+        raise ValueError(f"rhs_matrix shape must be ({n}, {k}), got {tuple(rhs.shape)}")
+    assert lhs.is_cuda and lhs.device == sparse_matrix.device, f"lhs must be on {sparse_matrix.device}, got {lhs.device}"
+    assert rhs.is_cuda and rhs.device == sparse_matrix.device, f"rhs must be on {sparse_matrix.device}, got {rhs.device}"
+    assert lhs.dtype in (torch.float32, torch.float16), f"lhs must be float32 or float16, got {lhs.dtype}"
+    assert rhs.dtype == lhs.dtype, f"rhs must be {lhs.dtype}, got {rhs.dtype}"
+    return rode_sddmm_hip.sddmm_forward(
+        sparse_matrix.block_indices, sparse_matrix.residue_indices, sparse_matrix.st_offsets,
+        sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,
+        sparse_matrix.values, m, n, lhs.contiguous(), rhs.contiguous(), k)
+
+
+def torch_sddmm_reference(sparse_csr, lhs_matrix, rhs_matrix):
+    """Library oracle used by the reference's tests: ``sampled_addmm`` with beta 0
+    samples lhs @ rhs^T on the pattern, then the pattern's values are multiplied
+    in (rode_sddmm.py:285-304)."""
+    sampled = torch.sparse.sampled_addmm(sparse_csr, lhs_matrix, rhs_matrix.T, beta=0.0, alpha=1.0)
+    return torch.sparse_csr_tensor(
+        sampled.crow_indices(), sampled.col_indices(), sampled.values() * sparse_csr.values(),
+        size=sampled.shape, device=sampled.device, dtype=sampled.dtype)
+
+
+def compare_results(rode_output, torch_sparse_output, rode_csr, tolerance=1e-3):
+    """Error statistics of a RoDe output against a sparse-CSR oracle; an entry is
+    an error when both its absolute and its relative difference exceed
+    ``tolerance`` (rode_sddmm.py:357-368).  Entries whose pattern value is exactly
+    0 are padding and are skipped (:333-339)."""
+    keep = (rode_csr.values != 0).cpu()
+    got = rode_output.detach().cpu().to(torch.float32)[keep]
+    ref = torch_sparse_output.values().detach().cpu().to(torch.float32)
+    if got.numel() != ref.numel():
+        inf = float("inf")
+        return {"passed": False, "error": f"Size mismatch: RoDe={got.numel()}, Torch={ref.numel()}",
+                "mae": inf, "mean_rel": inf, "max_abs": inf, "max_rel": inf,
+                "error_count": -1, "total_count": got.numel()}
+    if got.numel() == 0:
+        return {"passed": True, "mae": 0.0, "mean_rel": 0.0, "max_abs": 0.0, "max_rel": 0.0,
+                "error_count": 0, "total_count": 0}
+    diff = (got - ref).abs()
+    rel = diff / (ref.abs() + 1e-8)
+    errors = int(((diff > tolerance) & (rel > tolerance)).sum())
+    return {"passed": errors == 0, "mae": diff.mean().item(), "mean_rel": rel.mean().item(),
+            "max_abs": diff.max().item(), "max_rel": rel.max().item(),
+            "error_count": errors, "total_count": got.numel()}

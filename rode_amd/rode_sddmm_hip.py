@@ -1,0 +1,165 @@
+"""Tensor-level entry points, mirroring the reference's compiled torch module
+``rode_sddmm_cuda`` (``RoDe_SDDMM/rode_sddmm_cuda.cu:254-278``): ``preprocess``
+and ``sddmm_forward`` keep their argument names, order and error behaviour
+(``RuntimeError`` where the reference's ``TORCH_CHECK`` throws).  PyTorch is used
+for device memory and the current stream only; all work is done by
+``librode_hip.so`` through its C ABI.
+
+Additions with no counterpart in the reference module: ``preprocess_device``
+(decomposition of a row pointer that already lives on the GPU, results stay on
+the GPU) and ``spmm_forward``.
+"""
+import torch
+
+from . import _lib
+
+_SUPPORTED_K = (32, 64, 128)
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _check_input(x, name):
+    _check(x.device.type == "cuda", f"{name} must be a CUDA tensor")
+    _check(x.is_contiguous(), f"{name} must be contiguous")
+
+
+def _stream_handle(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def preprocess_capacity(m, nnz, seg_length, vec_len):
+    """Upper bound on the number of block segments (each row's aligned length is
+    at most len + vec_len - 1, and it yields at most aligned/seg + 1 segments)."""
+    return (nnz + (vec_len - 1) * m) // seg_length + m
+
+
+def preprocess_device(row_offsets, nnz, seg_length, k_block, vec_len):
+    """Row decomposition of a device-resident int32 row pointer.
+
+    Returns ``(block_indices, st_offsets, residue_indices, n_blk, n_res)`` with
+    the tensor sizes of the reference (``rode_sddmm_cuda.cu:115-117``):
+    ``block_indices[max(n_blk,1)]``, ``st_offsets[n_blk+1]``,
+    ``residue_indices[max(n_res,1)]``, all on ``row_offsets.device``.
+    """
+    _check_input(row_offsets, "row_offsets")
+    _check(row_offsets.dtype == torch.int32, "row_offsets must be int32")
+    _check(row_offsets.dim() == 1 and row_offsets.numel() >= 1, "row_offsets must hold m+1 entries")
+    _check(seg_length > 0 and k_block > 0 and vec_len > 0, "seg_length, k_block and vec_len must be positive")
+    lib = _lib.load()
+    dev = row_offsets.device
+    m = row_offsets.numel() - 1
+    cap = preprocess_capacity(m, int(nnz), seg_length, vec_len)
+    with torch.cuda.device(dev):
+        blk = torch.empty(cap + 1, dtype=torch.int32, device=dev)
+        st = torch.empty(cap + 2, dtype=torch.int32, device=dev)
+        res = torch.empty(max(m, 1), dtype=torch.int32, device=dev)
+        counts = torch.empty(2, dtype=torch.int32, device=dev)
+        ws_bytes = lib.rode_hip_preprocess_workspace_bytes(m)
+        ws = torch.empty((ws_bytes + 7) // 8, dtype=torch.int64, device=dev)
+        code = lib.rode_hip_preprocess(seg_length, k_block, vec_len, m, row_offsets.data_ptr(), blk.data_ptr(),
+                                       st.data_ptr(), res.data_ptr(), counts.data_ptr(),
+                                       counts.data_ptr() + 4, cap, ws.data_ptr(), ws_bytes, _stream_handle(dev))
+        _lib.check(code, "rode_hip_preprocess")
+        n_blk, n_res = (int(v) for v in counts.cpu())  # stream-ordered copy: waits for the kernels
+    return blk[: max(n_blk, 1)], st[: n_blk + 1], res[: max(n_res, 1)], n_blk, n_res
+
+
+def preprocess(row_offsets, nnz, seg_length, k_block, vec_len):
+    """``rode_sddmm_cuda.preprocess`` (``rode_sddmm_cuda.cu:54-131``): takes the CPU
+    int32 row pointer and returns CPU tensors, as the reference does; the
+    decomposition itself runs on the current GPU."""
+    _check(row_offsets.device.type == "cpu", "row_offsets must be on CPU for preprocessing")
+    _check(row_offsets.dtype == torch.int32, "row_offsets must be int32")
+    _lib.load()
+    dev = torch.device("cuda", torch.cuda.current_device())
+    blk, st, res, n_blk, n_res = preprocess_device(row_offsets.contiguous().to(dev), nnz, seg_length, k_block, vec_len)
+    return blk.cpu(), st.cpu(), res.cpu(), n_blk, n_res
+
+
+def _dense_kind(lhs_matrix, rhs_matrix, lhs_name, rhs_name):
+    if lhs_matrix.dtype == torch.float16 and rhs_matrix.dtype == torch.float16:
+        return "f16"
+    _check(lhs_matrix.dtype == torch.float32, f"{lhs_name} must be float32")
+    _check(rhs_matrix.dtype == torch.float32, f"{rhs_name} must be float32")
+    return "f32"
+
+
+def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, n,
+                  lhs_matrix, rhs_matrix, k_version):
+    """``rode_sddmm_cuda.sddmm_forward`` (``rode_sddmm_cuda.cu:136-249``).
+
+    Differences from the reference, none of which changes a result: k_version 64
+    and fp16 ``lhs_matrix``/``rhs_matrix`` (fp32 accumulate) are accepted too; the
+    kernels are queued on PyTorch's current stream instead of two streams that
+    are created, synchronised and destroyed per call (``:203-246``).
+    """
+    for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
+                    (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
+                    (values, "values"), (lhs_matrix, "lhs_matrix"), (rhs_matrix, "rhs_matrix")):
+        _check_input(t, name)
+    for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
+                    (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices")):
+        _check(t.dtype == torch.int32, f"{name} must be int32")
+    _check(values.dtype == torch.float32, "values must be float32")
+    kind = _dense_kind(lhs_matrix, rhs_matrix, "lhs_matrix", "rhs_matrix")
+
+    k = lhs_matrix.size(1)
+    nnz = values.size(0)
+    _check(k_version in _SUPPORTED_K, "k_version must be 32, 64 or 128")
+    _check(k == k_version, "k dimension must match k_version")
+    _check(lhs_matrix.size(0) == m, "lhs_matrix rows must equal m")
+    _check(rhs_matrix.size(0) == n, "rhs_matrix rows must equal n")
+    _check(rhs_matrix.size(1) == k, "rhs_matrix cols must equal k")
+
+    out = torch.zeros(nnz, dtype=torch.float32, device=values.device)
+    if m1 == 0 and m2 == 0:
+        return out
+    lib = _lib.load()
+    fn = lib.rode_hip_sddmm_f32 if kind == "f32" else lib.rode_hip_sddmm_f16
+    with torch.cuda.device(values.device):
+        s = _stream_handle(values.device)
+        code = fn(m1, m2, n, k, block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
+                  row_offsets.data_ptr(), column_indices.data_ptr(), values.data_ptr(), lhs_matrix.data_ptr(),
+                  rhs_matrix.data_ptr(), out.data_ptr(), s, s)
+    _lib.check(code, "rode_hip_sddmm")
+    return out
+
+
+def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, k,
+                 dense_matrix, out=None):
+    """C = A_csr @ dense_matrix through ``rode_hip_spmm_f32`` / ``_f16``
+    (host API ``RoDe_SpMM/RoDeSpmm.h:4-8``).  ``dense_matrix`` is (k, n) with n a
+    multiple of 32; the result is a new zero-initialised (m, n) fp32 tensor, or
+    ``out`` accumulated in place the way the reference kernels do (long rows add,
+    short rows overwrite)."""
+    for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
+                    (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
+                    (values, "values"), (dense_matrix, "dense_matrix")):
+        _check_input(t, name)
+    for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
+                    (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices")):
+        _check(t.dtype == torch.int32, f"{name} must be int32")
+    _check(values.dtype == torch.float32, "values must be float32")
+    _check(dense_matrix.dtype in (torch.float32, torch.float16), "dense_matrix must be float32 or float16")
+    _check(dense_matrix.dim() == 2 and dense_matrix.size(0) == k, "dense_matrix rows must equal k")
+    n = dense_matrix.size(1)
+    _check(n > 0 and n % 32 == 0, "dense_matrix cols must be a positive multiple of 32")
+    if out is None:
+        out = torch.zeros((m, n), dtype=torch.float32, device=values.device)
+    else:
+        _check_input(out, "out")
+        _check(out.dtype == torch.float32 and tuple(out.shape) == (m, n), "out must be float32 of shape (m, n)")
+    if m1 == 0 and m2 == 0:
+        return out
+    lib = _lib.load()
+    fn = lib.rode_hip_spmm_f32 if dense_matrix.dtype == torch.float32 else lib.rode_hip_spmm_f16
+    with torch.cuda.device(values.device):
+        s = _stream_handle(values.device)
+        code = fn(m1, m2, k, n, values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
+                  block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
+                  dense_matrix.data_ptr(), out.data_ptr(), s, s)
+    _lib.check(code, "rode_hip_spmm")
+    return out

@@ -1,0 +1,23 @@
+"""SpMM op on a ``RoDeCSR``.  The reference offers SpMM only as a C++ host API
+(``RoDe_SpMM/RoDeSpmm.h:4-8``); this wraps the same entry point for tensors."""
+import torch
+
+from . import rode_sddmm_hip
+
+
+def rode_spmm(sparse_matrix, dense, out=None):
+    """C = S @ dense.  ``dense`` is (n, width) float32 or float16 with ``width`` a
+    multiple of 32; returns an (m, width) float32 tensor."""
+    if dense.dim() != 2 or dense.shape[0] != sparse_matrix.n:
+        raise ValueError(f"dense shape must be ({sparse_matrix.n}, width), got {tuple(dense.shape)}")
+    if dense.shape[1] % 32 != 0:
+        raise ValueError(f"dense width must be a multiple of 32, got {dense.shape[1]}")
+    assert dense.is_cuda and dense.device == sparse_matrix.device, (
+        f"dense must be on {sparse_matrix.device}, got {dense.device}")
+    assert dense.dtype in (torch.float32, torch.float16), f"dense must be float32 or float16, got {dense.dtype}"
+    seg = sparse_matrix.config
+    assert seg["k_block"] == 32 and seg["vec_len"] == 4, "the kernels need k_block=32, vec_len=4"
+    return rode_sddmm_hip.spmm_forward(
+        sparse_matrix.block_indices, sparse_matrix.residue_indices, sparse_matrix.st_offsets,
+        sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,
+        sparse_matrix.values, sparse_matrix.m, sparse_matrix.n, dense.contiguous(), out)

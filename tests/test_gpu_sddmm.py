@@ -1,0 +1,230 @@
+"""SDDMM parity on the GPU, through the Python op and the C ABI.
+
+Oracles: oracle.sddmm_f32 (the reference tests' own CPU loop, judged with the
+reference tests' abs-AND-rel rule, tol 1e-3) and oracle.sddmm_f64 (judged with the
+row-L1-normalised bound: 1e-4 for fp32 operands, 2e-3 for fp16 operands with fp32
+accumulation)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+# The reference's own table, RoDe_SDDMM/run_test.py:81-132 (m, n, nnz_per_row).
+REFERENCE_CONFIGS = [
+    (64, 64, 8), (128, 128, 16), (256, 256, 32), (63, 67, 10), (97, 103, 15), (127, 131, 20),
+    (512, 512, 32), (1024, 1024, 64), (2048, 2048, 128), (511, 517, 33), (1023, 1031, 65), (2047, 2053, 127),
+    (2048, 256, 32), (4096, 512, 64), (1999, 257, 45), (256, 2048, 32), (512, 4096, 64), (257, 2003, 47),
+    (1, 1000, 100), (1000, 1, 1), (17, 1999, 150), (1999, 17, 5), (31, 4097, 200),
+    (1024, 1024, 1), (1024, 1024, 4), (1024, 1024, 16), (1024, 1024, 64), (1024, 1024, 256), (1024, 1024, 512),
+    (32, 32, 16), (33, 31, 10), (128, 32, 8), (32, 128, 8),
+    (127, 131, 23), (251, 257, 47), (509, 521, 67), (1021, 1031, 97),
+    (4096, 4096, 128), (4093, 4099, 129),
+]
+
+
+def _check(csr, rp, col, val, lhs, rhs, half=False, ref_rule=True):
+    import oracle
+    from gpu_common import TOL_F16, TOL_F32, check_csr_decomposition, round_half, run_sddmm
+    from helpers import reference_error_count, sddmm_row_l1_error
+    check_csr_decomposition(csr, rp)
+    out = run_sddmm(csr, lhs, rhs, half)
+    assert out.shape == (len(val),) and out.dtype == np.float32
+    if half:
+        lhs, rhs = round_half(lhs), round_half(rhs)
+    ref64, scale = oracle.sddmm_f64(rp, col, val, lhs, rhs, with_abs=True)
+    err = sddmm_row_l1_error(out, ref64, rp)
+    assert err <= (TOL_F16 if half else TOL_F32), f"row-L1 error {err}"
+    if not half:
+        # per element, against the magnitude of the terms that were summed: a few ulp per term
+        strict = np.abs(out - ref64) / np.maximum(scale, 1e-30)
+        assert strict.max(initial=0.0) <= 2e-6, f"per-element error {strict.max()}"
+        if ref_rule:
+            assert reference_error_count(out, oracle.sddmm_f32(rp, col, val, lhs, rhs)) == 0
+    return err
+
+
+@pytest.mark.parametrize("k", [128, 32])
+def test_reference_table(k):
+    """The reference's C++ test (test.cu for k=128, main.cu for k=32): its seeded
+    generators (rows padded to 4 with explicit zeros), its decomposition parameters,
+    its CPU loop and its pass rule."""
+    from gpu_common import make_csr
+    from rode_amd import workloads
+    worst = 0.0
+    for m, n, per_row in REFERENCE_CONFIGS:
+        rp, col, val = workloads.reference_csr(m, n, per_row, poisson=(k == 128), pad_to=4, seed=42)
+        lhs = workloads.reference_dense(m, k, 123)
+        rhs = workloads.reference_dense(n, k, 456)
+        csr = make_csr(rp, col, val, m, n, k)  # CONFIGS[k]: (512,32,4) for 32, (32,32,4) for 128
+        worst = max(worst, _check(csr, rp, col, val, lhs, rhs))
+    print(f"k={k}: worst row-L1 error over {len(REFERENCE_CONFIGS)} reference configs: {worst:.2e}")
+
+
+def test_reference_stress():
+    """run_test.py:427-439: random.seed(42), random shapes."""
+    import random
+    from gpu_common import make_csr
+    from rode_amd import workloads
+    random.seed(42)
+    for _ in range(12):
+        m, n = random.randint(10, 2000), random.randint(10, 2000)
+        per_row = random.randint(1, min(n, 200))
+        rp, col, val = workloads.reference_csr(m, n, per_row, poisson=True)
+        csr = make_csr(rp, col, val, m, n, 128)
+        _check(csr, rp, col, val, workloads.reference_dense(m, 128, 123), workloads.reference_dense(n, 128, 456))
+
+
+@pytest.mark.parametrize("k", [32, 64, 128])
+@pytest.mark.parametrize("seg", [32, 64, 512])
+def test_unpadded_rows(k, seg):
+    """Rows that start at any offset mod 4 (the reference's Python test path,
+    test_pytorch.py), long rows, empty rows, every K and several segment lengths."""
+    from gpu_common import make_csr
+    from helpers import random_csr
+    rng = np.random.default_rng(1000 * k + seg)
+    m, n = 1500, 1777
+    rp, col, val = random_csr(rng, m, n, 37, long_rows=6, long_len=1700, empty_frac=0.15)
+    assert (rp[:-1] % 4 != 0).any()
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    _check(make_csr(rp, col, val, m, n, k, seg), rp, col, val, lhs, rhs)
+
+
+@pytest.mark.parametrize("k", [32, 64, 128])
+def test_fp16_operands(k):
+    from gpu_common import make_csr
+    from helpers import random_csr
+    rng = np.random.default_rng(k)
+    m, n = 900, 1200
+    rp, col, val = random_csr(rng, m, n, 50, long_rows=4, long_len=1100)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    for seg in (32, 512):
+        _check(make_csr(rp, col, val, m, n, k, seg), rp, col, val, lhs, rhs, half=True)
+
+
+def test_special_cases_and_edges():
+    from gpu_common import DEV, make_csr, run_sddmm
+    from helpers import random_csr
+    from rode_amd import rode_sddmm
+    rng = np.random.default_rng(9)
+    m, n, k = 700, 650, 64
+    rp, col, val = random_csr(rng, m, n, 45, long_rows=3, long_len=600)
+    csr = make_csr(rp, col, val, m, n, k)
+    # all-ones operands: out = k * val exactly
+    out = run_sddmm(csr, np.ones((m, k), np.float32), np.ones((n, k), np.float32))
+    np.testing.assert_array_equal(out, val * np.float32(k))
+    # an Inf in an rhs row that one row references must not leak into other outputs
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    bad_col = int(col[rp[10]])
+    rhs[bad_col, 3] = np.inf
+    out = run_sddmm(csr, lhs, rhs)
+    assert np.isfinite(out[col != bad_col]).all() and not np.isfinite(out[col == bad_col]).any()
+    # empty matrix, matrix with empty rows only
+    empty = make_csr(np.zeros(6, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32), 5, 7, 32)
+    assert (empty.m1, empty.m2) == (0, 0)
+    assert rode_sddmm(empty, torch.zeros(5, 32, device=DEV), torch.zeros(7, 32, device=DEV)).numel() == 0
+    # non-contiguous operands are made contiguous by the op
+    lhs_t = torch.from_numpy(rng.standard_normal((k, m)).astype(np.float32)).to(DEV).t()
+    rhs_t = torch.from_numpy(rng.standard_normal((n, k)).astype(np.float32)).to(DEV)
+    a = rode_sddmm(csr, lhs_t, rhs_t)
+    b = rode_sddmm(csr, lhs_t.contiguous(), rhs_t)
+    assert torch.equal(a, b)
+
+
+def test_argument_errors():
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import RoDeCSR, rode_sddmm, rode_sddmm_hip
+    rng = np.random.default_rng(2)
+    rp, col, val = random_csr(rng, 40, 50, 8)
+    csr = make_csr(rp, col, val, 40, 50, 32)
+    lhs, rhs = torch.zeros(40, 32, device=DEV), torch.zeros(50, 32, device=DEV)
+    with pytest.raises(ValueError):
+        RoDeCSR(torch.from_numpy(rp), torch.from_numpy(col), torch.from_numpy(val), DEV, 40, 50, 48)
+    with pytest.raises(ValueError):
+        rode_sddmm(csr, lhs[:, :16], rhs)
+    with pytest.raises(ValueError):
+        rode_sddmm(csr, lhs, rhs[:49])
+    with pytest.raises(AssertionError):
+        rode_sddmm(csr, lhs.cpu(), rhs)
+    with pytest.raises(AssertionError):
+        rode_sddmm(csr, lhs.double(), rhs.double())
+    args = [csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2, csr.row_offsets,
+            csr.column_indices, csr.values, 40, 50, lhs, rhs, 32]
+    for pos, bad, msg in [(12, 48, "k_version"), (12, 128, "match k_version"), (8, 41, "rows must equal m"),
+                          (7, csr.values.double(), "float32"), (6, csr.column_indices.long(), "int32"),
+                          (10, lhs.cpu(), "CUDA tensor"), (11, rhs.t().contiguous().t(), "contiguous")]:
+        a = list(args)
+        a[pos] = bad
+        with pytest.raises(RuntimeError, match=msg):
+            rode_sddmm_hip.sddmm_forward(*a)
+
+
+def test_torch_oracle_and_compare_results():
+    """The reference's Python test flow (test_pytorch.py:163-207): RoDeCSR.from_random,
+    torch.sparse.sampled_addmm as the oracle, compare_results as the judge."""
+    from gpu_common import DEV
+    from rode_amd import RoDeCSR, compare_results, rode_sddmm, torch_sddmm_reference
+    torch.manual_seed(0)
+    for k in (32, 128):
+        csr = RoDeCSR.from_random(511, 517, 33, DEV, k)
+        torch.manual_seed(123); lhs = torch.randn(511, k, device=DEV)
+        torch.manual_seed(456); rhs = torch.randn(517, k, device=DEV)
+        out = rode_sddmm(csr, lhs, rhs)
+        ref = torch_sddmm_reference(csr.to_torch_sparse_csr(), lhs, rhs)
+        stats = compare_results(out, ref, csr)
+        assert stats["passed"] and stats["total_count"] == csr.nnz and stats["max_abs"] < 1e-3, stats
+        assert "RoDeCSR(m=511" in repr(csr)
+
+
+@pytest.mark.parametrize("name,k", [("c1_uniform", 32), ("c2_lognormal", 32), ("c2_lognormal", 128)])
+def test_benchmark_configs_against_oracle(name, k):
+    from gpu_common import make_csr
+    from rode_amd import workloads
+    m, n, rp, col, val = workloads.config(name)
+    rng = np.random.default_rng(3000 + k)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    for seg in (512, 32):
+        _check(make_csr(rp, col, val, m, n, k, seg), rp, col, val, lhs, rhs, ref_rule=(name == "c1_uniform"))
+
+
+@pytest.mark.parametrize("name,k,half", [("c3_banded", 32, False), ("c4_powerlaw", 64, False),
+                                         ("c5_attention", 64, False), ("c5_attention", 64, True)])
+def test_large_configs_scaled_against_oracle(name, k, half):
+    from gpu_common import make_csr
+    from rode_amd import workloads
+    scale = {"c3_banded": 1 / 16, "c4_powerlaw": 1 / 16, "c5_attention": 1 / 4}[name]
+    m, n, rp, col, val = workloads.config(name, scale)
+    rng = np.random.default_rng(4000 + k)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    _check(make_csr(rp, col, val, m, n, k, 512), rp, col, val, lhs, rhs, half=half, ref_rule=False)
+
+
+@pytest.mark.parametrize("name,k", [("c3_banded", 128), ("c4_powerlaw", 128), ("c4_powerlaw", 64), ("c5_attention", 64)])
+def test_full_size_properties(name, k):
+    """Full benchmark sizes, checked through size-independent facts: with one-hot
+    lhs rows and an rhs holding its own row number, out[idx] = val[idx] * col[idx]
+    exactly; with all-ones operands out = k * val; and out is linear in lhs."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import rode_sddmm, workloads
+    m, n, rp, col, val = workloads.config(name)
+    csr = make_csr(rp, col, val, m, n, k, 512)
+    v = torch.from_numpy(val).to(DEV)
+    ones = rode_sddmm(csr, torch.ones(m, k, device=DEV), torch.ones(n, k, device=DEV))
+    assert torch.equal(ones, v * k)
+    lhs = torch.zeros(m, k, device=DEV); lhs[:, k - 1] = 1
+    rhs = torch.zeros(n, k, device=DEV); rhs[:, k - 1] = torch.arange(n, device=DEV, dtype=torch.float32) % 4096
+    out = rode_sddmm(csr, lhs, rhs)
+    assert torch.equal(out, v * (torch.from_numpy(col).to(DEV) % 4096).float())
+    del lhs, rhs, ones, out
+    g = torch.Generator(device=DEV).manual_seed(k)
+    a = torch.randn(m, k, device=DEV, generator=g); b = torch.randn(m, k, device=DEV, generator=g)
+    r = torch.randn(n, k, device=DEV, generator=g)
+    oa, ob, oab = rode_sddmm(csr, a, r), rode_sddmm(csr, b, r), rode_sddmm(csr, a + b, r)
+    scale = (oa.abs() + ob.abs()).clamp_min(1e-20)
+    assert ((oab - (oa + ob)).abs() / (scale + v.abs() * 1e-1)).max().item() < 1e-3

@@ -1,0 +1,215 @@
+"""SpMM parity on the GPU, through the Python op and the C ABI.  The reference has
+no SpMM test or CPU SpMM; the oracle is the textbook CSR product in fp64
+(oracle.spmm_f64, pinned by scipy.sparse), judged with the row-L1-normalised
+bound: 1e-4 for fp32 B, 2e-3 for fp16 B with fp32 accumulation."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(csr, rp, col, val, B, half=False):
+    import oracle
+    from gpu_common import TOL_F16, TOL_F32, check_csr_decomposition, round_half, run_spmm
+    from helpers import spmm_row_l1_error
+    check_csr_decomposition(csr, rp)
+    C = run_spmm(csr, B, half)
+    assert C.shape == (csr.m, B.shape[1]) and C.dtype == np.float32
+    if half:
+        B = round_half(B)
+    ref64, scale = oracle.spmm_f64(rp, col, val, B, with_abs=True)
+    err = spmm_row_l1_error(C, ref64)
+    assert err <= (TOL_F16 if half else TOL_F32), f"row-L1 error {err}"
+    if not half:
+        strict = np.abs(C - ref64) / np.maximum(scale, 1e-30)
+        assert strict.max(initial=0.0) <= 2e-6, f"per-element error {strict.max()}"
+    return err
+
+
+@pytest.mark.parametrize("n", [32, 64, 128, 96, 256])
+@pytest.mark.parametrize("seg", [32, 512])
+def test_unpadded_rows(n, seg):
+    from gpu_common import make_csr
+    from helpers import random_csr
+    rng = np.random.default_rng(100 * n + seg)
+    m, k = 1500, 1333
+    rp, col, val = random_csr(rng, m, k, 37, long_rows=6, long_len=1300, empty_frac=0.15)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    _check(make_csr(rp, col, val, m, k, 32, seg), rp, col, val, B)
+
+
+def test_padded_reference_matrices():
+    """The reference generators' matrices (rows padded to 4 with explicit zeros)."""
+    from gpu_common import make_csr
+    from rode_amd import workloads
+    for m, k, per_row, n in [(63, 67, 10, 32), (1023, 1031, 65, 128), (31, 4097, 200, 64), (1000, 1, 1, 32),
+                             (1, 1000, 100, 128), (2048, 2048, 128, 64), (1024, 1024, 512, 32)]:
+        rp, col, val = workloads.reference_csr(m, k, per_row, poisson=True)
+        B = workloads.reference_dense(k, n, 456)
+        _check(make_csr(rp, col, val, m, k, 32, 512), rp, col, val, B)
+
+
+@pytest.mark.parametrize("n", [32, 64, 128])
+def test_fp16_dense(n):
+    from gpu_common import make_csr
+    from helpers import random_csr
+    rng = np.random.default_rng(n)
+    m, k = 900, 1200
+    rp, col, val = random_csr(rng, m, k, 50, long_rows=4, long_len=1100)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    for seg in (32, 512):
+        _check(make_csr(rp, col, val, m, k, 32, seg), rp, col, val, B, half=True)
+
+
+def test_special_cases_and_edges():
+    from gpu_common import DEV, make_csr, run_spmm
+    from helpers import random_csr
+    from rode_amd import rode_spmm
+    rng = np.random.default_rng(4)
+    m, k, n = 800, 700, 64
+    rp, col, val = random_csr(rng, m, k, 45, long_rows=3, long_len=650, empty_frac=0.2)
+    csr = make_csr(rp, col, val, m, k, 32, 512)
+    # B = 1 -> every column holds the row sums
+    C = run_spmm(csr, np.ones((k, n), np.float32))
+    sums = np.array([val[rp[r]:rp[r + 1]].astype(np.float64).sum() for r in range(m)])
+    assert np.abs(C - sums[:, None]).max() < 1e-4 and (C == C[:, :1]).all()
+    assert not C[np.diff(rp) == 0].any()
+    # permutation pattern with unit values moves rows of B exactly
+    perm = rng.permutation(k).astype(np.int32)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    pcsr = make_csr(np.arange(k + 1, dtype=np.int32), perm, np.ones(k, np.float32), k, k, 32, 512)
+    np.testing.assert_array_equal(run_spmm(pcsr, B), B[perm])
+    # a non-finite B row must only reach the rows that reference it (the head slots
+    # of an unaligned segment belong to the previous row and are skipped, not multiplied by 0)
+    B[0, :] = np.inf
+    bad = int(col[rp[17]])
+    B[bad, 5] = np.nan
+    C = run_spmm(csr, B)
+    touches = np.array([np.isin([0, bad], col[rp[r]:rp[r + 1]]).any() for r in range(m)])
+    assert np.isfinite(C[~touches]).all() and (~np.isfinite(C[touches])).any(axis=1).all()
+    # accumulate-in-place semantics of the reference kernels: rows with >= 32 aligned
+    # slots add to C, shorter rows overwrite, empty rows are left alone
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    base = run_spmm(csr, B)
+    pre = torch.full((m, n), 2.0, device=DEV)
+    got = rode_spmm(csr, torch.from_numpy(B).to(DEV), out=pre).cpu().numpy()
+    aligned = np.diff(rp) + rp[:-1] % 4
+    adds = aligned >= 32
+    # an empty row whose offset is a multiple of 4 is in no list; one at another offset is a zero-slot residue
+    keeps = (np.diff(rp) == 0) & (rp[:-1] % 4 == 0)
+    np.testing.assert_allclose(got[adds], base[adds] + 2.0, rtol=1e-5, atol=1e-5)
+    np.testing.assert_array_equal(got[~adds & ~keeps], base[~adds & ~keeps])
+    assert (got[keeps] == 2.0).all()
+    # empty matrix
+    empty = make_csr(np.zeros(6, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32), 5, 7, 32)
+    assert not rode_spmm(empty, torch.ones(7, 32, device=DEV)).any()
+    # width not a multiple of 32
+    with pytest.raises(ValueError):
+        rode_spmm(csr, torch.zeros(k, 40, device=DEV))
+    with pytest.raises(ValueError):
+        rode_spmm(csr, torch.zeros(k + 1, 32, device=DEV))
+
+
+def test_cxx_reference_signature_entry_points():
+    """RoDeSpmm_n32 / RoDeSpmm_n128 / RoDeSDDMM_n32 / RoDeSDDMM_n128 with the reference's
+    signatures (RoDeSpmm.h:4-8, RoDeSddmm.h:4-9), called through their mangled names
+    on two side streams, as a C++ caller would."""
+    import oracle
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr, sddmm_row_l1_error, spmm_row_l1_error
+    from rode_amd import _lib
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    rng = np.random.default_rng(11)
+    m, ncols = 1200, 1100
+    rp, col, val = random_csr(rng, m, ncols, 40, long_rows=5, long_len=1000)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for name, mangled, width in [("spmm", "_Z12RoDeSpmm_n32iiiiPKfPKiS2_S2_S2_S2_S0_PfP12ihipStream_tS5_", 32),
+                                 ("spmm", "_Z13RoDeSpmm_n128iiiiPKfPKiS2_S2_S2_S2_S0_PfP12ihipStream_tS5_", 128),
+                                 ("sddmm", "_Z13RoDeSDDMM_n32iiiiPKiS0_S0_S0_S0_PKfS2_S2_PfP12ihipStream_tS5_", 32),
+                                 ("sddmm", "_Z14RoDeSDDMM_n128iiiiPKiS0_S0_S0_S0_PKfS2_S2_PfP12ihipStream_tS5_", 128)]:
+        fn = getattr(lib, mangled)
+        fn.restype = None
+        fn.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 11 if name == "sddmm" else \
+            [ctypes.c_int] * 4 + [ctypes.c_void_p] * 10
+        seg = 32 if (name == "sddmm" and width == 128) else 512  # the reference's parameter sets
+        csr = make_csr(rp, col, val, m, ncols, 32, seg)
+        if name == "spmm":
+            B = rng.standard_normal((ncols, width)).astype(np.float32)
+            dB = torch.from_numpy(B).to(DEV)
+            C = torch.zeros(m, width, device=DEV)
+            torch.cuda.synchronize()
+            fn(csr.m1, csr.m2, ncols, width, csr.values.data_ptr(), csr.column_indices.data_ptr(),
+               csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
+               csr.st_offsets.data_ptr(), dB.data_ptr(), C.data_ptr(), s1.cuda_stream, s2.cuda_stream)
+            torch.cuda.synchronize()
+            assert spmm_row_l1_error(C.cpu().numpy(), oracle.spmm_f64(rp, col, val, B)) <= 1e-4
+        else:
+            lhs = rng.standard_normal((m, width)).astype(np.float32)
+            rhs = rng.standard_normal((ncols, width)).astype(np.float32)
+            dl, dr = torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV)
+            out = torch.full((len(val),), float("nan"), device=DEV)
+            torch.cuda.synchronize()
+            fn(csr.m1, csr.m2, ncols, width, csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
+               csr.st_offsets.data_ptr(), csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
+               csr.values.data_ptr(), dl.data_ptr(), dr.data_ptr(), out.data_ptr(), s1.cuda_stream, s2.cuda_stream)
+            torch.cuda.synchronize()
+            assert sddmm_row_l1_error(out.cpu().numpy(), oracle.sddmm_f64(rp, col, val, lhs, rhs), rp) <= 1e-4
+
+
+@pytest.mark.parametrize("name,n", [("c1_uniform", 32), ("c2_lognormal", 32), ("c2_lognormal", 128)])
+def test_benchmark_configs_against_oracle(name, n):
+    from gpu_common import make_csr
+    from rode_amd import workloads
+    m, k, rp, col, val = workloads.config(name)
+    B = np.random.default_rng(5000 + n).standard_normal((k, n)).astype(np.float32)
+    for seg in (512, 32):
+        _check(make_csr(rp, col, val, m, k, 32, seg), rp, col, val, B)
+
+
+@pytest.mark.parametrize("name,n,half", [("c3_banded", 128, False), ("c4_powerlaw", 64, False),
+                                         ("c5_attention", 64, False), ("c5_attention", 64, True)])
+def test_large_configs_scaled_against_oracle(name, n, half):
+    from gpu_common import make_csr
+    from rode_amd import workloads
+    scale = {"c3_banded": 1 / 16, "c4_powerlaw": 1 / 16, "c5_attention": 1 / 4}[name]
+    m, k, rp, col, val = workloads.config(name, scale)
+    B = np.random.default_rng(6000 + n).standard_normal((k, n)).astype(np.float32)
+    _check(make_csr(rp, col, val, m, k, 32, 512), rp, col, val, B, half=half)
+
+
+@pytest.mark.parametrize("name,n", [("c3_banded", 128), ("c4_powerlaw", 128), ("c4_powerlaw", 64), ("c5_attention", 64)])
+def test_full_size_properties(name, n):
+    """Full benchmark sizes through size-independent facts: B = 1 gives the row sums
+    (checked against a segmented fp64 sum), the result is linear in B, and a checksum
+    of C equals the checksum computed from column sums of the pattern."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import rode_spmm, workloads
+    m, k, rp, col, val = workloads.config(name)
+    csr = make_csr(rp, col, val, m, k, 32, 512)
+    C = rode_spmm(csr, torch.ones(k, n, device=DEV))
+    nonempty = np.nonzero(np.diff(rp) > 0)[0]
+    sums = np.zeros(m)
+    sums[nonempty] = np.add.reduceat(val.astype(np.float64), rp[nonempty].astype(np.int64))
+    abs_sums = np.zeros(m)
+    abs_sums[nonempty] = np.add.reduceat(np.abs(val.astype(np.float64)), rp[nonempty].astype(np.int64))
+    got = C[:, 0].double().cpu().numpy()
+    assert (C == C[:, :1]).all()
+    assert np.max(np.abs(got - sums) / np.maximum(abs_sums, 1e-30)) <= 1e-5
+    del C
+    # checksum of checksums: sum_r C[r, j] = sum_c w[c] * B[c, j] with w = column sums of A
+    g = torch.Generator(device=DEV).manual_seed(n)
+    B = torch.randn(k, n, device=DEV, generator=g)
+    C = rode_spmm(csr, B)
+    w = np.bincount(col, weights=val.astype(np.float64), minlength=k)
+    want = torch.from_numpy(w).to(DEV) @ B.double()
+    wabs = torch.from_numpy(np.bincount(col, weights=np.abs(val.astype(np.float64)), minlength=k)).to(DEV) @ B.double().abs()
+    assert ((C.double().sum(0) - want).abs() / wabs).max().item() < 1e-5
+    # linearity
+    B2 = torch.randn(k, n, device=DEV, generator=g)
+    C2 = rode_spmm(csr, B2)
+    C12 = rode_spmm(csr, B + B2)
+    denom = torch.from_numpy(abs_sums).to(DEV).float()[:, None] * 8 + 1e-20
+    assert ((C12 - (C + C2)).abs() / denom).max().item() < 1e-4
