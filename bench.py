@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the RoDe hot path on one MI355X.
+
+A step is one pass over one synthetic matrix: clear C, SpMM (C = A @ B), SDDMM
+(out = A (.) (L @ R^T)), all through the C ABI with every operand already in
+HBM.  Default workload: the power-law configuration at K = 128.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--k K] [--seg SEG]
+
+Prints one JSON line: GFLOP/s (2*nnz*K per operation), the roofline figures of
+the kernel that takes the most time (algorithmic bytes / measured duration
+against 8 TB/s), and the CPU baseline (the oracle, timed on this host).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--warmup", type=int, default=3)
+    p.add_argument("--workload", default="c4_powerlaw")
+    p.add_argument("--k", type=int, default=128, help="dense width (SpMM n, SDDMM k)")
+    p.add_argument("--seg", type=int, default=0, help="segment length (0: the library's choice for this k)")
+    p.add_argument("--dtype", default="f32", choices=["f32", "f16"], help="dense operand type (accumulation is fp32)")
+    p.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (debugging only)")
+    p.add_argument("--cpu-seconds", type=float, default=8.0, help="CPU time budget per operation of the baseline")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    return p.parse_args()
+
+
+def work_split(row_ptr, col, ncols):
+    """Which nonzeros the residue kernels own (tail rule of RoDeSpmm.cu:71-82) and how
+    many distinct dense rows each kernel family touches."""
+    rp = row_ptr.astype(np.int64)
+    s, e = rp[:-1], rp[1:]
+    pad = s % 4
+    N = e - s + pad
+    tail_first = np.where(N >= 32, s - pad + N // 32 * 32, s)
+    in_res = np.arange(rp[-1], dtype=np.int64) >= np.repeat(tail_first, e - s)
+    nnz_res = int(in_res.sum())
+    distinct_res = int((np.bincount(col[in_res], minlength=ncols) > 0).sum())
+    distinct_blk = int((np.bincount(col[~in_res], minlength=ncols) > 0).sum())
+    rows_blk = int((N >= 32).sum())
+    return {"nnz_res": nnz_res, "nnz_blk": int(rp[-1]) - nnz_res, "distinct_res": distinct_res,
+            "distinct_blk": distinct_blk, "rows_blk": rows_blk}
+
+
+def algorithmic_bytes(kernel, split, m1, m2, k, elem):
+    """Compulsory traffic of one launch: every array element it needs, once."""
+    if kernel.endswith("block"):
+        nnz, rows, distinct, meta = split["nnz_blk"], split["rows_blk"], split["distinct_blk"], m1 * 12 + 4
+    else:
+        nnz, rows, distinct, meta = split["nnz_res"], m2, split["distinct_res"], m2 * 12
+    if kernel.startswith("spmm"):
+        # (col, val) + metadata + distinct B rows + C rows (atomic rows are read and written)
+        c_bytes = rows * k * 4 * (2 if kernel.endswith("block") else 1)
+        return nnz * 8 + meta + distinct * k * elem + c_bytes
+    # sddmm: (col, val) + metadata + lhs rows + distinct rhs rows + out
+    return nnz * 8 + meta + rows * k * elem + distinct * k * elem + nnz * 4
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this build has no multi-GPU path)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from rode_amd import RoDeCSR, _lib, workloads
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    lib = _lib.load()
+    k = args.k
+    elem = 4 if args.dtype == "f32" else 2
+    tdtype = torch.float32 if args.dtype == "f32" else torch.float16
+
+    t0 = time.time()
+    m, n, row_ptr, col, val = workloads.config(args.workload, args.scale)
+    nnz = int(row_ptr[-1])
+    cfg = None if args.seg == 0 else {"seg_length": args.seg, "k_block": 32, "vec_len": 4}
+    csr = RoDeCSR(torch.from_numpy(row_ptr), torch.from_numpy(col), torch.from_numpy(val), dev, m, n,
+                  k if k in RoDeCSR.CONFIGS else 128, config=cfg)
+    gen = torch.Generator(device=dev).manual_seed(3000)
+    B = torch.randn(n, k, device=dev, generator=gen).to(tdtype)     # SpMM dense operand, also SDDMM rhs
+    L = torch.randn(m, k, device=dev, generator=gen).to(tdtype)     # SDDMM lhs
+    C = torch.zeros(m, k, device=dev)
+    out = torch.empty(nnz, device=dev)
+    setup_s = time.time() - t0
+
+    stream = torch.cuda.current_stream().cuda_stream
+    spmm_fn = lib.rode_hip_spmm_f32 if args.dtype == "f32" else lib.rode_hip_spmm_f16
+    sddmm_fn = lib.rode_hip_sddmm_f32 if args.dtype == "f32" else lib.rode_hip_sddmm_f16
+
+    def spmm(m1, m2):
+        _lib.check(spmm_fn(m1, m2, n, k, csr.values.data_ptr(), csr.column_indices.data_ptr(),
+                           csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
+                           csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, stream), "spmm")
+
+    def sddmm(m1, m2):
+        _lib.check(sddmm_fn(m1, m2, n, k, csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
+                            csr.st_offsets.data_ptr(), csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
+                            csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), out.data_ptr(), stream, stream),
+                   "sddmm")
+
+    def step():
+        C.zero_()
+        spmm(csr.m1, csr.m2)
+        sddmm(csr.m1, csr.m2)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    flops_per_step = 2 * (2.0 * nnz * k)
+    gflops = flops_per_step / (ms_per_step * 1e-3) / 1e9
+
+    # ---- per-kernel durations, HIP events on the launch stream ----------------
+    def event_time(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        b.synchronize()
+        return a.elapsed_time(b) / reps  # ms
+
+    reps = max(3, min(args.steps, 20))
+    kernels = {}
+    if csr.m1 > 0:
+        kernels["spmm_block"] = event_time(lambda: spmm(csr.m1, 0), reps)
+        kernels["sddmm_block"] = event_time(lambda: sddmm(csr.m1, 0), reps)
+    if csr.m2 > 0:
+        kernels["spmm_residue"] = event_time(lambda: spmm(0, csr.m2), reps)
+        kernels["sddmm_residue"] = event_time(lambda: sddmm(0, csr.m2), reps)
+    spmm_ms = event_time(lambda: (C.zero_(), spmm(csr.m1, csr.m2)), reps)
+    sddmm_ms = event_time(lambda: sddmm(csr.m1, csr.m2), reps)
+
+    split = work_split(row_ptr, col, n)
+    per_kernel = {}
+    for name, ms in kernels.items():
+        ab = algorithmic_bytes(name, split, csr.m1, csr.m2, k, elem)
+        knnz = split["nnz_blk"] if name.endswith("block") else split["nnz_res"]
+        per_kernel[name] = {"ms": round(ms, 4), "algorithmic_bytes": ab,
+                            "algorithmic_GBs": round(ab / ms / 1e6, 1),
+                            "gather_model_GBs": round((knnz * (8 + k * elem)) / ms / 1e6, 1),
+                            "GFLOPs": round(2.0 * knnz * k / ms / 1e6, 1)}
+    dominant = max(kernels, key=kernels.get)
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        key = f"{args.workload}/k{k}/{args.dtype}/{dominant}"
+        traffic = json.load(open(tpath)).get(key)
+    dom = per_kernel[dominant]
+    roofline = {"bound": "hbm", "kernel": dominant, "achieved": dom["algorithmic_GBs"], "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(dom["algorithmic_GBs"] / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "gather_model_frac": round(dom["gather_model_GBs"] / HBM_PEAK_GBS, 4)}
+
+    # ---- CPU baseline: the oracle on a bounded sample of the same matrix --------
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+        Bh, Lh = B.float().cpu().numpy(), L.float().cpu().numpy()
+
+        def cpu_ops(rows, threads):
+            rp = row_ptr[: rows + 1]
+            cnt = int(rp[-1])
+            t = time.perf_counter()
+            c_ref = oracle.spmm_f32(rp, col[:cnt], val[:cnt], Bh, threads=threads)
+            t_spmm = time.perf_counter() - t
+            t = time.perf_counter()
+            o_ref = oracle.sddmm_f32(rp, col[:cnt], val[:cnt], Lh[:rows], Bh, threads=threads)
+            t_sddmm = time.perf_counter() - t
+            return cnt, t_spmm, t_sddmm, c_ref, o_ref
+
+        probe_rows = min(m, 20000)
+        cnt, a, b, _, _ = cpu_ops(probe_rows, 1)
+        per_nnz = max((a + b) / max(cnt, 1), 1e-12)
+        target_nnz = min(nnz, int(2 * args.cpu_seconds / per_nnz))
+        rows = int(np.searchsorted(row_ptr, target_nnz, side="right")) - 1
+        rows = max(1, min(m, rows))
+        cnt, t_spmm, t_sddmm, c_ref, o_ref = cpu_ops(rows, 1)
+        threads = oracle.num_threads()
+        _, mt_spmm, mt_sddmm, _, _ = cpu_ops(rows, threads)
+        # the same rows from the GPU run, as a parity gate of this very benchmark
+        step()
+        torch.cuda.synchronize()
+        c_gpu, o_gpu = C[:rows].cpu().numpy(), out[:cnt].cpu().numpy()
+        # SpMM: max over rows of |err|_inf / |ref row|_1 (reference values in fp64)
+        c64 = oracle.spmm_f64(row_ptr[: rows + 1], col[:cnt], val[:cnt], Bh)
+        l1 = np.abs(c64).sum(axis=1)
+        spmm_err = float(np.max(np.abs(c_gpu - c64).max(axis=1) / np.maximum(l1, 1e-30)))
+        # SDDMM: the same per CSR row over rows with condition number <= 100 (a row made of
+        # one cancelling dot product defeats any fp32 summation), and per element against
+        # the magnitude of the summed terms everywhere
+        o64, scale = oracle.sddmm_f64(row_ptr[: rows + 1], col[:cnt], val[:cnt], Lh[:rows], Bh, with_abs=True)
+        nonempty = np.nonzero(np.diff(row_ptr[: rows + 1]) > 0)[0]
+        starts = row_ptr[:rows][nonempty].astype(np.int64)
+        row_l1 = np.maximum(np.add.reduceat(np.abs(o64), starts), 1e-300)
+        row_err = np.maximum.reduceat(np.abs(o_gpu - o64), starts) / row_l1
+        good = np.add.reduceat(scale, starts) / row_l1 <= 100.0
+        sddmm_err = float(row_err[good].max(initial=0.0))
+        sddmm_strict = float(np.max(np.abs(o_gpu - o64) / np.maximum(scale, 1e-30)))
+        oblk, ost, ores = oracle.preprocess(row_ptr, csr.config["seg_length"])
+        bit_exact = (csr.m1 == len(oblk) and csr.m2 == len(ores)
+                     and csr.block_indices.cpu().numpy()[: csr.m1].tobytes() == oblk.tobytes()
+                     and csr.st_offsets.cpu().numpy().tobytes() == ost.tobytes()
+                     and csr.residue_indices.cpu().numpy()[: csr.m2].tobytes() == ores.tobytes())
+        cpu = {"value": round(2 * (2.0 * cnt * k) / (t_spmm + t_sddmm) / 1e9, 3), "unit": "GFLOP/s", "cores": 1,
+               "kind": "port",
+               "sample": f"first {rows} rows ({cnt} nnz) of the same matrix, SpMM (textbook CSR stand-in: the "
+                         f"reference has no CPU SpMM) + SDDMM (restated main.cu:65-91), fp32, one thread",
+               "spmm_ms": round(t_spmm * 1e3, 1), "sddmm_ms": round(t_sddmm * 1e3, 1),
+               "all_cores": {"cores": threads,
+                             "value": round(2 * (2.0 * cnt * k) / (mt_spmm + mt_sddmm) / 1e9, 3)},
+               "parity_vs_gpu": {"spmm_rowL1_err": spmm_err, "sddmm_rowL1_err_cond_le_100": sddmm_err,
+                                 "sddmm_err_over_term_magnitude": sddmm_strict,
+                                 "preprocess_bit_exact": bool(bit_exact)}}
+
+    line = {
+        "metric": "SpMM & SDDMM GFLOP/s (2*nnz*K/t)", "value": round(gflops, 1), "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32" if elem == 4 else "f16->f32",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload} ({workloads.CONFIGS[args.workload][5]}), K={k}, "
+                               f"step = clear C + SpMM + SDDMM",
+                   "rows": m, "cols": n, "nnz": nnz, "K": k, "seg_length": csr.config["seg_length"],
+                   "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale},
+        "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C"},
+        "sddmm": {"ms": round(sddmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / sddmm_ms / 1e6, 1)},
+        "kernels": per_kernel,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "setup_s": round(setup_s, 1),
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -15,14 +15,21 @@ class RoDeCSR:
     residue_indices, st_offsets, m1, m2``.
     """
 
-    # Decomposition parameters per hidden size k.  32 and 128 are the
-    # reference's table (rode_sddmm.py:35-38); 64 is an addition.  The kernels
-    # walk a segment in 64-slot steps whatever its length, so any seg_length that
-    # is a multiple of 32 is valid for any k.
+    # The reference's table (rode_sddmm.py:35-38): its K=128 kernels handle exactly
+    # one 32-slot chunk per segment, hence seg_length 32 there.
+    REFERENCE_CONFIGS = {
+        32: {"seg_length": 512, "k_block": 32, "vec_len": 4},
+        128: {"seg_length": 32, "k_block": 32, "vec_len": 4},
+    }
+    # Decomposition used here, per hidden size k.  The wave64 kernels walk a segment
+    # in 64-slot steps whatever its length, so one segment length serves every k;
+    # 512 measured best on MI355X (short segments multiply the atomics of SpMM,
+    # longer ones unbalance the waves).  Any multiple of 32 is valid, including the
+    # reference's values, through the ``config`` argument.
     CONFIGS = {
         32: {"seg_length": 512, "k_block": 32, "vec_len": 4},
         64: {"seg_length": 512, "k_block": 32, "vec_len": 4},
-        128: {"seg_length": 32, "k_block": 32, "vec_len": 4},
+        128: {"seg_length": 512, "k_block": 32, "vec_len": 4},
     }
 
     def __init__(self, row_offsets, column_indices, values, device, m, n, k=128, config=None):

@@ -91,6 +91,20 @@ def sddmm_row_l1_error(got, ref64, row_ptr):
     return float(np.max(emax / np.maximum(l1, 1e-30)))
 
 
+def sddmm_row_l1_errors(got, ref64, scale, row_ptr):
+    """Per non-empty row: (max|got-ref| / sum|ref|, condition number sum(scale) / sum|ref|),
+    where scale[idx] = |val| * sum_k |lhs*rhs| is the magnitude of the summed terms."""
+    rp = np.asarray(row_ptr, dtype=np.int64)
+    nonempty = np.nonzero(np.diff(rp) > 0)[0]
+    if len(nonempty) == 0:
+        return np.zeros(0), np.zeros(0)
+    err = np.abs(got.astype(np.float64) - ref64)
+    emax = np.maximum.reduceat(err, rp[nonempty])
+    l1 = np.maximum(np.add.reduceat(np.abs(ref64), rp[nonempty]), 1e-300)
+    cond = np.add.reduceat(scale, rp[nonempty]) / l1
+    return emax / l1, cond
+
+
 def spmm_row_l1_error(got, ref64):
     """max over rows of  max_j|got-ref| / sum_j|ref|."""
     err = np.abs(got.astype(np.float64) - ref64).max(axis=1)

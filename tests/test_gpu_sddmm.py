@@ -23,25 +23,43 @@ REFERENCE_CONFIGS = [
 ]
 
 
+WELL_CONDITIONED = 100.0
+
+
 def _check(csr, rp, col, val, lhs, rhs, half=False, ref_rule=True):
+    """Tolerances.  (1) Row-L1 bound of the target: max|err| over a row's outputs /
+    sum|ref| over the row <= 1e-4 (fp32) or 2e-3 (fp16 operands), asserted on every row
+    whose condition number sum|terms| / sum|ref| is <= 100.  A row that consists of one
+    or two cancelling dot products can exceed it under ANY fp32 summation order; there the
+    GPU must not be worse than twice the reference's own CPU loop (main.cu:65-91).
+    (2) Per element, |err| <= 2e-6 * |val| * sum_k|lhs*rhs| (fp32 operands), everywhere.
+    (3) The reference tests' own rule against the reference's CPU loop: no element with
+    both abs and rel error > 1e-3."""
     import oracle
     from gpu_common import TOL_F16, TOL_F32, check_csr_decomposition, round_half, run_sddmm
-    from helpers import reference_error_count, sddmm_row_l1_error
+    from helpers import reference_error_count, sddmm_row_l1_errors
     check_csr_decomposition(csr, rp)
     out = run_sddmm(csr, lhs, rhs, half)
     assert out.shape == (len(val),) and out.dtype == np.float32
     if half:
         lhs, rhs = round_half(lhs), round_half(rhs)
+    tol = TOL_F16 if half else TOL_F32
     ref64, scale = oracle.sddmm_f64(rp, col, val, lhs, rhs, with_abs=True)
-    err = sddmm_row_l1_error(out, ref64, rp)
-    assert err <= (TOL_F16 if half else TOL_F32), f"row-L1 error {err}"
+    err, cond = sddmm_row_l1_errors(out, ref64, scale, rp)
+    good = cond <= WELL_CONDITIONED
+    worst = float(err[good].max(initial=0.0))
+    assert worst <= tol, f"row-L1 error {worst}"
+    if (~good).any():
+        cpu32 = oracle.sddmm_f32(rp, col, val, lhs, rhs)
+        cpu_err, _ = sddmm_row_l1_errors(cpu32, ref64, scale, rp)
+        assert float(err[~good].max()) <= max(tol, 2 * float(cpu_err[~good].max())), \
+            f"ill-conditioned rows: GPU {err[~good].max()} vs reference CPU loop {cpu_err[~good].max()}"
     if not half:
-        # per element, against the magnitude of the terms that were summed: a few ulp per term
         strict = np.abs(out - ref64) / np.maximum(scale, 1e-30)
         assert strict.max(initial=0.0) <= 2e-6, f"per-element error {strict.max()}"
         if ref_rule:
             assert reference_error_count(out, oracle.sddmm_f32(rp, col, val, lhs, rhs)) == 0
-    return err
+    return worst
 
 
 @pytest.mark.parametrize("k", [128, 32])
@@ -50,14 +68,16 @@ def test_reference_table(k):
     generators (rows padded to 4 with explicit zeros), its decomposition parameters,
     its CPU loop and its pass rule."""
     from gpu_common import make_csr
-    from rode_amd import workloads
+    from rode_amd import RoDeCSR, workloads
     worst = 0.0
     for m, n, per_row in REFERENCE_CONFIGS:
         rp, col, val = workloads.reference_csr(m, n, per_row, poisson=(k == 128), pad_to=4, seed=42)
         lhs = workloads.reference_dense(m, k, 123)
         rhs = workloads.reference_dense(n, k, 456)
-        csr = make_csr(rp, col, val, m, n, k)  # CONFIGS[k]: (512,32,4) for 32, (32,32,4) for 128
-        worst = max(worst, _check(csr, rp, col, val, lhs, rhs))
+        ref_seg = RoDeCSR.REFERENCE_CONFIGS[k]["seg_length"]  # (512,32,4) for 32, (32,32,4) for 128
+        for seg in sorted({ref_seg, RoDeCSR.CONFIGS[k]["seg_length"]}):
+            csr = make_csr(rp, col, val, m, n, k, seg)
+            worst = max(worst, _check(csr, rp, col, val, lhs, rhs))
     print(f"k={k}: worst row-L1 error over {len(REFERENCE_CONFIGS)} reference configs: {worst:.2e}")
 
 
@@ -71,7 +91,7 @@ def test_reference_stress():
         m, n = random.randint(10, 2000), random.randint(10, 2000)
         per_row = random.randint(1, min(n, 200))
         rp, col, val = workloads.reference_csr(m, n, per_row, poisson=True)
-        csr = make_csr(rp, col, val, m, n, 128)
+        csr = make_csr(rp, col, val, m, n, 128, 32)
         _check(csr, rp, col, val, workloads.reference_dense(m, 128, 123), workloads.reference_dense(n, 128, 456))
 
 
