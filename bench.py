@@ -38,6 +38,8 @@ def parse_args():
     p.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (debugging only)")
     p.add_argument("--cpu-seconds", type=float, default=8.0, help="CPU time budget per operation of the baseline")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--calibrate", action="store_true",
+                   help="also run one plain device copy of 256 MiB (a known size to scale profiler counters by)")
     return p.parse_args()
 
 
@@ -157,6 +159,13 @@ def main():
         kernels["sddmm_residue"] = event_time(lambda: sddmm(0, csr.m2), reps)
     spmm_ms = event_time(lambda: (C.zero_(), spmm(csr.m1, csr.m2)), reps)
     sddmm_ms = event_time(lambda: sddmm(csr.m1, csr.m2), reps)
+
+    if args.calibrate:
+        src = torch.ones(64 * 2**20, device=dev)  # 256 MiB read + 256 MiB written by one elementwise copy kernel
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     split = work_split(row_ptr, col, n)
     per_kernel = {}
