@@ -38,6 +38,8 @@ def parse_args():
     p.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (debugging only)")
     p.add_argument("--cpu-seconds", type=float, default=8.0, help="CPU time budget per operation of the baseline")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--two-streams", action="store_true",
+                   help="residue kernels on a second stream (forked from / joined to the first with events)")
     p.add_argument("--calibrate", action="store_true",
                    help="also run one plain device copy of 256 MiB (a known size to scale profiler counters by)")
     return p.parse_args()
@@ -109,16 +111,33 @@ def main():
     spmm_fn = lib.rode_hip_spmm_f32 if args.dtype == "f32" else lib.rode_hip_spmm_f16
     sddmm_fn = lib.rode_hip_sddmm_f32 if args.dtype == "f32" else lib.rode_hip_sddmm_f16
 
+    main_stream = torch.cuda.current_stream()
+    side = torch.cuda.Stream() if args.two_streams else None
+
+    def fork():
+        if side is None:
+            return stream
+        side.wait_stream(main_stream)
+        return side.cuda_stream
+
+    def join():
+        if side is not None:
+            main_stream.wait_stream(side)
+
     def spmm(m1, m2):
+        s2 = fork()
         _lib.check(spmm_fn(m1, m2, n, k, csr.values.data_ptr(), csr.column_indices.data_ptr(),
                            csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
-                           csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, stream), "spmm")
+                           csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, s2), "spmm")
+        join()
 
     def sddmm(m1, m2):
+        s2 = fork()
         _lib.check(sddmm_fn(m1, m2, n, k, csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
                             csr.st_offsets.data_ptr(), csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
-                            csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), out.data_ptr(), stream, stream),
+                            csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), out.data_ptr(), stream, s2),
                    "sddmm")
+        join()
 
     def step():
         C.zero_()

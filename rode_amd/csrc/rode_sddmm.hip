@@ -14,7 +14,9 @@
 //     product of slot e in lane e;
 //   * block kernel: one wave walks one block segment, 64 slots per step, the
 //     lhs row slice stays in registers for the whole segment;
-//   * residue kernel: each half-wave takes one residue row (< 32 slots).
+//   * residue kernel: each group of LPR lanes takes one residue row (< 32 slots),
+//     so a wave works on 64 / LPR rows at once (2 at K=128 fp32, 8 at K=32):
+//     short rows are latency-bound and need many rows in flight per wave.
 #include "rode_device.hpp"
 #include "rode_internal.hpp"
 
@@ -126,9 +128,10 @@ sddmm_block_kernel(int m1, const int* __restrict__ block_rows, const int* __rest
     }
 }
 
-// One 32-lane half per residue row.  Tail selection follows RoDeSddmm.cu:237-243:
+// One group of LPR lanes per residue row.  Tail selection follows RoDeSddmm.cu:237-243:
 // with N = len + (s & 3), rows with N >= 32 keep only their last N % 32 slots
 // starting at (s & ~3) + floor(N / 32) * 32; shorter rows are taken whole.
+// Lane ls of the group owns the slots ls, ls + LPR, ... (value, result, store).
 template <typename T, int K>
 __global__ void __launch_bounds__(kWgThreads)
 sddmm_residue_kernel(int m2, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
@@ -136,35 +139,78 @@ sddmm_residue_kernel(int m2, const int* __restrict__ residue_rows, const int* __
                      const T* __restrict__ rhs, float* __restrict__ out)
 {
     using S = SddmmShape<T, K>;
-    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
+    constexpr int VEC = S::kVec, LPR = S::kLpr;
+    constexpr int RPW = kWave / LPR;          // rows per wave
+    constexpr int OWN = kBlockItems / LPR;    // slots owned by one lane
+    constexpr int LQ = LPR / 4;               // lane quads per group
+    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * RPW * kBlockItems];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * 2 + (lane >> 5);
+    const int group = lane / LPR, ls = lane % LPR;
+    const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * RPW + group;
+    if (item >= m2) return;
 
-    int row = 0, first = 0, cnt = 0;
-    if (item < m2) {
-        row = residue_rows[item];
-        const int s = row_ptr[row], e = row_ptr[row + 1];
-        const int pad = s & (kVecLen - 1);
-        const int N = e - s + pad;
-        if (N >= kBlockItems) {
-            first = (s - pad) + N / kBlockItems * kBlockItems;
-            cnt = N % kBlockItems;
-        } else {
-            first = s;
-            cnt = e - s;
-        }
+    const int row = residue_rows[item];
+    const int s = row_ptr[row], e = row_ptr[row + 1];
+    const int pad = s & (kVecLen - 1);
+    const int N = e - s + pad;
+    int first = s, cnt = e - s;
+    if (N >= kBlockItems) {
+        first = (s - pad) + N / kBlockItems * kBlockItems;
+        cnt = N % kBlockItems;
     }
     if (cnt <= 0) return; // an empty, unaligned row is listed as a residue but owns no slot
 
-    const int slot = lane & 31;
-    const int idx = first + min(slot, cnt - 1);
-    const int c = col[idx];
-    const float v = val[idx];
-    float a[S::kVec];
+    int* my_cols = lds + (wave * RPW + group) * kBlockItems;
+    float v[OWN];
+    const int padded = (cnt + 3) & ~3; // slots past the tail repeat its last column
+#pragma unroll
+    for (int i = 0; i < OWN; ++i) {
+        const int slot = ls + i * LPR;
+        v[i] = 0.f;
+        if (slot < padded) {
+            const int idx = first + min(slot, cnt - 1);
+            my_cols[slot] = col[idx];
+            v[i] = val[idx];
+        }
+    }
+    float a[VEC];
     load_lhs_slice<T, K>(lhs, row, lane, a);
-    const T* rhs_lane = rhs + (lane % S::kLpr) * S::kVec;
-    const float d = sddmm_unit<T, K, false>(rhs_lane, a, c, cnt, lds + wave * kWave, lane);
-    if (slot < cnt) out[idx] = v * d;
+    const T* rhs_lane = rhs + ls * VEC;
+    wave_lds_sync();
+
+    float res[OWN];
+#pragma unroll
+    for (int i = 0; i < OWN; ++i) res[i] = 0.f;
+    const int nquads = padded / 4;
+#pragma unroll
+    for (int q = 0; q < kBlockItems / 4; ++q) {
+        if (q < nquads) {
+            const int4 c4 = *reinterpret_cast<const int4*>(my_cols + 4 * q);
+            const int c[4] = {c4.x, c4.y, c4.z, c4.w};
+            float p[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float b[VEC];
+                DenseVec<T>::load(rhs_lane + (size_t)c[j] * K, b);
+                float d = 0.f;
+#pragma unroll
+                for (int x = 0; x < VEC; ++x) d = fmaf(a[x], b[x], d);
+                p[j] = d;
+            }
+            const bool hi2 = ls & 2, hi1 = ls & 1;
+            const float q0 = (hi2 ? p[2] : p[0]) + lane_xor2(hi2 ? p[0] : p[2]);
+            const float q1 = (hi2 ? p[3] : p[1]) + lane_xor2(hi2 ? p[1] : p[3]);
+            float r = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
+            r = butterfly_sum<4, LPR>(r);
+            // slot 4q + (ls & 3) belongs to lane (4q + (ls & 3)) % LPR, register (4q) / LPR
+            if ((ls >> 2) == q % LQ) res[q / LQ] = r;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < OWN; ++i) {
+        const int slot = ls + i * LPR;
+        if (slot < cnt) out[first + slot] = v[i] * res[i];
+    }
 }
 
 inline int grid_for_waves(long long nwaves)
@@ -184,7 +230,8 @@ hipError_t launch(int m1, int m2, const int* block_rows, const int* residue_rows
                                                                             lhs, rhs, out);
     }
     if (m2 > 0) {
-        sddmm_residue_kernel<T, K><<<grid_for_waves(((long long)m2 + 1) / 2), kWgThreads, 0, s2>>>(
+        constexpr int RPW = kWave / SddmmShape<T, K>::kLpr;
+        sddmm_residue_kernel<T, K><<<grid_for_waves(((long long)m2 + RPW - 1) / RPW), kWgThreads, 0, s2>>>(
             m2, residue_rows, row_ptr, col, val, lhs, rhs, out);
     }
     return hipGetLastError();

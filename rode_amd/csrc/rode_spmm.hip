@@ -13,9 +13,10 @@
 //     interleaved slot quads, the partial rows are combined with a butterfly
 //     over the groups and added to C with hardware fp32 atomics (always, as in
 //     RoDeSpmm.cu:464-474: a long row has several segments and usually a residue);
-//   * residue kernel: one 32-lane half per residue row; rows shorter than 32
-//     slots are stored with plain 128-bit stores, tails of longer rows are
-//     added atomically (RoDeSpmm.cu:76-82, 173-194).
+//   * residue kernel: one group of LPR lanes per residue row, 64 / LPR rows per
+//     wave (short rows are latency-bound and need many rows in flight); rows
+//     shorter than 32 slots are stored with plain 128-bit stores, tails of
+//     longer rows are added atomically (RoDeSpmm.cu:76-82, 173-194).
 //
 // Slots that belong to the previous row (the `start & 3` head of an unaligned
 // segment) are neutralised with value 0 *and* the column of the first real slot,
@@ -33,7 +34,6 @@ struct SpmmShape {
     static constexpr int kVec = DenseVec<T>::kElems;
     static constexpr int kLpr = TN / kVec;          // lanes that cover one B-row tile
     static constexpr int kGroupsWave = kWave / kLpr; // lane groups per wave
-    static constexpr int kGroupsHalf = 32 / kLpr;    // lane groups per 32-lane half
     static_assert(TN % kVec == 0 && kLpr >= 4 && kLpr <= 32 && (kLpr & (kLpr - 1)) == 0,
                   "unsupported tile width for this dense type");
 };
@@ -136,7 +136,8 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
     }
 }
 
-// One 32-lane half per residue row (tail selection: RoDeSpmm.cu:71-82).
+// One group of LPR lanes per residue row (tail selection: RoDeSpmm.cu:71-82); the
+// group walks its row's slot quads one after the other, no cross-lane reduction.
 template <typename T, int TN>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
@@ -144,11 +145,14 @@ spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const i
                     float* __restrict__ C)
 {
     using S = SpmmShape<T, TN>;
-    constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsHalf;
-    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
-    __shared__ __attribute__((aligned(16))) float lds_v[kWavesPerWg * kWave];
+    constexpr int VEC = S::kVec, LPR = S::kLpr;
+    constexpr int RPW = kWave / LPR;        // rows per wave
+    constexpr int OWN = kBlockItems / LPR;  // slots staged by one lane
+    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * RPW * kBlockItems];
+    __shared__ __attribute__((aligned(16))) float lds_v[kWavesPerWg * RPW * kBlockItems];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * 2 + (lane >> 5);
+    const int group = lane / LPR, ls = lane % LPR;
+    const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * RPW + group;
     if (item >= m2) return;
 
     const int row = residue_rows[item];
@@ -162,35 +166,34 @@ spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const i
         cnt = N % kBlockItems;
     }
 
-    const int slot = lane & 31;
-    const int ls = slot % LPR, group = slot / LPR;
     const int tile = blockIdx.y * TN;
-    int* my_c = lds_c + wave * kWave + (lane & 32);
-    float* my_v = lds_v + wave * kWave + (lane & 32);
+    int* my_c = lds_c + (wave * RPW + group) * kBlockItems;
+    float* my_v = lds_v + (wave * RPW + group) * kBlockItems;
 
     float acc[VEC];
 #pragma unroll
     for (int x = 0; x < VEC; ++x) acc[x] = 0.f;
 
     if (cnt > 0) {
-        // slots past the tail repeat its last column with value 0
-        my_c[slot] = col[first + min(slot, cnt - 1)];
-        my_v[slot] = slot < cnt ? val[first + slot] : 0.f;
+        const int padded = (cnt + 3) & ~3; // slots past the tail repeat its last column with value 0
+#pragma unroll
+        for (int i = 0; i < OWN; ++i) {
+            const int slot = ls + i * LPR;
+            if (slot < padded) {
+                my_c[slot] = col[first + min(slot, cnt - 1)];
+                my_v[slot] = slot < cnt ? val[first + slot] : 0.f;
+            }
+        }
         wave_lds_sync();
-        spmm_gather<T, TN, 8 / G, false>(B + tile + ls * VEC, (size_t)n, acc, my_c, my_v, group, G, (cnt + 3) / 4);
+        spmm_gather<T, TN, kBlockItems / 4, false>(B + tile + ls * VEC, (size_t)n, acc, my_c, my_v, 0, 1, padded / 4);
     }
 
-#pragma unroll
-    for (int x = 0; x < VEC; ++x) acc[x] = butterfly_sum<LPR, 32>(acc[x]);
-
     float* c_lane = C + (size_t)row * n + tile + ls * VEC;
-    if (group == 0) {
-        if (accumulate) {
+    if (accumulate) {
 #pragma unroll
-            for (int x = 0; x < VEC; ++x) atomicAdd(c_lane + x, acc[x]);
-        } else {
-            store_row<VEC>(c_lane, acc);
-        }
+        for (int x = 0; x < VEC; ++x) atomicAdd(c_lane + x, acc[x]);
+    } else {
+        store_row<VEC>(c_lane, acc);
     }
 }
 
@@ -212,7 +215,8 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
         spmm_block_kernel<T, TN><<<grid, kWgThreads, 0, s1>>>(m1, n, block_rows, st_off, row_ptr, col, val, B, C);
     }
     if (m2 > 0) {
-        dim3 grid(grid_for_waves(((long long)m2 + 1) / 2), tiles);
+        constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
+        dim3 grid(grid_for_waves(((long long)m2 + RPW - 1) / RPW), tiles);
         spmm_residue_kernel<T, TN><<<grid, kWgThreads, 0, s2>>>(m2, n, residue_rows, row_ptr, col, val, B, C);
     }
     return hipGetLastError();
