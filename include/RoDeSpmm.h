@@ -17,4 +17,15 @@ void RoDeSpmm_n128(int m1, int m2, int k, int n, const float* values, const int*
                    const int* row_seg_st_offsets, const float* B, float* C, hipStream_t stream1,
                    hipStream_t stream2);
 
+// fp64 overloads (RoDe_SpMM/RoDeSpmm.h:10-14).
+void RoDeSpmm_n32(int m1, int m2, int k, int n, const double* values, const int* column_indices,
+                  const int* row_offsets, const int* row_indices1, const int* row_indices2,
+                  const int* row_seg_st_offsets, const double* B, double* C, hipStream_t stream1,
+                  hipStream_t stream2);
+
+void RoDeSpmm_n128(int m1, int m2, int k, int n, const double* values, const int* column_indices,
+                   const int* row_offsets, const int* row_indices1, const int* row_indices2,
+                   const int* row_seg_st_offsets, const double* B, double* C, hipStream_t stream1,
+                   hipStream_t stream2);
+
 #endif

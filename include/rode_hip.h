@@ -71,6 +71,13 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
                       const int* d_row_seg_st_offsets, const float* d_B, float* d_C, void* stream1,
                       void* stream2);
 
+/* fp64 values, B and C.  Replaces the double overloads of RoDeSpmm_n32 / RoDeSpmm_n128,
+ * RoDe_SpMM/RoDeSpmm.h:10-14, RoDeSpmm.cu:521-529.  Same contract as rode_hip_spmm_f32. */
+int rode_hip_spmm_f64(int m1, int m2, int k, int n, const double* d_values, const int* d_column_indices,
+                      const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
+                      const int* d_row_seg_st_offsets, const double* d_B, double* d_C, void* stream1,
+                      void* stream2);
+
 /* Same with B stored as IEEE fp16 (no reference entry point; operand semantics of the
  * unused helper VectorCompute<half4>::FMA, RoDe_SpMM/common_utils.h:183-230:
  * widen to fp32, fp32 FMA). */

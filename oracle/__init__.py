@@ -10,5 +10,6 @@ from .oracle import (  # noqa: F401
     sddmm_f32,
     sddmm_f64,
     spmm_f32,
+    spmm_d,
     spmm_f64,
 )

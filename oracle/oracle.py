@@ -40,6 +40,7 @@ def _load():
     for name in ("oracle_spmm_f32", "oracle_spmm_f32_mt"):
         getattr(lib, name).argtypes = [c_int, c_int, _i32p, _i32p, _f32p, _f32p, _f32p]
     lib.oracle_spmm_f64.argtypes = [c_int, c_int, _i32p, _i32p, _f32p, _f32p, _f64p, ctypes.c_void_p]
+    lib.oracle_spmm_d.argtypes = [c_int, c_int, _i32p, _i32p, _f64p, _f64p, _f64p]
     _lib = lib
     return lib
 
@@ -107,3 +108,13 @@ def spmm_f64(row_ptr, col, val, B, with_abs=False):
     ab = np.zeros((m, n), dtype=np.float64) if with_abs else None
     _load().oracle_spmm_f64(m, n, row_ptr, col, val, B, C, ab.ctypes.data if with_abs else None)
     return (C, ab) if with_abs else C
+
+
+def spmm_d(row_ptr, col, val, B):
+    """SpMM with fp64 values and operands (the reference's double overloads)."""
+    row_ptr, col = _i32(row_ptr), _i32(col)
+    val, B = np.ascontiguousarray(val, dtype=np.float64), np.ascontiguousarray(B, dtype=np.float64)
+    m, n = row_ptr.size - 1, B.shape[1]
+    C = np.zeros((m, n), dtype=np.float64)
+    _load().oracle_spmm_d(m, n, row_ptr, col, val, B, C)
+    return C

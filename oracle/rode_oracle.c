@@ -217,3 +217,22 @@ void oracle_spmm_f64(int m, int n, const int *row_offsets, const int *column_ind
         }
     }
 }
+
+/* SpMM with fp64 values, B and C: the arithmetic of the double overloads
+ * RoDe_SpMM/RoDeSpmm.cu:521-529 (same kernels instantiated for double). */
+void oracle_spmm_d(int m, int n, const int *row_offsets, const int *column_indices,
+                   const double *values, const double *B, double *C)
+{
+#pragma omp parallel for schedule(guided, 64)
+    for (int row = 0; row < m; ++row) {
+        double *c = C + (size_t)row * n;
+        for (int j = 0; j < n; ++j)
+            c[j] = 0.0;
+        for (int idx = row_offsets[row]; idx < row_offsets[row + 1]; ++idx) {
+            const double *b = B + (size_t)column_indices[idx] * n;
+            double v = values[idx];
+            for (int j = 0; j < n; ++j)
+                c[j] += v * b[j];
+        }
+    }
+}

@@ -49,6 +49,18 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
                                     d_column_indices, d_values, d_B, d_C, as_stream(stream1), as_stream(stream2));
 }
 
+int rode_hip_spmm_f64(int m1, int m2, int k, int n, const double* d_values, const int* d_column_indices,
+                      const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
+                      const int* d_row_seg_st_offsets, const double* d_B, double* d_C, void* stream1, void* stream2)
+{
+    (void)k;
+    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
+    if (m1 == 0 && m2 == 0) return hipSuccess;
+    if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
+    return rode::spmm_launch<double>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
+                                     d_column_indices, d_values, d_B, d_C, as_stream(stream1), as_stream(stream2));
+}
+
 int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
                       const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
                       const int* d_row_seg_st_offsets, const void* d_B_half, float* d_C, void* stream1,
@@ -118,6 +130,24 @@ void RoDeSpmm_n128(int m1, int m2, int k, int n, const float* values, const int*
 {
     report("RoDeSpmm_n128", (n % 64) ? (int)hipErrorInvalidValue
                                      : rode_hip_spmm_f32(m1, m2, k, n, values, column_indices, row_offsets,
+                                                         row_indices1, row_indices2, row_seg_st_offsets, B, C,
+                                                         stream1, stream2));
+}
+
+void RoDeSpmm_n32(int m1, int m2, int k, int n, const double* values, const int* column_indices,
+                  const int* row_offsets, const int* row_indices1, const int* row_indices2,
+                  const int* row_seg_st_offsets, const double* B, double* C, hipStream_t stream1, hipStream_t stream2)
+{
+    report("RoDeSpmm_n32", rode_hip_spmm_f64(m1, m2, k, n, values, column_indices, row_offsets, row_indices1,
+                                             row_indices2, row_seg_st_offsets, B, C, stream1, stream2));
+}
+
+void RoDeSpmm_n128(int m1, int m2, int k, int n, const double* values, const int* column_indices,
+                   const int* row_offsets, const int* row_indices1, const int* row_indices2,
+                   const int* row_seg_st_offsets, const double* B, double* C, hipStream_t stream1, hipStream_t stream2)
+{
+    report("RoDeSpmm_n128", (n % 64) ? (int)hipErrorInvalidValue
+                                     : rode_hip_spmm_f64(m1, m2, k, n, values, column_indices, row_offsets,
                                                          row_indices1, row_indices2, row_seg_st_offsets, B, C,
                                                          stream1, stream2));
 }

@@ -67,14 +67,26 @@ __device__ __forceinline__ float butterfly_sum(float v)
     return v;
 }
 
+__device__ __forceinline__ double lane_xor_any(double v, int m) { return __shfl_xor(v, m, kWave); }
+
+template <int LO, int HI>
+__device__ __forceinline__ double butterfly_sum(double v)
+{
+#pragma unroll
+    for (int m = LO; m < HI; m <<= 1) v += lane_xor_any(v, m);
+    return v;
+}
+
 // ---- dense operand access --------------------------------------------------
 // One lane reads DenseVec<T>::kElems consecutive dense elements with a single
-// 128-bit load and widens them to fp32.
+// 128-bit load and widens them to the accumulation type (fp32 for fp32 / fp16
+// operands, fp64 for fp64 operands).
 template <typename T>
 struct DenseVec;
 
 template <>
 struct DenseVec<float> {
+    using Acc = float;
     static constexpr int kElems = 4;
     __device__ __forceinline__ static void load(const float* p, float (&out)[4])
     {
@@ -84,7 +96,19 @@ struct DenseVec<float> {
 };
 
 template <>
+struct DenseVec<double> {
+    using Acc = double;
+    static constexpr int kElems = 2;
+    __device__ __forceinline__ static void load(const double* p, double (&out)[2])
+    {
+        const double2 v = *reinterpret_cast<const double2*>(p);
+        out[0] = v.x; out[1] = v.y;
+    }
+};
+
+template <>
 struct DenseVec<__half> {
+    using Acc = float;
     static constexpr int kElems = 8;
     __device__ __forceinline__ static void load(const __half* p, float (&out)[8])
     {

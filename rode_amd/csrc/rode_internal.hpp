@@ -12,10 +12,15 @@ hipError_t preprocess_launch(int seg, int kblock, int veclen, int M, const int* 
                              int* st_off, int* residue_r_ind, int* n_blk, int* n_res, void* workspace,
                              int capacity_blocks, hipStream_t stream);
 
+// T = dense operand type; values, accumulators and C are float for T = float / __half
+// and double for T = double.
+template <typename T> struct SpmmAcc { using type = float; };
+template <> struct SpmmAcc<double> { using type = double; };
+
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
-                       const int* row_ptr, const int* col, const float* val, const T* B, float* C, hipStream_t s1,
-                       hipStream_t s2);
+                       const int* row_ptr, const int* col, const typename SpmmAcc<T>::type* val, const T* B,
+                       typename SpmmAcc<T>::type* C, hipStream_t s1, hipStream_t s2);
 
 template <typename T>
 hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int* residue_rows, const int* st_off,

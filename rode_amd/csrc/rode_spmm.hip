@@ -25,12 +25,15 @@
 #include "rode_device.hpp"
 #include "rode_internal.hpp"
 
+#include <type_traits>
+
 namespace rode {
 
 namespace {
 
 template <typename T, int TN>
 struct SpmmShape {
+    using Acc = typename DenseVec<T>::Acc;          // type of values, accumulators and C
     static constexpr int kVec = DenseVec<T>::kElems;
     static constexpr int kLpr = TN / kVec;          // lanes that cover one B-row tile
     static constexpr int kGroupsWave = kWave / kLpr; // lane groups per wave
@@ -38,29 +41,42 @@ struct SpmmShape {
                   "unsupported tile width for this dense type");
 };
 
+__device__ __forceinline__ void load_quad(const float* p, float (&v)[4])
+{
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load_quad(const double* p, double (&v)[4])
+{
+    const double2 t0 = *reinterpret_cast<const double2*>(p), t1 = *reinterpret_cast<const double2*>(p + 2);
+    v[0] = t0.x; v[1] = t0.y; v[2] = t1.x; v[3] = t1.y;
+}
+
 // acc += sum over the slot quads {first_quad, first_quad + stride, ...} < nquads of
 // value * B[col, tile].  QUADS_MAX bounds the trip count at compile time.
 template <typename T, int TN, int QUADS_MAX, bool FULL>
 __device__ __forceinline__ void spmm_gather(const T* __restrict__ b_lane, size_t ldb,
-                                            float (&acc)[SpmmShape<T, TN>::kVec], const int* lds_col,
-                                            const float* lds_val, int first_quad, int stride, int nquads)
+                                            typename DenseVec<T>::Acc (&acc)[SpmmShape<T, TN>::kVec],
+                                            const int* lds_col, const typename DenseVec<T>::Acc* lds_val,
+                                            int first_quad, int stride, int nquads)
 {
+    using A = typename DenseVec<T>::Acc;
     constexpr int VEC = SpmmShape<T, TN>::kVec;
 #pragma unroll
     for (int i = 0; i < QUADS_MAX; ++i) {
         const int q = first_quad + i * stride;
         if (FULL || q < nquads) {
             const int4 c4 = *reinterpret_cast<const int4*>(lds_col + 4 * q);
-            const float4 v4 = *reinterpret_cast<const float4*>(lds_val + 4 * q);
             const int c[4] = {c4.x, c4.y, c4.z, c4.w};
-            const float v[4] = {v4.x, v4.y, v4.z, v4.w};
-            float b[4][VEC];
+            A v[4];
+            load_quad(lds_val + 4 * q, v);
+            A b[4][VEC];
 #pragma unroll
             for (int j = 0; j < 4; ++j) DenseVec<T>::load(b_lane + (size_t)c[j] * ldb, b[j]);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int x = 0; x < VEC; ++x) acc[x] = fmaf(v[j], b[j][x], acc[x]);
+                for (int x = 0; x < VEC; ++x) acc[x] = fma(v[j], b[j][x], acc[x]);
         }
     }
 }
@@ -73,18 +89,27 @@ __device__ __forceinline__ void store_row(float* dst, const float (&acc)[VEC])
         *reinterpret_cast<float4*>(dst + x) = make_float4(acc[x], acc[x + 1], acc[x + 2], acc[x + 3]);
 }
 
+template <int VEC>
+__device__ __forceinline__ void store_row(double* dst, const double (&acc)[VEC])
+{
+#pragma unroll
+    for (int x = 0; x < VEC; x += 2) *reinterpret_cast<double2*>(dst + x) = make_double2(acc[x], acc[x + 1]);
+}
+
 // One wave per block segment (see sddmm_block_kernel for the slot arithmetic,
 // identical at RoDeSpmm.cu:210-234).
 template <typename T, int TN>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* __restrict__ st_off,
-                  const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
-                  const T* __restrict__ B, float* __restrict__ C)
+                  const int* __restrict__ row_ptr, const int* __restrict__ col,
+                  const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
+                  typename DenseVec<T>::Acc* __restrict__ C)
 {
     using S = SpmmShape<T, TN>;
+    using A = typename S::Acc;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
-    __shared__ __attribute__((aligned(16))) float lds_v[kWavesPerWg * kWave];
+    __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int seg = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (seg >= m1) return;
@@ -100,21 +125,21 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
     const int tile = blockIdx.y * TN;
     const T* b_lane = B + tile + ls * VEC;
     int* my_c = lds_c + wave * kWave;
-    float* my_v = lds_v + wave * kWave;
+    A* my_v = lds_v + wave * kWave;
 
-    float acc[VEC];
+    A acc[VEC];
 #pragma unroll
-    for (int x = 0; x < VEC; ++x) acc[x] = 0.f;
+    for (int x = 0; x < VEC; ++x) acc[x] = A(0);
 
     for (int off = 0; off < cnt; off += kWave) {
         const int slot = off + lane;
         const int live = min(cnt - off, kWave); // 64, or 32 on a trailing half step
         int c = 0;
-        float v = 0.f;
+        A v = A(0);
         if (lane < live) {
             const bool head = slot < mask; // previous row's slots
             c = col[base + (head ? mask : slot)];
-            v = head ? 0.f : val[base + slot];
+            v = head ? A(0) : val[base + slot];
         }
         my_c[lane] = c;
         my_v[lane] = v;
@@ -128,10 +153,10 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
 
     // combine the lane groups, then spread the atomics over them
     constexpr int EPG = VEC / G > 0 ? VEC / G : 1; // elements each group adds
-    float* c_lane = C + (size_t)row * n + tile + ls * VEC;
+    A* c_lane = C + (size_t)row * n + tile + ls * VEC;
 #pragma unroll
     for (int x = 0; x < VEC; ++x) {
-        const float total = butterfly_sum<LPR, kWave>(acc[x]);
+        const A total = butterfly_sum<LPR, kWave>(acc[x]);
         if (group == x / EPG) atomicAdd(c_lane + x, total);
     }
 }
@@ -141,15 +166,16 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
 template <typename T, int TN>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
-                    const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ B,
-                    float* __restrict__ C)
+                    const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
+                    const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C)
 {
     using S = SpmmShape<T, TN>;
+    using A = typename S::Acc;
     constexpr int VEC = S::kVec, LPR = S::kLpr;
     constexpr int RPW = kWave / LPR;        // rows per wave
     constexpr int OWN = kBlockItems / LPR;  // slots staged by one lane
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * RPW * kBlockItems];
-    __shared__ __attribute__((aligned(16))) float lds_v[kWavesPerWg * RPW * kBlockItems];
+    __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * RPW * kBlockItems];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int group = lane / LPR, ls = lane % LPR;
     const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * RPW + group;
@@ -168,11 +194,11 @@ spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const i
 
     const int tile = blockIdx.y * TN;
     int* my_c = lds_c + (wave * RPW + group) * kBlockItems;
-    float* my_v = lds_v + (wave * RPW + group) * kBlockItems;
+    A* my_v = lds_v + (wave * RPW + group) * kBlockItems;
 
-    float acc[VEC];
+    A acc[VEC];
 #pragma unroll
-    for (int x = 0; x < VEC; ++x) acc[x] = 0.f;
+    for (int x = 0; x < VEC; ++x) acc[x] = A(0);
 
     if (cnt > 0) {
         const int padded = (cnt + 3) & ~3; // slots past the tail repeat its last column with value 0
@@ -181,14 +207,14 @@ spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const i
             const int slot = ls + i * LPR;
             if (slot < padded) {
                 my_c[slot] = col[first + min(slot, cnt - 1)];
-                my_v[slot] = slot < cnt ? val[first + slot] : 0.f;
+                my_v[slot] = slot < cnt ? val[first + slot] : A(0);
             }
         }
         wave_lds_sync();
         spmm_gather<T, TN, kBlockItems / 4, false>(B + tile + ls * VEC, (size_t)n, acc, my_c, my_v, 0, 1, padded / 4);
     }
 
-    float* c_lane = C + (size_t)row * n + tile + ls * VEC;
+    A* c_lane = C + (size_t)row * n + tile + ls * VEC;
     if (accumulate) {
 #pragma unroll
         for (int x = 0; x < VEC; ++x) atomicAdd(c_lane + x, acc[x]);
@@ -206,8 +232,8 @@ inline int grid_for_waves(long long nwaves)
 
 template <typename T, int TN>
 hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
-                  const int* row_ptr, const int* col, const float* val, const T* B, float* C, hipStream_t s1,
-                  hipStream_t s2)
+                  const int* row_ptr, const int* col, const typename DenseVec<T>::Acc* val, const T* B,
+                  typename DenseVec<T>::Acc* C, hipStream_t s1, hipStream_t s2)
 {
     const int tiles = n / TN;
     if (m1 > 0) {
@@ -226,11 +252,17 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
 
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
-                       const int* row_ptr, const int* col, const float* val, const T* B, float* C, hipStream_t s1,
-                       hipStream_t s2)
+                       const int* row_ptr, const int* col, const typename SpmmAcc<T>::type* val, const T* B,
+                       typename SpmmAcc<T>::type* C, hipStream_t s1, hipStream_t s2)
 {
+    static_assert(std::is_same<typename SpmmAcc<T>::type, typename DenseVec<T>::Acc>::value, "accumulation type");
     if (n <= 0 || n % 32 != 0) return hipErrorInvalidValue;
-    if (n % 128 == 0) return launch<T, 128>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
+    // widest tile whose row is covered by at most 32 lanes of 128-bit loads
+    constexpr int kMaxTile = 32 * DenseVec<T>::kElems >= 128 ? 128 : 32 * DenseVec<T>::kElems;
+    if constexpr (kMaxTile >= 128) {
+        if (n % 128 == 0)
+            return launch<T, 128>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
+    }
     if (n % 64 == 0) return launch<T, 64>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
     return launch<T, 32>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
 }
@@ -239,5 +271,7 @@ template hipError_t spmm_launch<float>(int, int, int, const int*, const int*, co
                                        const float*, const float*, float*, hipStream_t, hipStream_t);
 template hipError_t spmm_launch<__half>(int, int, int, const int*, const int*, const int*, const int*, const int*,
                                         const float*, const __half*, float*, hipStream_t, hipStream_t);
+template hipError_t spmm_launch<double>(int, int, int, const int*, const int*, const int*, const int*, const int*,
+                                        const double*, const double*, double*, hipStream_t, hipStream_t);
 
 } // namespace rode

@@ -132,7 +132,8 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
                  dense_matrix, out=None):
     """C = A_csr @ dense_matrix through ``rode_hip_spmm_f32`` / ``_f16``
     (host API ``RoDe_SpMM/RoDeSpmm.h:4-8``).  ``dense_matrix`` is (k, n) with n a
-    multiple of 32; the result is a new zero-initialised (m, n) fp32 tensor, or
+    multiple of 32, fp32 / fp16 (fp32 ``values``) or fp64 (fp64 ``values``); the
+    result is a new zero-initialised (m, n) tensor of the dtype of ``values``, or
     ``out`` accumulated in place the way the reference kernels do (long rows add,
     short rows overwrite)."""
     for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
@@ -142,20 +143,26 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
                     (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices")):
         _check(t.dtype == torch.int32, f"{name} must be int32")
-    _check(values.dtype == torch.float32, "values must be float32")
-    _check(dense_matrix.dtype in (torch.float32, torch.float16), "dense_matrix must be float32 or float16")
+    if dense_matrix.dtype == torch.float64:
+        _check(values.dtype == torch.float64, "values must be float64 when dense_matrix is float64")
+    else:
+        _check(values.dtype == torch.float32, "values must be float32")
+        _check(dense_matrix.dtype in (torch.float32, torch.float16),
+               "dense_matrix must be float32, float16 or float64")
+    out_dtype = values.dtype
     _check(dense_matrix.dim() == 2 and dense_matrix.size(0) == k, "dense_matrix rows must equal k")
     n = dense_matrix.size(1)
     _check(n > 0 and n % 32 == 0, "dense_matrix cols must be a positive multiple of 32")
     if out is None:
-        out = torch.zeros((m, n), dtype=torch.float32, device=values.device)
+        out = torch.zeros((m, n), dtype=out_dtype, device=values.device)
     else:
         _check_input(out, "out")
-        _check(out.dtype == torch.float32 and tuple(out.shape) == (m, n), "out must be float32 of shape (m, n)")
+        _check(out.dtype == out_dtype and tuple(out.shape) == (m, n), f"out must be {out_dtype} of shape (m, n)")
     if m1 == 0 and m2 == 0:
         return out
     lib = _lib.load()
-    fn = lib.rode_hip_spmm_f32 if dense_matrix.dtype == torch.float32 else lib.rode_hip_spmm_f16
+    fn = {torch.float32: lib.rode_hip_spmm_f32, torch.float16: lib.rode_hip_spmm_f16,
+          torch.float64: lib.rode_hip_spmm_f64}[dense_matrix.dtype]
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
         code = fn(m1, m2, k, n, values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),

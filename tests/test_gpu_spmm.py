@@ -64,6 +64,62 @@ def test_fp16_dense(n):
         _check(make_csr(rp, col, val, m, k, 32, seg), rp, col, val, B, half=True)
 
 
+@pytest.mark.parametrize("n", [32, 64, 128, 96])
+def test_fp64(n):
+    """The double overloads (RoDeSpmm.h:10-14): fp64 values, B and C; bound 1e-12 of the row's L1 norm."""
+    import oracle
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(n)
+    m, k = 1100, 900
+    rp, col, val = random_csr(rng, m, k, 41, long_rows=5, long_len=850, empty_frac=0.1)
+    val64 = rng.uniform(-1, 1, len(val))
+    B = rng.standard_normal((k, n))
+    for seg in (32, 512):
+        csr = make_csr(rp, col, val, m, k, 32, seg)
+        C = rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                        csr.row_offsets, csr.column_indices, torch.from_numpy(val64).to(DEV), m, k,
+                                        torch.from_numpy(B).to(DEV)).cpu().numpy()
+        assert C.dtype == np.float64
+        ref = oracle.spmm_d(rp, col, val64, B)
+        l1 = np.abs(ref).sum(axis=1)
+        assert (np.abs(C - ref).max(axis=1) <= 1e-12 * np.maximum(l1, 1e-300) + 1e-300).all()
+        assert not C[np.diff(rp) == 0].any()
+    with pytest.raises(RuntimeError, match="float64"):
+        rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                    csr.row_offsets, csr.column_indices, csr.values, m, k, torch.from_numpy(B).to(DEV))
+
+
+def test_fp64_cxx_overloads():
+    """RoDeSpmm_n32(double) / RoDeSpmm_n128(double) through their mangled names."""
+    import oracle
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import _lib
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    rng = np.random.default_rng(21)
+    m, k = 700, 640
+    rp, col, val = random_csr(rng, m, k, 45, long_rows=3, long_len=600)
+    val64 = rng.uniform(-1, 1, len(val))
+    csr = make_csr(rp, col, val, m, k, 32, 512)
+    dv = torch.from_numpy(val64).to(DEV)
+    for mangled, width in [("_Z12RoDeSpmm_n32iiiiPKdPKiS2_S2_S2_S2_S0_PdP12ihipStream_tS5_", 32),
+                           ("_Z13RoDeSpmm_n128iiiiPKdPKiS2_S2_S2_S2_S0_PdP12ihipStream_tS5_", 64)]:
+        fn = getattr(lib, mangled)
+        fn.restype = None
+        fn.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 10
+        B = rng.standard_normal((k, width))
+        dB = torch.from_numpy(B).to(DEV)
+        C = torch.zeros(m, width, dtype=torch.float64, device=DEV)
+        torch.cuda.synchronize()
+        fn(csr.m1, csr.m2, k, width, dv.data_ptr(), csr.column_indices.data_ptr(), csr.row_offsets.data_ptr(),
+           csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(), dB.data_ptr(),
+           C.data_ptr(), None, None)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(C.cpu().numpy(), oracle.spmm_d(rp, col, val64, B), rtol=1e-11, atol=1e-11)
+
+
 def test_special_cases_and_edges():
     from gpu_common import DEV, make_csr, run_spmm
     from helpers import random_csr

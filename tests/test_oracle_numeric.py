@@ -96,3 +96,14 @@ def test_spmm_special_cases():
     perm = rng.permutation(k).astype(np.int32)
     got = oracle.spmm_f32(np.arange(k + 1, dtype=np.int32), perm, np.ones(k, np.float32), B)
     np.testing.assert_array_equal(got, B[perm])
+
+
+def test_spmm_double_against_scipy():
+    import scipy.sparse as sp
+    rng = np.random.default_rng(3)
+    m, k, n = 200, 150, 64
+    rp, col, val = random_csr(rng, m, k, 20, long_rows=2, long_len=140)
+    val64 = rng.uniform(-1, 1, len(val))
+    B = rng.standard_normal((k, n))
+    ref = sp.csr_matrix((val64, col, rp), shape=(m, k)) @ B
+    np.testing.assert_allclose(oracle.spmm_d(rp, col, val64, B), ref, rtol=1e-13, atol=1e-13)
