@@ -108,6 +108,20 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
                        const int* d_column_indices, const float* d_values, const void* d_lhs_half,
                        const void* d_rhs_half, float* d_out, void* stream1, void* stream2);
 
+/*
+ * Row softmax over the values of a CSR pattern, out[idx] = softmax over the row of
+ * scale * in[idx]; rows without nonzeros are skipped; out may alias in.  No
+ * counterpart in the reference: it is the step between its SDDMM and SpMM when
+ * the two are chained as sparse attention (the reference op is forward-only SDDMM,
+ * RoDe_SDDMM/rode_sddmm.py:194-248).
+ */
+int rode_hip_csr_softmax_f32(int M, const int* d_row_offsets, const float* d_in, float* d_out, float scale,
+                             void* stream);
+
+/* Its gradient: ds[idx] = scale * p[idx] * (dp[idx] - sum over the row of dp * p); ds may alias dp. */
+int rode_hip_csr_softmax_backward_f32(int M, const int* d_row_offsets, const float* d_p, const float* d_dp,
+                                      float* d_ds, float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,8 @@ SIGNATURES = {
     "rode_hip_spmm_f64": (c_int, [c_int] * 4 + [c_void_p] * 10),
     "rode_hip_sddmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 11),
     "rode_hip_sddmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 11),
+    "rode_hip_csr_softmax_f32": (c_int, [c_int, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p]),
+    "rode_hip_csr_softmax_backward_f32": (c_int, [c_int] + [c_void_p] * 4 + [ctypes.c_float, c_void_p]),
 }
 
 _lib = None

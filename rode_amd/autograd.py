@@ -1,0 +1,128 @@
+"""Gradients of SDDMM and SpMM, CSR row softmax, and the sparse-attention chain
+SDDMM -> softmax -> SpMM on one decomposed pattern.
+
+The reference's op is forward-only (``RoDe_SDDMM/rode_sddmm.py:194-248``).  Every
+gradient is again one of the two kernels on the same pattern or on its transpose:
+
+    out = v (.) (L R^T)|pattern :  dL = (g (.) v) R          (SpMM, same pattern)
+                                   dR = (g (.) v)^T L        (SpMM, transposed pattern)
+                                   dv = g (.) (L R^T)|pattern (SDDMM)
+    C   = A B                   :  dB = A^T dC               (SpMM, transposed pattern)
+                                   dv = (dC B^T)|pattern      (SDDMM with unit values)
+"""
+import torch
+
+from . import _lib, rode_sddmm_hip
+
+
+def _sddmm(csr, values, lhs, rhs):
+    return rode_sddmm_hip.sddmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                        csr.row_offsets, csr.column_indices, values.contiguous(), csr.m, csr.n,
+                                        lhs.contiguous(), rhs.contiguous(), lhs.shape[1])
+
+
+def _spmm(csr, values, dense):
+    return rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                       csr.row_offsets, csr.column_indices, values.contiguous(), csr.m, csr.n,
+                                       dense.contiguous())
+
+
+class SddmmFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, csr, values, lhs, rhs):
+        ctx.csr = csr
+        ctx.save_for_backward(values, lhs, rhs)
+        return _sddmm(csr, values.detach().float(), lhs.detach(), rhs.detach())
+
+    @staticmethod
+    def backward(ctx, g):
+        csr = ctx.csr
+        values, lhs, rhs = ctx.saved_tensors
+        g = g.contiguous().float()
+        gv = g * values.float()
+        d_values = d_lhs = d_rhs = None
+        if ctx.needs_input_grad[2]:
+            d_lhs = _spmm(csr, gv, rhs.float()).to(lhs.dtype)
+        if ctx.needs_input_grad[3]:
+            csr_t, perm = csr.transpose()
+            d_rhs = _spmm(csr_t, gv[perm], lhs.float()).to(rhs.dtype)
+        if ctx.needs_input_grad[1]:
+            d_values = _sddmm(csr, g, lhs, rhs).to(values.dtype)
+        return None, d_values, d_lhs, d_rhs
+
+
+class SpmmFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, csr, values, dense):
+        ctx.csr = csr
+        ctx.save_for_backward(values, dense)
+        return _spmm(csr, values.detach().float(), dense.detach())
+
+    @staticmethod
+    def backward(ctx, g):
+        csr = ctx.csr
+        values, dense = ctx.saved_tensors
+        g = g.contiguous().float()
+        d_values = d_dense = None
+        if ctx.needs_input_grad[2]:
+            csr_t, perm = csr.transpose()
+            d_dense = _spmm(csr_t, values.float()[perm], g).to(dense.dtype)
+        if ctx.needs_input_grad[1]:
+            if g.shape[1] not in (32, 64, 128):
+                raise NotImplementedError("gradient with respect to the sparse values needs a dense width of 32, 64 or 128")
+            d_values = _sddmm(csr, torch.ones_like(values, dtype=torch.float32), g, dense.float()).to(values.dtype)
+        return None, d_values, d_dense
+
+
+def _softmax_call(fn_name, row_offsets, a, b, scale):
+    lib = _lib.load()
+    out = torch.empty_like(a)
+    m = row_offsets.numel() - 1
+    with torch.cuda.device(a.device):
+        s = torch.cuda.current_stream(a.device).cuda_stream
+        if b is None:
+            code = lib.rode_hip_csr_softmax_f32(m, row_offsets.data_ptr(), a.data_ptr(), out.data_ptr(), scale, s)
+        else:
+            code = lib.rode_hip_csr_softmax_backward_f32(m, row_offsets.data_ptr(), a.data_ptr(), b.data_ptr(),
+                                                         out.data_ptr(), scale, s)
+    _lib.check(code, fn_name)
+    return out
+
+
+class CsrSoftmaxFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, csr, scores, scale):
+        p = _softmax_call("rode_hip_csr_softmax_f32", csr.row_offsets, scores.detach().contiguous().float(), None,
+                          float(scale))
+        ctx.csr, ctx.scale = csr, float(scale)
+        ctx.save_for_backward(p)
+        return p
+
+    @staticmethod
+    def backward(ctx, g):
+        (p,) = ctx.saved_tensors
+        ds = _softmax_call("rode_hip_csr_softmax_backward_f32", ctx.csr.row_offsets, p, g.contiguous().float(),
+                           ctx.scale)
+        return None, ds, None
+
+
+def csr_row_softmax(sparse_matrix, scores, scale=1.0):
+    """softmax(scale * scores) over every row of the pattern; (nnz,) float32."""
+    if scores.shape != sparse_matrix.values.shape:
+        raise ValueError(f"scores shape must be {tuple(sparse_matrix.values.shape)}, got {tuple(scores.shape)}")
+    assert scores.is_cuda and scores.device == sparse_matrix.device, f"scores must be on {sparse_matrix.device}"
+    return CsrSoftmaxFunction.apply(sparse_matrix, scores, scale)
+
+
+def sparse_attention(mask, q, k, v, scale=None):
+    """softmax(scale * mask (.) (q k^T)) v on the sparsity pattern of ``mask`` (a
+    ``RoDeCSR``; its values multiply the scores, use 1 for a pure mask).  q is (m, d),
+    k is (n, d) with d in {32, 64, 128}; v is (n, dv) with dv a multiple of 32.  One
+    row decomposition serves all three kernels; differentiable in q, k and v."""
+    from .rode_sddmm import rode_sddmm
+    from .rode_spmm import rode_spmm
+    if scale is None:
+        scale = q.shape[1] ** -0.5
+    scores = rode_sddmm(mask, q, k)
+    probs = csr_row_softmax(mask, scores, scale)
+    return rode_spmm(mask, v, values=probs)

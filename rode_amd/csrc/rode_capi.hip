@@ -104,6 +104,20 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
                                       d_out, as_stream(stream1), as_stream(stream2));
 }
 
+int rode_hip_csr_softmax_f32(int M, const int* d_row_offsets, const float* d_in, float* d_out, float scale,
+                             void* stream)
+{
+    if (M < 0 || !d_row_offsets || (M > 0 && (!d_in || !d_out))) return hipErrorInvalidValue;
+    return rode::csr_softmax_launch(M, d_row_offsets, d_in, d_out, scale, as_stream(stream));
+}
+
+int rode_hip_csr_softmax_backward_f32(int M, const int* d_row_offsets, const float* d_p, const float* d_dp,
+                                      float* d_ds, float scale, void* stream)
+{
+    if (M < 0 || !d_row_offsets || (M > 0 && (!d_p || !d_dp || !d_ds))) return hipErrorInvalidValue;
+    return rode::csr_softmax_backward_launch(M, d_row_offsets, d_p, d_dp, d_ds, scale, as_stream(stream));
+}
+
 } // extern "C"
 
 // ---- reference-signature C++ entry points ----------------------------------

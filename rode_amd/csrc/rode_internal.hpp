@@ -27,4 +27,9 @@ hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int*
                         const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs,
                         float* out, hipStream_t s1, hipStream_t s2);
 
+hipError_t csr_softmax_launch(int M, const int* row_ptr, const float* in, float* out, float scale,
+                              hipStream_t stream);
+hipError_t csr_softmax_backward_launch(int M, const int* row_ptr, const float* p, const float* dp, float* ds,
+                                       float scale, hipStream_t stream);
+
 } // namespace rode

@@ -59,6 +59,37 @@ class RoDeCSR:
         self.m1 = m1
         self.m2 = m2
 
+    def with_values(self, values):
+        """The same pattern and decomposition with other values (no preprocessing is
+        repeated): how the output of one op becomes the sparse operand of the next,
+        e.g. SDDMM scores -> softmax -> SpMM."""
+        if values.shape != self.values.shape:
+            raise ValueError(f"values shape must be {tuple(self.values.shape)}, got {tuple(values.shape)}")
+        other = object.__new__(RoDeCSR)
+        other.__dict__.update(self.__dict__)
+        other.values = values if values.dtype == torch.float64 else values.to(torch.float32)
+        other.values = other.values.to(self.device).contiguous()
+        return other
+
+    def transpose(self):
+        """``(csr_t, perm)``: the decomposed pattern of the transposed matrix and the
+        permutation with ``csr_t.values == self.values[perm]`` (built on the GPU once,
+        then cached).  Needed by the gradients with respect to the column-side operands."""
+        cached = self.__dict__.get("_transpose")
+        if cached is None:
+            lens = (self.row_offsets[1:] - self.row_offsets[:-1]).to(torch.int64)
+            rows = torch.repeat_interleave(torch.arange(self.m, device=self.device), lens)
+            cols = self.column_indices.to(torch.int64)
+            _, perm = torch.sort(cols, stable=True)  # rows stay ascending inside a column
+            row_offsets_t = torch.zeros(self.n + 1, dtype=torch.int64, device=self.device)
+            row_offsets_t[1:] = torch.cumsum(torch.bincount(cols, minlength=self.n), 0)
+            csr_t = RoDeCSR(row_offsets_t.to(torch.int32), rows[perm].to(torch.int32), self.values.float()[perm],
+                            self.device, self.n, self.m, self.k, config=self.config)
+            cached = (csr_t, perm)
+            self.__dict__["_transpose"] = cached
+        csr_t, perm = cached
+        return csr_t.with_values(self.values[perm]), perm
+
     @classmethod
     def from_random(cls, m, n, nnz_per_row, device, k=128):
         """Random pattern with about ``nnz_per_row`` entries per row (duplicates
@@ -93,10 +124,12 @@ class RoDeCSR:
                 f"m1={self.m1}, m2={self.m2}, device={self.device})")
 
 
-def rode_sddmm(sparse_matrix, lhs, rhs):
+def rode_sddmm(sparse_matrix, lhs, rhs, values=None):
     """out = S (.) (lhs @ rhs^T) sampled at the nonzeros of S; returns the (nnz,)
     values in CSR order.  lhs is (m, k), rhs is (n, k); float32, or float16 with
-    fp32 accumulation."""
+    fp32 accumulation.  ``values`` (optional) replaces the values of S for this call.
+    Differentiable with respect to lhs, rhs and values (the reference op is
+    forward-only)."""
     m, n, k = sparse_matrix.m, sparse_matrix.n, sparse_matrix.k
     if tuple(lhs.shape) != (m, k):
         raise ValueError(f"lhs_matrix shape must be ({m}, {k}), got {tuple(lhs.shape)}")
@@ -106,6 +139,12 @@ def rode_sddmm(sparse_matrix, lhs, rhs):
     assert rhs.is_cuda and rhs.device == sparse_matrix.device, f"rhs must be on {sparse_matrix.device}, got {rhs.device}"
     assert lhs.dtype in (torch.float32, torch.float16), f"lhs must be float32 or float16, got {lhs.dtype}"
     assert rhs.dtype == lhs.dtype, f"rhs must be {lhs.dtype}, got {rhs.dtype}"
+    vals = sparse_matrix.values if values is None else values
+    if torch.is_grad_enabled() and (lhs.requires_grad or rhs.requires_grad or vals.requires_grad):
+        from .autograd import SddmmFunction
+        return SddmmFunction.apply(sparse_matrix, vals, lhs, rhs)
+    if values is not None:
+        sparse_matrix = sparse_matrix.with_values(values)
     return rode_sddmm_hip.sddmm_forward(
         sparse_matrix.block_indices, sparse_matrix.residue_indices, sparse_matrix.st_offsets,
         sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,

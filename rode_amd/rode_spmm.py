@@ -5,9 +5,11 @@ import torch
 from . import rode_sddmm_hip
 
 
-def rode_spmm(sparse_matrix, dense, out=None):
+def rode_spmm(sparse_matrix, dense, out=None, values=None):
     """C = S @ dense.  ``dense`` is (n, width) float32 or float16 with ``width`` a
-    multiple of 32; returns an (m, width) float32 tensor."""
+    multiple of 32; returns an (m, width) float32 tensor.  ``values`` (optional)
+    replaces the values of S for this call.  Differentiable with respect to dense
+    and values when ``out`` is not given."""
     if dense.dim() != 2 or dense.shape[0] != sparse_matrix.n:
         raise ValueError(f"dense shape must be ({sparse_matrix.n}, width), got {tuple(dense.shape)}")
     if dense.shape[1] % 32 != 0:
@@ -17,6 +19,12 @@ def rode_spmm(sparse_matrix, dense, out=None):
     assert dense.dtype in (torch.float32, torch.float16), f"dense must be float32 or float16, got {dense.dtype}"
     seg = sparse_matrix.config
     assert seg["k_block"] == 32 and seg["vec_len"] == 4, "the kernels need k_block=32, vec_len=4"
+    vals = sparse_matrix.values if values is None else values
+    if out is None and torch.is_grad_enabled() and (dense.requires_grad or vals.requires_grad):
+        from .autograd import SpmmFunction
+        return SpmmFunction.apply(sparse_matrix, vals, dense)
+    if values is not None:
+        sparse_matrix = sparse_matrix.with_values(values)
     return rode_sddmm_hip.spmm_forward(
         sparse_matrix.block_indices, sparse_matrix.residue_indices, sparse_matrix.st_offsets,
         sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,

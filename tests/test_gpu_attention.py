@@ -1,0 +1,154 @@
+"""The chain around the op that benchmark configuration 5 describes: SDDMM scores ->
+(row softmax) -> SpMM on one decomposed pattern, plus gradients.  None of this exists
+in the reference (forward-only SDDMM), so the oracles are the CPU oracle for the two
+products and dense fp64 PyTorch (autograd) for softmax and gradients."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _dense(rp, col, val, m, n, dtype=torch.float64):
+    from gpu_common import DEV
+    from helpers import row_of_index
+    A = torch.zeros(m, n, dtype=dtype, device=DEV)
+    A[torch.from_numpy(row_of_index(rp)).to(DEV), torch.from_numpy(col.astype(np.int64)).to(DEV)] = \
+        torch.from_numpy(val).to(DEV, dtype)
+    return A
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_sddmm_then_spmm_pipeline(half):
+    """S = mask (.) (Q K^T), O = S V with the decomposition computed once
+    (configuration 5 at 1/4 size; fp16 operands accumulate in fp32)."""
+    import oracle
+    from gpu_common import DEV, TOL_F16, TOL_F32, make_csr, round_half
+    from helpers import spmm_row_l1_error
+    from rode_amd import rode_sddmm, rode_spmm, workloads
+    m, n, rp, col, val = workloads.config("c5_attention", 1 / 4)
+    d = 64
+    rng = np.random.default_rng(5)
+    q, k, v = (rng.standard_normal((m, d)).astype(np.float32) for _ in range(3))
+    dt = torch.float16 if half else torch.float32
+    mask = make_csr(rp, col, val, m, n, d)
+    scores = rode_sddmm(mask, torch.from_numpy(q).to(DEV, dt), torch.from_numpy(k).to(DEV, dt))
+    out = rode_spmm(mask.with_values(scores), torch.from_numpy(v).to(DEV, dt)).cpu().numpy()
+    assert mask.with_values(scores).block_indices.data_ptr() == mask.block_indices.data_ptr()
+    if half:
+        q, k, v = round_half(q), round_half(k), round_half(v)
+    s64 = oracle.sddmm_f64(rp, col, val, q, k)
+    # the second product starts from the fp32 scores the first one delivered
+    ref = oracle.spmm_f64(rp, col, scores.cpu().numpy(), v)
+    assert spmm_row_l1_error(out, ref) <= (TOL_F16 if half else TOL_F32)
+    # end to end against fp64 all the way: errors of both stages, still inside the bound
+    ref_all = oracle.spmm_d(rp, col, s64, v.astype(np.float64))
+    assert spmm_row_l1_error(out, ref_all) <= (TOL_F16 if half else TOL_F32)
+
+
+def test_transpose():
+    from gpu_common import make_csr
+    from helpers import random_csr
+    rng = np.random.default_rng(1)
+    m, n = 300, 411
+    rp, col, val = random_csr(rng, m, n, 30, long_rows=2, long_len=400)
+    csr = make_csr(rp, col, val, m, n, 32)
+    csr_t, perm = csr.transpose()
+    assert (csr_t.m, csr_t.n, csr_t.nnz) == (n, m, csr.nnz)
+    A = _dense(rp, col, val, m, n)
+    At = _dense(csr_t.row_offsets.cpu().numpy(), csr_t.column_indices.cpu().numpy(), csr_t.values.cpu().numpy(), n, m)
+    assert torch.equal(At, A.t())
+    assert torch.equal(csr_t.values, csr.values[perm])
+    again, _ = csr.transpose()
+    assert again.block_indices.data_ptr() == csr_t.block_indices.data_ptr()  # cached
+
+
+def test_row_softmax_forward_backward():
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import csr_row_softmax
+    rng = np.random.default_rng(2)
+    m, n = 500, 3000
+    rp, col, val = random_csr(rng, m, n, 60, long_rows=3, long_len=2500, empty_frac=0.1)
+    csr = make_csr(rp, col, val, m, n, 32)
+    s = torch.from_numpy(rng.standard_normal(len(val)).astype(np.float32) * 4).to(DEV).requires_grad_()
+    w = torch.from_numpy(rng.standard_normal(len(val)).astype(np.float32)).to(DEV)
+    p = csr_row_softmax(csr, s, 0.7)
+    (p * w).sum().backward()
+    # dense fp64 reference with -inf outside the pattern
+    rows = torch.from_numpy(np.repeat(np.arange(m), np.diff(rp))).to(DEV)
+    cols = torch.from_numpy(col.astype(np.int64)).to(DEV)
+    sd = s.detach().double().requires_grad_()
+    dense = torch.full((m, n), float("-inf"), dtype=torch.float64, device=DEV).index_put((rows, cols), 0.7 * sd)
+    nonempty = torch.from_numpy(np.diff(rp) > 0).to(DEV)
+    pd = torch.softmax(dense[nonempty], dim=1)
+    full = torch.zeros(m, n, dtype=torch.float64, device=DEV).index_put((torch.nonzero(nonempty)[:, 0],), pd)
+    pref = full[rows, cols]
+    (pref * w.double()).sum().backward()
+    assert (p.detach().double() - pref.detach()).abs().max().item() < 1e-6
+    sums = torch.zeros(m, dtype=torch.float64, device=DEV).index_add(0, rows, p.detach().double())
+    assert (sums[nonempty] - 1).abs().max().item() < 1e-5
+    assert (s.grad.double() - sd.grad).abs().max().item() < 1e-5
+
+
+@pytest.mark.parametrize("k", [32, 64, 128])
+def test_sddmm_and_spmm_gradients(k):
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import rode_sddmm, rode_spmm
+    rng = np.random.default_rng(k)
+    m, n = 260, 333
+    rp, col, val = random_csr(rng, m, n, 25, long_rows=2, long_len=300)
+    csr = make_csr(rp, col, val, m, n, k)
+    rows = torch.from_numpy(np.repeat(np.arange(m), np.diff(rp))).to(DEV)
+    cols = torch.from_numpy(col.astype(np.int64)).to(DEV)
+    mk = lambda *shape: torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to(DEV)
+    lhs, rhs, w = mk(m, k).requires_grad_(), mk(n, k).requires_grad_(), mk(len(val))
+    vals = csr.values.clone().requires_grad_()
+    out = rode_sddmm(csr, lhs, rhs, values=vals)
+    (out * w).sum().backward()
+    l64, r64, v64 = (t.detach().double().requires_grad_() for t in (lhs, rhs, vals))
+    ref = v64 * (l64 @ r64.t())[rows, cols]
+    (ref * w.double()).sum().backward()
+    for got, want in ((out, ref), (lhs.grad, l64.grad), (rhs.grad, r64.grad), (vals.grad, v64.grad)):
+        scale = want.abs().max().item() + 1e-12
+        assert (got.detach().double() - want.detach()).abs().max().item() <= 2e-5 * scale
+    # SpMM: C = A B
+    dense, wc = mk(n, k).requires_grad_(), mk(m, k)
+    vals2 = csr.values.clone().requires_grad_()
+    C = rode_spmm(csr, dense, values=vals2)
+    (C * wc).sum().backward()
+    d64, v64 = dense.detach().double().requires_grad_(), vals2.detach().double().requires_grad_()
+    A = torch.zeros(m, n, dtype=torch.float64, device=DEV).index_put((rows, cols), v64)
+    Cref = A @ d64
+    (Cref * wc.double()).sum().backward()
+    for got, want in ((C, Cref), (dense.grad, d64.grad), (vals2.grad, v64.grad)):
+        scale = want.abs().max().item() + 1e-12
+        assert (got.detach().double() - want.detach()).abs().max().item() <= 2e-5 * scale
+    # without requires_grad the plain path is taken and nothing is recorded
+    assert not rode_sddmm(csr, lhs.detach(), rhs.detach()).requires_grad
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_sparse_attention_against_dense(half):
+    from gpu_common import DEV, make_csr
+    from rode_amd import sparse_attention, workloads
+    m, n, rp, col, val = workloads.config("c5_attention", 1 / 16)
+    d = 64
+    rng = np.random.default_rng(8)
+    dt = torch.float16 if half else torch.float32
+    mk = lambda r: torch.from_numpy(rng.standard_normal((r, d)).astype(np.float32)).to(DEV, dt)
+    q, k, v = mk(m).requires_grad_(), mk(n).requires_grad_(), mk(n).requires_grad_()
+    w = torch.from_numpy(rng.standard_normal((m, d)).astype(np.float32)).to(DEV)
+    mask = make_csr(rp, col, val, m, n, d)
+    out = sparse_attention(mask, q, k, v)
+    (out * w).sum().backward()
+    q64, k64, v64 = (t.detach().double().requires_grad_() for t in (q, k, v))
+    allowed = _dense(rp, col, val, m, n) != 0
+    scores = (q64 @ k64.t()) * d ** -0.5
+    ref = torch.softmax(scores.masked_fill(~allowed, float("-inf")), dim=1) @ v64
+    (ref * w.double()).sum().backward()
+    tol = 3e-3 if half else 2e-5
+    for got, want in ((out, ref), (q.grad, q64.grad), (k.grad, k64.grad), (v.grad, v64.grad)):
+        scale = want.abs().max().item()
+        assert (got.detach().double() - want.detach()).abs().max().item() <= tol * scale
