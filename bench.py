@@ -40,6 +40,8 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--two-streams", action="store_true",
                    help="residue kernels on a second stream (forked from / joined to the first with events)")
+    p.add_argument("--chain", action="store_true",
+                   help="step = SDDMM scores -> row softmax -> clear C -> SpMM with those values (sparse attention)")
     p.add_argument("--calibrate", action="store_true",
                    help="also run one plain device copy of 256 MiB (a known size to scale profiler counters by)")
     return p.parse_args()
@@ -139,7 +141,21 @@ def main():
                    "sddmm")
         join()
 
+    probs = torch.empty(nnz, device=dev) if args.chain else None
+
+    def spmm_chain():
+        _lib.check(spmm_fn(csr.m1, csr.m2, n, k, probs.data_ptr(), csr.column_indices.data_ptr(),
+                           csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
+                           csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, stream), "spmm")
+
     def step():
+        if args.chain:
+            sddmm(csr.m1, csr.m2)
+            _lib.check(lib.rode_hip_csr_softmax_f32(m, csr.row_offsets.data_ptr(), out.data_ptr(), probs.data_ptr(),
+                                                    float(k) ** -0.5, stream), "softmax")
+            C.zero_()
+            spmm_chain()
+            return
         C.zero_()
         spmm(csr.m1, csr.m2)
         sddmm(csr.m1, csr.m2)
@@ -273,7 +289,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32" if elem == 4 else "f16->f32",
         "data": "synthetic",
         "config": {"workload": f"{args.workload} ({workloads.CONFIGS[args.workload][5]}), K={k}, "
-                               f"step = clear C + SpMM + SDDMM",
+                               + ("step = SDDMM -> row softmax -> clear C -> SpMM (chained)" if args.chain
+                                  else "step = clear C + SpMM + SDDMM"),
                    "rows": m, "cols": n, "nnz": nnz, "K": k, "seg_length": csr.config["seg_length"],
                    "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale},
         "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C"},
