@@ -1,0 +1,80 @@
+"""Matrix Market ingest and row padding (host side, no GPU)."""
+import gzip
+
+import numpy as np
+import pytest
+import scipy.io
+import scipy.sparse as sp
+
+from rode_amd import io as rio
+
+
+def _same(csr, ref):
+    m, n, rp, col, val = csr
+    ref = sp.csr_matrix(ref)
+    ref.sum_duplicates()
+    ref.sort_indices()
+    assert (m, n) == ref.shape
+    np.testing.assert_array_equal(rp, ref.indptr)
+    np.testing.assert_array_equal(col, ref.indices)
+    np.testing.assert_allclose(val, ref.data.astype(np.float32), rtol=1e-6)
+
+
+@pytest.mark.parametrize("symmetry", ["general", "symmetric", "skew-symmetric"])
+def test_reads_what_scipy_reads(tmp_path, symmetry):
+    rng = np.random.default_rng(0)
+    A = sp.random(60, 60, density=0.08, random_state=1, format="coo")
+    if symmetry == "symmetric":
+        A = sp.coo_matrix(sp.tril(A) + sp.tril(A, -1).T)
+    elif symmetry == "skew-symmetric":
+        A = sp.coo_matrix(sp.tril(A, -1) - sp.tril(A, -1).T)
+    path = tmp_path / "a.mtx"
+    scipy.io.mmwrite(str(path), A, symmetry=symmetry if symmetry != "general" else "general")
+    _same(rio.read_matrix_market(path), scipy.io.mmread(str(path)))
+
+
+def test_pattern_rectangular_duplicates_and_gzip(tmp_path):
+    text = "%%MatrixMarket matrix coordinate pattern general\n% comment\n\n3 5 5\n1 1\n3 5\n3 2\n1 1\n2 4\n"
+    path = tmp_path / "p.mtx.gz"
+    with gzip.open(path, "wt") as f:
+        f.write(text)
+    m, n, rp, col, val = rio.read_matrix_market(path)
+    assert (m, n) == (3, 5) and rp.tolist() == [0, 1, 2, 4] and col.tolist() == [0, 3, 1, 4]
+    assert val.tolist() == [2.0, 1.0, 1.0, 1.0]  # the duplicate (1,1) is summed
+    empty = tmp_path / "e.mtx"
+    empty.write_text("%%MatrixMarket matrix coordinate real general\n4 4 0\n")
+    m, n, rp, col, val = rio.read_matrix_market(empty)
+    assert rp.tolist() == [0] * 5 and len(col) == 0
+
+
+def test_rejects_bad_files(tmp_path):
+    bad = tmp_path / "b.mtx"
+    bad.write_text("%%MatrixMarket matrix array real general\n2 2\n1\n2\n3\n4\n")
+    with pytest.raises(ValueError, match="coordinate"):
+        rio.read_matrix_market(bad)
+    bad.write_text("%%MatrixMarket matrix coordinate real general\n2 2 2\n1 1 1.0\n")
+    with pytest.raises(ValueError, match="promises"):
+        rio.read_matrix_market(bad)
+    bad.write_text("%%MatrixMarket matrix coordinate real general\n2 2 1\n3 1 1.0\n")
+    with pytest.raises(ValueError, match="out of range"):
+        rio.read_matrix_market(bad)
+    bad.write_text("hello\n")
+    with pytest.raises(ValueError, match="not a Matrix Market"):
+        rio.read_matrix_market(bad)
+
+
+def test_pad_rows_matches_the_reference_generators():
+    """The reference generators emit exactly `pad_rows(unpadded)`: drop their explicit
+    zeros, pad again, get the same arrays back."""
+    from rode_amd import workloads
+    rp, col, val = workloads.reference_csr(97, 103, 15, poisson=True, pad_to=4, seed=42)
+    assert (rp % 4 == 0).all()
+    raw_rp, raw_col, raw_val = workloads.reference_csr(97, 103, 15, poisson=True, pad_to=1, seed=42)
+    prp, pcol, pval = rio.pad_rows(raw_rp, raw_col, raw_val, 4)
+    np.testing.assert_array_equal(prp, rp)
+    np.testing.assert_array_equal(pcol, col)
+    np.testing.assert_array_equal(pval, val)
+    # empty rows stay empty; already aligned rows are untouched
+    prp, pcol, pval = rio.pad_rows([0, 0, 4, 5], [1, 2, 3, 4, 9], np.arange(5, dtype=np.float32) + 1)
+    assert prp.tolist() == [0, 0, 4, 8] and pcol.tolist() == [1, 2, 3, 4, 9, 9, 9, 9]
+    assert pval.tolist() == [1, 2, 3, 4, 5, 0, 0, 0]
