@@ -63,8 +63,9 @@ int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const i
  * segments, the residue kernel on stream2 over m2 rows.  As in the reference
  * C must be zero on entry: segments and tails of long rows are added with
  * atomics, short rows are stored, rows without nonzeros are not touched.
- * n must be a multiple of 32 (the reference tiles are 32 / 64 wide and
- * unguarded); the decomposition must have been made with k_block 32, vec_len 4.
+ * n: any positive multiple of 4 (the reference needs a multiple of its 32- or
+ * 64-wide tile and does not guard the edge); multiples of 32 take the unguarded
+ * fast path.  The decomposition must have been made with k_block 32, vec_len 4.
  */
 int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
                       const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
@@ -72,13 +73,14 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
                       void* stream2);
 
 /* fp64 values, B and C.  Replaces the double overloads of RoDeSpmm_n32 / RoDeSpmm_n128,
- * RoDe_SpMM/RoDeSpmm.h:10-14, RoDeSpmm.cu:521-529.  Same contract as rode_hip_spmm_f32. */
+ * RoDe_SpMM/RoDeSpmm.h:10-14, RoDeSpmm.cu:521-529.  Same contract as rode_hip_spmm_f32
+ * (n a multiple of 2). */
 int rode_hip_spmm_f64(int m1, int m2, int k, int n, const double* d_values, const int* d_column_indices,
                       const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
                       const int* d_row_seg_st_offsets, const double* d_B, double* d_C, void* stream1,
                       void* stream2);
 
-/* Same with B stored as IEEE fp16 (no reference entry point; operand semantics of the
+/* Same with B stored as IEEE fp16, n a multiple of 8 (no reference entry point; operand semantics of the
  * unused helper VectorCompute<half4>::FMA, RoDe_SpMM/common_utils.h:183-230:
  * widen to fp32, fp32 FMA). */
 int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
@@ -89,8 +91,8 @@ int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const
 /*
  * SDDMM  out[idx] = values[idx] * <lhs[row(idx),:], rhs[col(idx),:]>.
  * Replaces RoDeSDDMM_n32 / RoDeSDDMM_n128, RoDe_SDDMM/RoDeSddmm.h:4-9,
- * RoDeSddmm.cu:496-545.  k must be 32, 64 or 128 (the reference has 32 and
- * 128).  Segments may have any length that the decomposition produced, so one
+ * RoDeSddmm.cu:496-545.  k: any positive multiple of 4 up to 512 (the reference
+ * has 32 and 128); 32, 64 and 128 take the unguarded fast path.  Segments may have any length that the decomposition produced, so one
  * entry point serves both reference parameter sets (512,32,4) and (32,32,4).
  * Every out[idx], idx < nnz, is written exactly once; out needs no clearing.
  * A launch is skipped only when its count is zero (the reference also skips it
@@ -102,7 +104,7 @@ int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_bl
                        const int* d_column_indices, const float* d_values, const float* d_lhs_matrix,
                        const float* d_rhs_matrix, float* d_out, void* stream1, void* stream2);
 
-/* Same with lhs / rhs stored as IEEE fp16, fp32 accumulate (no reference entry point). */
+/* Same with lhs / rhs stored as IEEE fp16, fp32 accumulate, k a multiple of 8 (no reference entry point). */
 int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_block,
                        const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                        const int* d_column_indices, const float* d_values, const void* d_lhs_half,

@@ -24,25 +24,46 @@ namespace rode {
 
 namespace {
 
-template <typename T, int K>
+// KT = width of the lane tile (32, 64 or 128 elements): LPR = KT / VEC lanes read KT
+// consecutive elements of a dense row per load instruction.  A row of K elements is
+// covered by NS such slabs (KT * NS >= K); EDGE says that the last slab is partial, in
+// which case the lanes past K read nothing and contribute zero.
+template <typename T, int KT>
 struct SddmmShape {
     static constexpr int kVec = DenseVec<T>::kElems;
-    static constexpr int kLpr = K / kVec;      // lanes that cover one dense row
+    static constexpr int kLpr = KT / kVec;     // lanes that cover one slab of a dense row
     static constexpr int kQuads = kLpr / 4;    // slot quads per lane group per unit
-    static_assert(K % kVec == 0 && kLpr >= 4 && kLpr <= 32 && (kLpr & (kLpr - 1)) == 0,
-                  "unsupported K for this dense type");
+    static_assert(KT % kVec == 0 && kLpr >= 4 && kLpr <= 32 && (kLpr & (kLpr - 1)) == 0,
+                  "unsupported tile width for this dense type");
 };
 
-// Dot products of one 32-slot unit.  `my_col` is the column of this lane's
-// slot; `nslots` (half-uniform) is how many leading slots of the half need a
-// result.  Returns the dot product for this lane's slot (0 for slots that were
-// skipped).  FULL promises nslots == 32 and removes the per-quad tests.
-template <typename T, int K, bool FULL>
-__device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane, const float (&a)[SddmmShape<T, K>::kVec],
-                                            int my_col, int nslots, int* lds_cols, int lane)
+// <lhs row, rhs row> restricted to this lane's elements.
+template <typename T, int KT, int NS, bool EDGE>
+__device__ __forceinline__ float lane_dot(const float (&a)[NS][SddmmShape<T, KT>::kVec], const T* __restrict__ row_lane,
+                                          int k, int lane_elem)
 {
-    using S = SddmmShape<T, K>;
-    constexpr int VEC = S::kVec, LPR = S::kLpr;
+    constexpr int VEC = SddmmShape<T, KT>::kVec;
+    float d = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        if (!EDGE || lane_elem + s * KT < k) {
+            float b[VEC];
+            DenseVec<T>::load(row_lane + s * KT, b);
+#pragma unroll
+            for (int x = 0; x < VEC; ++x) d = fmaf(a[s][x], b[x], d);
+        }
+    }
+    return d;
+}
+
+// Dot products of one 32-slot unit of a block segment.  `my_col` is the column of this
+// lane's slot.  Returns the dot product for this lane's slot.
+template <typename T, int KT, int NS, bool EDGE>
+__device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane, const float (&a)[NS][SddmmShape<T, KT>::kVec],
+                                            int my_col, int k, int* lds_cols, int lane)
+{
+    using S = SddmmShape<T, KT>;
+    constexpr int LPR = S::kLpr;
 
     lds_cols[lane] = my_col;
     wave_lds_sync();
@@ -54,52 +75,50 @@ __device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane, cons
 
 #pragma unroll
     for (int q = 0; q < S::kQuads; ++q) {
-        if (FULL || group_first + 4 * q < nslots) {
-            const int4 c4 = *reinterpret_cast<const int4*>(group_cols + 4 * q);
-            const int c[4] = {c4.x, c4.y, c4.z, c4.w};
-            float p[4];
+        const int4 c4 = *reinterpret_cast<const int4*>(group_cols + 4 * q);
+        const int c[4] = {c4.x, c4.y, c4.z, c4.w};
+        float p[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float b[VEC];
-                DenseVec<T>::load(rhs_lane + (size_t)c[j] * K, b);
-                float d = 0.f;
-#pragma unroll
-                for (int x = 0; x < VEC; ++x) d = fmaf(a[x], b[x], d);
-                p[j] = d;
-            }
-            // transpose-reduce: afterwards lane (ls & 3) == j holds slot j of the quad
-            const bool hi2 = ls & 2, hi1 = ls & 1;
-            const float k0 = hi2 ? p[2] : p[0], s0 = hi2 ? p[0] : p[2];
-            const float k1 = hi2 ? p[3] : p[1], s1 = hi2 ? p[1] : p[3];
-            const float q0 = k0 + lane_xor2(s0);
-            const float q1 = k1 + lane_xor2(s1);
-            float r = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
-            r = butterfly_sum<4, LPR>(r);
-            if ((ls >> 2) == q) result = r;
-        }
+        for (int j = 0; j < 4; ++j)
+            p[j] = lane_dot<T, KT, NS, EDGE>(a, rhs_lane + (size_t)c[j] * k, k, ls * S::kVec);
+        // transpose-reduce: afterwards lane (ls & 3) == j holds slot j of the quad
+        const bool hi2 = ls & 2, hi1 = ls & 1;
+        const float k0 = hi2 ? p[2] : p[0], s0 = hi2 ? p[0] : p[2];
+        const float k1 = hi2 ? p[3] : p[1], s1 = hi2 ? p[1] : p[3];
+        const float q0 = k0 + lane_xor2(s0);
+        const float q1 = k1 + lane_xor2(s1);
+        float r = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
+        r = butterfly_sum<4, LPR>(r);
+        if ((ls >> 2) == q) result = r;
     }
     return result;
 }
 
-template <typename T, int K>
-__device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int row, int lane,
-                                               float (&a)[SddmmShape<T, K>::kVec])
+template <typename T, int KT, int NS, bool EDGE>
+__device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int row, int k, int lane,
+                                               float (&a)[NS][SddmmShape<T, KT>::kVec])
 {
-    using S = SddmmShape<T, K>;
-    DenseVec<T>::load(lhs + (size_t)row * K + (lane % S::kLpr) * S::kVec, a);
+    using S = SddmmShape<T, KT>;
+    const int e0 = (lane % S::kLpr) * S::kVec;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+#pragma unroll
+        for (int x = 0; x < S::kVec; ++x) a[s][x] = 0.f;
+        if (!EDGE || e0 + s * KT < k) DenseVec<T>::load(lhs + (size_t)row * k + e0 + s * KT, a[s]);
+    }
 }
 
 // One wave per block segment.  Segment s covers the aligned slots
 // [base, base + cnt) with base = st_off[s] & ~3 and cnt = floor((len + mask) / 32) * 32
 // (RoDeSddmm.cu:35-54); the first `mask` slots belong to the previous row and are
 // computed but never stored (RoDeSddmm.cu:56-58, 197).
-template <typename T, int K>
+template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_block_kernel(int m1, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+sddmm_block_kernel(int m1, int k, const int* __restrict__ block_rows, const int* __restrict__ st_off,
                    const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                    const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
 {
-    using S = SddmmShape<T, K>;
+    using S = SddmmShape<T, KT>;
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int seg = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
@@ -112,8 +131,8 @@ sddmm_block_kernel(int m1, const int* __restrict__ block_rows, const int* __rest
     const int base = start - mask;
     const int cnt = (end - start + mask) / kBlockItems * kBlockItems;
 
-    float a[S::kVec];
-    load_lhs_slice<T, K>(lhs, row, lane, a);
+    float a[NS][S::kVec];
+    load_lhs_slice<T, KT, NS, EDGE>(lhs, row, k, lane, a);
     const T* rhs_lane = rhs + (lane % S::kLpr) * S::kVec;
     int* lds_cols = lds + wave * kWave;
 
@@ -122,7 +141,7 @@ sddmm_block_kernel(int m1, const int* __restrict__ block_rows, const int* __rest
             const int slot = off + lane;
             const int c = col[base + slot];
             const float v = val[base + slot];
-            const float d = sddmm_unit<T, K, true>(rhs_lane, a, c, 32, lds_cols, lane);
+            const float d = sddmm_unit<T, KT, NS, EDGE>(rhs_lane, a, c, k, lds_cols, lane);
             if (slot >= mask) out[base + slot] = v * d;
         }
     }
@@ -132,13 +151,13 @@ sddmm_block_kernel(int m1, const int* __restrict__ block_rows, const int* __rest
 // with N = len + (s & 3), rows with N >= 32 keep only their last N % 32 slots
 // starting at (s & ~3) + floor(N / 32) * 32; shorter rows are taken whole.
 // Lane ls of the group owns the slots ls, ls + LPR, ... (value, result, store).
-template <typename T, int K>
+template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_residue_kernel(int m2, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
+sddmm_residue_kernel(int m2, int k, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
                      const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
                      const T* __restrict__ rhs, float* __restrict__ out)
 {
-    using S = SddmmShape<T, K>;
+    using S = SddmmShape<T, KT>;
     constexpr int VEC = S::kVec, LPR = S::kLpr;
     constexpr int RPW = kWave / LPR;          // rows per wave
     constexpr int OWN = kBlockItems / LPR;    // slots owned by one lane
@@ -173,8 +192,8 @@ sddmm_residue_kernel(int m2, const int* __restrict__ residue_rows, const int* __
             v[i] = val[idx];
         }
     }
-    float a[VEC];
-    load_lhs_slice<T, K>(lhs, row, lane, a);
+    float a[NS][VEC];
+    load_lhs_slice<T, KT, NS, EDGE>(lhs, row, k, lane, a);
     const T* rhs_lane = rhs + ls * VEC;
     wave_lds_sync();
 
@@ -189,14 +208,8 @@ sddmm_residue_kernel(int m2, const int* __restrict__ residue_rows, const int* __
             const int c[4] = {c4.x, c4.y, c4.z, c4.w};
             float p[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float b[VEC];
-                DenseVec<T>::load(rhs_lane + (size_t)c[j] * K, b);
-                float d = 0.f;
-#pragma unroll
-                for (int x = 0; x < VEC; ++x) d = fmaf(a[x], b[x], d);
-                p[j] = d;
-            }
+            for (int j = 0; j < 4; ++j)
+                p[j] = lane_dot<T, KT, NS, EDGE>(a, rhs_lane + (size_t)c[j] * k, k, ls * VEC);
             const bool hi2 = ls & 2, hi1 = ls & 1;
             const float q0 = (hi2 ? p[2] : p[0]) + lane_xor2(hi2 ? p[0] : p[2]);
             const float q1 = (hi2 ? p[3] : p[1]) + lane_xor2(hi2 ? p[1] : p[3]);
@@ -220,36 +233,54 @@ inline int grid_for_waves(long long nwaves)
     return (int)wgs;
 }
 
-template <typename T, int K>
-hipError_t launch(int m1, int m2, const int* block_rows, const int* residue_rows, const int* st_off,
+template <typename T, int KT, int NS, bool EDGE>
+hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* residue_rows, const int* st_off,
                   const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
                   hipStream_t s1, hipStream_t s2)
 {
     if (m1 > 0) {
-        sddmm_block_kernel<T, K><<<grid_for_waves(m1), kWgThreads, 0, s1>>>(m1, block_rows, st_off, row_ptr, col, val,
-                                                                            lhs, rhs, out);
+        sddmm_block_kernel<T, KT, NS, EDGE><<<grid_for_waves(m1), kWgThreads, 0, s1>>>(
+            m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
     }
     if (m2 > 0) {
-        constexpr int RPW = kWave / SddmmShape<T, K>::kLpr;
-        sddmm_residue_kernel<T, K><<<grid_for_waves(((long long)m2 + RPW - 1) / RPW), kWgThreads, 0, s2>>>(
-            m2, residue_rows, row_ptr, col, val, lhs, rhs, out);
+        constexpr int RPW = kWave / SddmmShape<T, KT>::kLpr;
+        sddmm_residue_kernel<T, KT, NS, EDGE><<<grid_for_waves(((long long)m2 + RPW - 1) / RPW), kWgThreads, 0, s2>>>(
+            m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out);
     }
     return hipGetLastError();
 }
 
+template <typename T, int KT, int NS>
+hipError_t launch_edge(bool edge, int m1, int m2, int k, const int* block_rows, const int* residue_rows,
+                       const int* st_off, const int* row_ptr, const int* col, const float* val, const T* lhs,
+                       const T* rhs, float* out, hipStream_t s1, hipStream_t s2)
+{
+    return edge ? launch<T, KT, NS, true>(m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out,
+                                          s1, s2)
+                : launch<T, KT, NS, false>(m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs,
+                                           out, s1, s2);
+}
+
 } // namespace
 
+// k: any positive multiple of the 128-bit vector width (4 for fp32, 8 for fp16) up to 512.
+// 32, 64 and 128 (the reference has 32 and 128) run without any bounds test.
 template <typename T>
 hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int* residue_rows, const int* st_off,
                         const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs,
                         float* out, hipStream_t s1, hipStream_t s2)
 {
-    switch (k) {
-    case 32: return launch<T, 32>(m1, m2, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, s1, s2);
-    case 64: return launch<T, 64>(m1, m2, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, s1, s2);
-    case 128: return launch<T, 128>(m1, m2, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, s1, s2);
-    default: return hipErrorInvalidValue;
-    }
+    if (k <= 0 || k % DenseVec<T>::kElems != 0 || k > 512) return hipErrorInvalidValue;
+#define RODE_SDDMM_CASE(KT, NS)                                                                                   \
+    return launch_edge<T, KT, NS>(k != (KT) * (NS), m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, \
+                                  lhs, rhs, out, s1, s2)
+    if (k <= 32) RODE_SDDMM_CASE(32, 1);
+    if (k <= 64) RODE_SDDMM_CASE(64, 1);
+    if (k <= 128) RODE_SDDMM_CASE(128, 1);
+    if (k <= 256) RODE_SDDMM_CASE(128, 2);
+    if (k <= 384) RODE_SDDMM_CASE(128, 3);
+    RODE_SDDMM_CASE(128, 4);
+#undef RODE_SDDMM_CASE
 }
 
 template hipError_t sddmm_launch<float>(int, int, int, const int*, const int*, const int*, const int*, const int*,

@@ -98,7 +98,7 @@ __device__ __forceinline__ void store_row(double* dst, const double (&acc)[VEC])
 
 // One wave per block segment (see sddmm_block_kernel for the slot arithmetic,
 // identical at RoDeSpmm.cu:210-234).
-template <typename T, int TN>
+template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* __restrict__ st_off,
                   const int* __restrict__ row_ptr, const int* __restrict__ col,
@@ -123,7 +123,10 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
 
     const int ls = lane % LPR, group = lane / LPR;
     const int tile = blockIdx.y * TN;
-    const T* b_lane = B + tile + ls * VEC;
+    // EDGE: n is not a multiple of TN; lanes past the last column re-read the tile's
+    // first columns (a valid address) and never write
+    const bool col_ok = !EDGE || tile + ls * VEC < n;
+    const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
     int* my_c = lds_c + wave * kWave;
     A* my_v = lds_v + wave * kWave;
 
@@ -157,13 +160,13 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
 #pragma unroll
     for (int x = 0; x < VEC; ++x) {
         const A total = butterfly_sum<LPR, kWave>(acc[x]);
-        if (group == x / EPG) atomicAdd(c_lane + x, total);
+        if (group == x / EPG && col_ok) atomicAdd(c_lane + x, total);
     }
 }
 
 // One group of LPR lanes per residue row (tail selection: RoDeSpmm.cu:71-82); the
 // group walks its row's slot quads one after the other, no cross-lane reduction.
-template <typename T, int TN>
+template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
                     const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
@@ -193,6 +196,7 @@ spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const i
     }
 
     const int tile = blockIdx.y * TN;
+    const bool col_ok = !EDGE || tile + ls * VEC < n;
     int* my_c = lds_c + (wave * RPW + group) * kBlockItems;
     A* my_v = lds_v + (wave * RPW + group) * kBlockItems;
 
@@ -211,10 +215,12 @@ spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const i
             }
         }
         wave_lds_sync();
-        spmm_gather<T, TN, kBlockItems / 4, false>(B + tile + ls * VEC, (size_t)n, acc, my_c, my_v, 0, 1, padded / 4);
+        spmm_gather<T, TN, kBlockItems / 4, false>(B + tile + (col_ok ? ls * VEC : 0), (size_t)n, acc, my_c, my_v, 0, 1,
+                                                   padded / 4);
     }
 
     A* c_lane = C + (size_t)row * n + tile + ls * VEC;
+    if (!col_ok) return;
     if (accumulate) {
 #pragma unroll
         for (int x = 0; x < VEC; ++x) atomicAdd(c_lane + x, acc[x]);
@@ -230,41 +236,57 @@ inline int grid_for_waves(long long nwaves)
     return (int)wgs;
 }
 
-template <typename T, int TN>
+template <typename T, int TN, bool EDGE>
 hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                   const int* row_ptr, const int* col, const typename DenseVec<T>::Acc* val, const T* B,
                   typename DenseVec<T>::Acc* C, hipStream_t s1, hipStream_t s2)
 {
-    const int tiles = n / TN;
+    const int tiles = (n + TN - 1) / TN;
     if (m1 > 0) {
         dim3 grid(grid_for_waves(m1), tiles);
-        spmm_block_kernel<T, TN><<<grid, kWgThreads, 0, s1>>>(m1, n, block_rows, st_off, row_ptr, col, val, B, C);
+        spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_rows, st_off, row_ptr, col, val, B, C);
     }
     if (m2 > 0) {
         constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
         dim3 grid(grid_for_waves(((long long)m2 + RPW - 1) / RPW), tiles);
-        spmm_residue_kernel<T, TN><<<grid, kWgThreads, 0, s2>>>(m2, n, residue_rows, row_ptr, col, val, B, C);
+        spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, residue_rows, row_ptr, col, val, B, C);
     }
     return hipGetLastError();
 }
 
+template <typename T, int TN>
+hipError_t launch_edge(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
+                       const int* row_ptr, const int* col, const typename DenseVec<T>::Acc* val, const T* B,
+                       typename DenseVec<T>::Acc* C, hipStream_t s1, hipStream_t s2)
+{
+    return n % TN ? launch<T, TN, true>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2)
+                  : launch<T, TN, false>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
+}
+
 } // namespace
 
+// n: any positive multiple of the 128-bit vector width (4 fp32, 8 fp16, 2 fp64).  The
+// dense row is cut into tiles of 32, 64 or 128 columns (at most 32 lanes per tile row);
+// the tile width with the least padding wins, the widest on a tie.  Multiples of 32 (all
+// the reference supports) run without any bounds test.
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                        const int* row_ptr, const int* col, const typename SpmmAcc<T>::type* val, const T* B,
                        typename SpmmAcc<T>::type* C, hipStream_t s1, hipStream_t s2)
 {
     static_assert(std::is_same<typename SpmmAcc<T>::type, typename DenseVec<T>::Acc>::value, "accumulation type");
-    if (n <= 0 || n % 32 != 0) return hipErrorInvalidValue;
-    // widest tile whose row is covered by at most 32 lanes of 128-bit loads
+    if (n <= 0 || n % DenseVec<T>::kElems != 0) return hipErrorInvalidValue;
     constexpr int kMaxTile = 32 * DenseVec<T>::kElems >= 128 ? 128 : 32 * DenseVec<T>::kElems;
+    auto padded = [n](int tn) { return (n + tn - 1) / tn * tn; };
+    int best = 32;
+    if (padded(64) <= padded(best)) best = 64;
+    if (kMaxTile >= 128 && padded(128) <= padded(best)) best = 128;
     if constexpr (kMaxTile >= 128) {
-        if (n % 128 == 0)
-            return launch<T, 128>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
+        if (best == 128)
+            return launch_edge<T, 128>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
     }
-    if (n % 64 == 0) return launch<T, 64>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
-    return launch<T, 32>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
+    if (best == 64) return launch_edge<T, 64>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
+    return launch_edge<T, 32>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
 }
 
 template hipError_t spmm_launch<float>(int, int, int, const int*, const int*, const int*, const int*, const int*,

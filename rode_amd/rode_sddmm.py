@@ -32,15 +32,18 @@ class RoDeCSR:
         128: {"seg_length": 512, "k_block": 32, "vec_len": 4},
     }
 
+    DEFAULT_CONFIG = {"seg_length": 512, "k_block": 32, "vec_len": 4}  # for a k that is not in CONFIGS
+    MAX_K = 512
+
     def __init__(self, row_offsets, column_indices, values, device, m, n, k=128, config=None):
-        if k not in self.CONFIGS:
-            raise ValueError(f"k must be one of {sorted(self.CONFIGS)}, got {k}")
+        if not (isinstance(k, int) and 0 < k <= self.MAX_K and k % 4 == 0):
+            raise ValueError(f"k must be a positive multiple of 4 up to {self.MAX_K} (the reference: 32 or 128), got {k}")
         self.m = m
         self.n = n
         self.k = k
         self.nnz = values.numel()
         self.device = torch.device(device)
-        self.config = dict(config) if config is not None else dict(self.CONFIGS[k])
+        self.config = dict(config) if config is not None else dict(self.CONFIGS.get(k, self.DEFAULT_CONFIG))
 
         self.row_offsets_cpu = row_offsets.to(dtype=torch.int32, device="cpu").contiguous()
         self.column_indices = column_indices.to(dtype=torch.int32, device=self.device).contiguous()

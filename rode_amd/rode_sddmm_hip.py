@@ -13,7 +13,8 @@ import torch
 
 from . import _lib
 
-_SUPPORTED_K = (32, 64, 128)
+_VEC = {torch.float32: 4, torch.float16: 8, torch.float64: 2}  # elements per 128-bit load
+_MAX_K = 512
 
 
 def _check(cond, msg):
@@ -91,8 +92,9 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
                   lhs_matrix, rhs_matrix, k_version):
     """``rode_sddmm_cuda.sddmm_forward`` (``rode_sddmm_cuda.cu:136-249``).
 
-    Differences from the reference, none of which changes a result: k_version 64
-    and fp16 ``lhs_matrix``/``rhs_matrix`` (fp32 accumulate) are accepted too; the
+    Differences from the reference, none of which changes a result: any k_version
+    that is a multiple of 4 up to 512 (multiple of 8 for fp16) and fp16
+    ``lhs_matrix``/``rhs_matrix`` (fp32 accumulate) are accepted too; the
     kernels are queued on PyTorch's current stream instead of two streams that
     are created, synchronised and destroyed per call (``:203-246``).
     """
@@ -108,7 +110,9 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
 
     k = lhs_matrix.size(1)
     nnz = values.size(0)
-    _check(k_version in _SUPPORTED_K, "k_version must be 32, 64 or 128")
+    vec = _VEC[lhs_matrix.dtype]
+    _check(0 < k_version <= _MAX_K and k_version % vec == 0,
+           f"k_version must be a positive multiple of {vec} up to {_MAX_K} (the reference has 32 and 128)")
     _check(k == k_version, "k dimension must match k_version")
     _check(lhs_matrix.size(0) == m, "lhs_matrix rows must equal m")
     _check(rhs_matrix.size(0) == n, "rhs_matrix rows must equal n")
@@ -132,7 +136,7 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
                  dense_matrix, out=None):
     """C = A_csr @ dense_matrix through ``rode_hip_spmm_f32`` / ``_f16``
     (host API ``RoDe_SpMM/RoDeSpmm.h:4-8``).  ``dense_matrix`` is (k, n) with n a
-    multiple of 32, fp32 / fp16 (fp32 ``values``) or fp64 (fp64 ``values``); the
+    multiple of 4 (8 for fp16, 2 for fp64), fp32 / fp16 (fp32 ``values``) or fp64 (fp64 ``values``); the
     result is a new zero-initialised (m, n) tensor of the dtype of ``values``, or
     ``out`` accumulated in place the way the reference kernels do (long rows add,
     short rows overwrite)."""
@@ -152,7 +156,8 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     out_dtype = values.dtype
     _check(dense_matrix.dim() == 2 and dense_matrix.size(0) == k, "dense_matrix rows must equal k")
     n = dense_matrix.size(1)
-    _check(n > 0 and n % 32 == 0, "dense_matrix cols must be a positive multiple of 32")
+    vec = _VEC[dense_matrix.dtype]
+    _check(n > 0 and n % vec == 0, f"dense_matrix cols must be a positive multiple of {vec}")
     if out is None:
         out = torch.zeros((m, n), dtype=out_dtype, device=values.device)
     else:

@@ -7,13 +7,15 @@ from . import rode_sddmm_hip
 
 def rode_spmm(sparse_matrix, dense, out=None, values=None):
     """C = S @ dense.  ``dense`` is (n, width) float32 or float16 with ``width`` a
-    multiple of 32; returns an (m, width) float32 tensor.  ``values`` (optional)
+    multiple of 4 (8 for float16; multiples of 32 are the fast path); returns an
+    (m, width) float32 tensor.  ``values`` (optional)
     replaces the values of S for this call.  Differentiable with respect to dense
     and values when ``out`` is not given."""
     if dense.dim() != 2 or dense.shape[0] != sparse_matrix.n:
         raise ValueError(f"dense shape must be ({sparse_matrix.n}, width), got {tuple(dense.shape)}")
-    if dense.shape[1] % 32 != 0:
-        raise ValueError(f"dense width must be a multiple of 32, got {dense.shape[1]}")
+    vec = 8 if dense.dtype == torch.float16 else 4
+    if dense.shape[1] == 0 or dense.shape[1] % vec != 0:
+        raise ValueError(f"dense width must be a positive multiple of {vec}, got {dense.shape[1]}")
     assert dense.is_cuda and dense.device == sparse_matrix.device, (
         f"dense must be on {sparse_matrix.device}, got {dense.device}")
     assert dense.dtype in (torch.float32, torch.float16), f"dense must be float32 or float16, got {dense.dtype}"

@@ -111,6 +111,23 @@ def test_unpadded_rows(k, seg):
     _check(make_csr(rp, col, val, m, n, k, seg), rp, col, val, lhs, rhs)
 
 
+@pytest.mark.parametrize("k", [4, 8, 20, 48, 96, 100, 160, 256, 300, 384, 512])
+def test_any_k(k):
+    """k beyond the reference's 32 / 128: any multiple of 4 up to 512 (row tiles of 32 /
+    64 / 128 elements, up to four slabs, the partial last slab guarded)."""
+    from gpu_common import make_csr
+    from helpers import random_csr
+    rng = np.random.default_rng(k)
+    m, n = 700, 800
+    rp, col, val = random_csr(rng, m, n, 35, long_rows=4, long_len=750, empty_frac=0.1)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    csr = make_csr(rp, col, val, m, n, k)
+    _check(csr, rp, col, val, lhs, rhs)
+    if k % 8 == 0:
+        _check(csr, rp, col, val, lhs, rhs, half=True)
+
+
 @pytest.mark.parametrize("k", [32, 64, 128])
 def test_fp16_operands(k):
     from gpu_common import make_csr
@@ -163,7 +180,7 @@ def test_argument_errors():
     csr = make_csr(rp, col, val, 40, 50, 32)
     lhs, rhs = torch.zeros(40, 32, device=DEV), torch.zeros(50, 32, device=DEV)
     with pytest.raises(ValueError):
-        RoDeCSR(torch.from_numpy(rp), torch.from_numpy(col), torch.from_numpy(val), DEV, 40, 50, 48)
+        RoDeCSR(torch.from_numpy(rp), torch.from_numpy(col), torch.from_numpy(val), DEV, 40, 50, 50)
     with pytest.raises(ValueError):
         rode_sddmm(csr, lhs[:, :16], rhs)
     with pytest.raises(ValueError):
@@ -174,7 +191,7 @@ def test_argument_errors():
         rode_sddmm(csr, lhs.double(), rhs.double())
     args = [csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2, csr.row_offsets,
             csr.column_indices, csr.values, 40, 50, lhs, rhs, 32]
-    for pos, bad, msg in [(12, 48, "k_version"), (12, 128, "match k_version"), (8, 41, "rows must equal m"),
+    for pos, bad, msg in [(12, 50, "k_version must be"), (12, 128, "match k_version"), (8, 41, "rows must equal m"),
                           (7, csr.values.double(), "float32"), (6, csr.column_indices.long(), "int32"),
                           (10, lhs.cpu(), "CUDA tensor"), (11, rhs.t().contiguous().t(), "contiguous")]:
         a = list(args)

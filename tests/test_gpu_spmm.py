@@ -41,6 +41,55 @@ def test_unpadded_rows(n, seg):
     _check(make_csr(rp, col, val, m, k, 32, seg), rp, col, val, B)
 
 
+@pytest.mark.parametrize("n", [4, 8, 20, 36, 72, 100, 160, 200, 264])
+def test_any_width(n):
+    """Widths beyond the reference's multiples of 32: any multiple of 4 (the partial last
+    tile is guarded; the columns next to it must stay untouched)."""
+    import oracle
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr, spmm_row_l1_error
+    from rode_amd import rode_spmm
+    rng = np.random.default_rng(n)
+    m, k = 600, 650
+    rp, col, val = random_csr(rng, m, k, 35, long_rows=4, long_len=600, empty_frac=0.1)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    csr = make_csr(rp, col, val, m, k, 32)
+    _check(csr, rp, col, val, B)
+    if n % 8 == 0:
+        _check(csr, rp, col, val, B, half=True)
+    assert rode_spmm(csr, torch.from_numpy(B).to(DEV)).shape == (m, n)
+    # an fp64 run of the same width (vector of 2)
+    from rode_amd import rode_sddmm_hip
+    C64 = rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                      csr.row_offsets, csr.column_indices, csr.values.double(), m, k,
+                                      torch.from_numpy(B).to(DEV).double()).cpu().numpy()
+    ref = oracle.spmm_f64(rp, col, val, B)
+    assert spmm_row_l1_error(C64, ref) <= 1e-12
+
+
+def test_edge_tile_does_not_write_past_the_row():
+    """C is (m, n) with n = 36: the second 32-wide tile has 4 live columns.  A canary row
+    appended after C and the next row's first columns must be unchanged / correct."""
+    import oracle
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(77)
+    m, k, n = 300, 320, 36
+    rp, col, val = random_csr(rng, m, k, 40, long_rows=3, long_len=300)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    csr = make_csr(rp, col, val, m, k, 32)
+    buf = torch.zeros((m + 1) * n, device=DEV)
+    buf[m * n:] = 123.0
+    out = buf[: m * n].view(m, n)
+    rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                csr.row_offsets, csr.column_indices, csr.values, m, k, torch.from_numpy(B).to(DEV),
+                                out=out)
+    assert (buf[m * n:] == 123.0).all()
+    ref = oracle.spmm_f64(rp, col, val, B)
+    assert np.abs(out.cpu().numpy() - ref).max() <= 1e-4 * np.abs(ref).sum(axis=1).max()
+
+
 def test_padded_reference_matrices():
     """The reference generators' matrices (rows padded to 4 with explicit zeros)."""
     from gpu_common import make_csr
@@ -164,7 +213,7 @@ def test_special_cases_and_edges():
     assert not rode_spmm(empty, torch.ones(7, 32, device=DEV)).any()
     # width not a multiple of 32
     with pytest.raises(ValueError):
-        rode_spmm(csr, torch.zeros(k, 40, device=DEV))
+        rode_spmm(csr, torch.zeros(k, 42, device=DEV))
     with pytest.raises(ValueError):
         rode_spmm(csr, torch.zeros(k + 1, 32, device=DEV))
 

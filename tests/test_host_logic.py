@@ -18,7 +18,9 @@ def test_config_tables():
 def test_errors_raised_before_any_device_work():
     rp = torch.tensor([0, 2, 4], dtype=torch.int32)
     with pytest.raises(ValueError, match="k must be"):
-        RoDeCSR(rp, torch.zeros(4, dtype=torch.int32), torch.zeros(4), "cpu", 2, 4, k=48)
+        RoDeCSR(rp, torch.zeros(4, dtype=torch.int32), torch.zeros(4), "cpu", 2, 4, k=50)
+    with pytest.raises(ValueError, match="k must be"):
+        RoDeCSR(rp, torch.zeros(4, dtype=torch.int32), torch.zeros(4), "cpu", 2, 4, k=1024)
     with pytest.raises(RuntimeError, match="int32"):
         rode_sddmm_hip.preprocess(rp.long(), 4, 512, 32, 4)
     with pytest.raises(RuntimeError, match="CUDA tensor"):
