@@ -319,3 +319,34 @@ def test_full_size_properties(name, n):
     C12 = rode_spmm(csr, B + B2)
     denom = torch.from_numpy(abs_sums).to(DEV).float()[:, None] * 8 + 1e-20
     assert ((C12 - (C + C2)).abs() / denom).max().item() < 1e-4
+
+
+def test_dense_operand_beyond_2_gib():
+    """B and rhs of 2.4 GB: byte offsets col * n * 4 exceed 2^31, where the reference's
+    32-bit offset arithmetic (RoDeSpmm.cu:153,287) overflows.  Checked on the rows'
+    exact expected values: B[c, j] = (c % 1000) + j / 256 is exactly representable."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import rode_sddmm, rode_spmm
+    rng = np.random.default_rng(31)
+    m, n, k = 2000, 4_700_000, 128
+    lens = rng.integers(0, 90, m)
+    lens[7] = 3000
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(n, size=l, replace=False)) for l in lens]).astype(np.int32)
+    col[rp[7 + 1] - 1] = n - 1  # the very last dense row
+    val = np.ones(len(col), np.float32)
+    csr = make_csr(rp, col, val, m, n, k)
+    B = (torch.arange(n, device=DEV) % 1000).float()[:, None] + torch.arange(k, device=DEV).float()[None, :] / 256
+    assert B.numel() * 4 > 2**31
+    C = rode_spmm(csr, B).cpu().numpy().astype(np.float64)
+    colsum = np.zeros(m)
+    nonempty = np.nonzero(lens > 0)[0]
+    colsum[nonempty] = np.add.reduceat((col % 1000).astype(np.float64), rp[nonempty].astype(np.int64))
+    want = colsum[:, None] + lens[:, None] * (np.arange(k) / 256.0)[None, :]
+    # fp32 accumulation of up to 3000 terms per row
+    assert (np.abs(C - want).max(axis=1) <= 1e-4 * np.abs(want).max(axis=1) + 1e-30).all()
+    # SDDMM with lhs = e_0: out[idx] = rhs[col, 0] = col % 1000
+    lhs = torch.zeros(m, k, device=DEV)
+    lhs[:, 0] = 1
+    out = rode_sddmm(csr, lhs, B).cpu().numpy()
+    np.testing.assert_array_equal(out, (col % 1000).astype(np.float32))
