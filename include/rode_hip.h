@@ -47,8 +47,10 @@ size_t rode_hip_preprocess_workspace_bytes(int M);
  *   d_st_off         int[cap+1]  out: first nonzero of every block segment, then the sentinel
  *   d_residue_r_ind  int[>=M]    out: rows that own a residue
  *   d_n_blk, d_n_res int[1] each out: segment / residue counts
- *   capacity_blocks  cap above; must be >= (nnz + (vec_len-1)*M)/seg_length + M
- *                    (the reference sizes it nnz/seg + M, _preprocess.cu:426)
+ *   capacity_blocks  cap above; (nnz + (vec_len-1)*M)/seg_length + M always suffices
+ *                    (the reference sizes it nnz/seg + M, _preprocess.cu:426).  If it is
+ *                    too small nothing is written past it and *d_n_blk still reports
+ *                    the true count, so the caller can detect the overflow.
  *   d_workspace      rode_hip_preprocess_workspace_bytes(M) bytes, 8-byte aligned
  */
 int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const int* d_row_ptr,

@@ -84,9 +84,10 @@ tile_reduce_kernel(int seg, int kblock, int veclen, int M, const int* __restrict
 
 // One workgroup: exclusive scan of the tile sums, totals, sentinel.
 __global__ void __launch_bounds__(kWgThreads)
-tile_scan_kernel(int M, int ntiles, const int* __restrict__ row_ptr, const unsigned long long* __restrict__ tile_sum,
-                 unsigned long long* __restrict__ tile_prefix, int* __restrict__ row_blk_prefix,
-                 int* __restrict__ st_off, int* __restrict__ n_blk, int* __restrict__ n_res)
+tile_scan_kernel(int M, int ntiles, int capacity, const int* __restrict__ row_ptr,
+                 const unsigned long long* __restrict__ tile_sum, unsigned long long* __restrict__ tile_prefix,
+                 int* __restrict__ row_blk_prefix, int* __restrict__ st_off, int* __restrict__ n_blk,
+                 int* __restrict__ n_res)
 {
     unsigned long long carry = 0;
     for (int base = 0; base < ntiles; base += kWgThreads) {
@@ -102,7 +103,9 @@ tile_scan_kernel(int M, int ntiles, const int* __restrict__ row_ptr, const unsig
         *n_blk = nb;
         *n_res = (int)(carry & 0xffffffffull);
         row_blk_prefix[M] = nb;
-        st_off[nb] = row_ptr[M];
+        // a caller whose arrays are too small still gets the true counts, and nothing is
+        // written past `capacity` segments (st_off holds capacity + 1 entries)
+        if (nb <= capacity) st_off[nb] = row_ptr[M];
     }
 }
 
@@ -136,11 +139,11 @@ row_scan_kernel(int seg, int kblock, int veclen, int M, const int* __restrict__ 
 
 // One thread per block segment j: its row is the last r with prefix[r] <= j.
 __global__ void __launch_bounds__(kWgThreads)
-fill_segments_kernel(int seg, int veclen, int M, const int* __restrict__ row_ptr,
+fill_segments_kernel(int seg, int veclen, int M, int capacity, const int* __restrict__ row_ptr,
                      const int* __restrict__ row_blk_prefix, int* __restrict__ block_r_ind,
                      int* __restrict__ st_off)
 {
-    const int n_blk = row_blk_prefix[M];
+    const int n_blk = min(row_blk_prefix[M], capacity);
     for (int j = blockIdx.x * kWgThreads + threadIdx.x; j < n_blk; j += gridDim.x * kWgThreads) {
         int lo = 0, hi = M; // invariant: prefix[lo] <= j < prefix[hi]
         while (hi - lo > 1) {
@@ -174,8 +177,8 @@ hipError_t preprocess_launch(int seg, int kblock, int veclen, int M, const int* 
 
     if (ntiles > 0)
         tile_reduce_kernel<<<ntiles, kWgThreads, 0, stream>>>(seg, kblock, veclen, M, row_ptr, tile_sum);
-    tile_scan_kernel<<<1, kWgThreads, 0, stream>>>(M, ntiles, row_ptr, tile_sum, tile_prefix, row_blk_prefix,
-                                                    st_off, n_blk, n_res);
+    tile_scan_kernel<<<1, kWgThreads, 0, stream>>>(M, ntiles, capacity_blocks, row_ptr, tile_sum, tile_prefix,
+                                                    row_blk_prefix, st_off, n_blk, n_res);
     if (ntiles > 0) {
         row_scan_kernel<<<ntiles, kWgThreads, 0, stream>>>(seg, kblock, veclen, M, row_ptr, tile_prefix,
                                                             row_blk_prefix, residue_r_ind);
@@ -183,8 +186,8 @@ hipError_t preprocess_launch(int seg, int kblock, int veclen, int M, const int* 
         // capacity bound and let the kernel stride.
         long long want = ((long long)capacity_blocks + kWgThreads - 1) / kWgThreads;
         const int grid = (int)(want < 1 ? 1 : (want > 4096 ? 4096 : want));
-        fill_segments_kernel<<<grid, kWgThreads, 0, stream>>>(seg, veclen, M, row_ptr, row_blk_prefix,
-                                                               block_r_ind, st_off);
+        fill_segments_kernel<<<grid, kWgThreads, 0, stream>>>(seg, veclen, M, capacity_blocks, row_ptr,
+                                                               row_blk_prefix, block_r_ind, st_off);
     }
     return hipGetLastError();
 }

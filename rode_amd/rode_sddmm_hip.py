@@ -65,7 +65,9 @@ def preprocess_device(row_offsets, nnz, seg_length, k_block, vec_len):
                                        counts.data_ptr() + 4, cap, ws.data_ptr(), ws_bytes, _stream_handle(dev))
         _lib.check(code, "rode_hip_preprocess")
         n_blk, n_res = (int(v) for v in counts.cpu())  # stream-ordered copy: waits for the kernels
-    return blk[: max(n_blk, 1)], st[: n_blk + 1], res[: max(n_res, 1)], n_blk, n_res
+    _check(n_blk <= cap and n_res <= max(m, 1), "row decomposition larger than its capacity bound")
+    # copies, so that the capacity-sized buffers are released
+    return blk[: max(n_blk, 1)].clone(), st[: n_blk + 1].clone(), res[: max(n_res, 1)].clone(), n_blk, n_res
 
 
 def preprocess(row_offsets, nnz, seg_length, k_block, vec_len):

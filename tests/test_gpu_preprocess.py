@@ -113,3 +113,33 @@ def test_cxx_reference_signature_entry_point():
     assert blk[:nb].cpu().numpy().tobytes() == oblk.tobytes()
     assert st[: nb + 1].cpu().numpy().tobytes() == ost.tobytes()
     assert res[:nr].cpu().numpy().tobytes() == ores.tobytes()
+
+
+def test_capacity_too_small_is_detected_not_overrun():
+    """With room for fewer segments than the matrix has, nothing is written past the
+    capacity and the true count comes back."""
+    import oracle
+    from rode_amd import _lib
+    lib = _lib.load()
+    rp = (np.arange(1001, dtype=np.int32) * 64)  # 1000 rows of 64 -> 2000 segments at seg 32
+    d_rp = torch.from_numpy(rp).cuda()
+    cap = 700
+    blk = torch.full((cap + 8,), -7, dtype=torch.int32, device="cuda")
+    st = torch.full((cap + 9,), -7, dtype=torch.int32, device="cuda")
+    res = torch.empty(1000, dtype=torch.int32, device="cuda")
+    cnt = torch.zeros(2, dtype=torch.int32, device="cuda")
+    nbytes = lib.rode_hip_preprocess_workspace_bytes(1000)
+    ws = torch.empty((nbytes + 7) // 8, dtype=torch.int64, device="cuda")
+    code = lib.rode_hip_preprocess(32, 32, 4, 1000, d_rp.data_ptr(), blk.data_ptr(), st.data_ptr(), res.data_ptr(),
+                                   cnt.data_ptr(), cnt.data_ptr() + 4, cap, ws.data_ptr(), nbytes, None)
+    assert code == 0
+    torch.cuda.synchronize()
+    oblk, ost, _ = oracle.preprocess(rp, 32)
+    assert cnt.tolist() == [2000, 0]
+    assert blk[:cap].cpu().numpy().tobytes() == oblk[:cap].tobytes() and (blk[cap:] == -7).all()
+    assert st[:cap].cpu().numpy().tobytes() == ost[:cap].tobytes() and (st[cap:] == -7).all()
+    # bad arguments are rejected before any launch
+    assert lib.rode_hip_preprocess(0, 32, 4, 1000, d_rp.data_ptr(), blk.data_ptr(), st.data_ptr(), res.data_ptr(),
+                                   cnt.data_ptr(), cnt.data_ptr() + 4, cap, ws.data_ptr(), nbytes, None) != 0
+    assert lib.rode_hip_preprocess(32, 32, 4, 1000, d_rp.data_ptr(), blk.data_ptr(), st.data_ptr(), res.data_ptr(),
+                                   cnt.data_ptr(), cnt.data_ptr() + 4, cap, ws.data_ptr(), 16, None) != 0
