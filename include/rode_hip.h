@@ -9,6 +9,10 @@
  * Return value: 0 on success, otherwise a hipError_t value
  * (rode_hip_error_string() turns it into text).
  *
+ * C of the SpMM calls must be ordinary (coarse-grained) device memory, as hipMalloc
+ * returns: long rows are summed with hardware floating-point atomics, which
+ * fine-grained or host-coherent allocations do not support.
+ *
  * Layout and alignment contract (same as the reference kernels, which use
  * 128-bit accesses throughout, e.g. RoDe_SpMM/RoDeSpmm.cu:89,247-248 and
  * RoDe_SDDMM/RoDeSddmm.cu:75,80,88): all arrays row-major and 16-byte aligned.
