@@ -78,6 +78,15 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
                       const int* d_row_seg_st_offsets, const float* d_B, float* d_C, void* stream1,
                       void* stream2);
 
+/*
+ * Prepares an uninitialised C[M x n] for one of the SpMM calls: zeroes exactly the rows
+ * that SpMM adds to (aligned length >= 32) or never touches (rows in no list) and
+ * leaves alone the rows it stores.  A cheaper replacement for clearing all of C; the
+ * reference has no counterpart (its callers memset C).  elem_bytes is 4 (f32, f16
+ * variants) or 8 (f64).  Must be ordered before both SpMM streams.
+ */
+int rode_hip_spmm_clear_rows(int M, int n, int elem_bytes, const int* d_row_offsets, void* d_C, void* stream);
+
 /* fp64 values, B and C.  Replaces the double overloads of RoDeSpmm_n32 / RoDeSpmm_n128,
  * RoDe_SpMM/RoDeSpmm.h:10-14, RoDeSpmm.cu:521-529.  Same contract as rode_hip_spmm_f32
  * (n a multiple of 2). */

@@ -49,6 +49,15 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
                                     d_column_indices, d_values, d_B, d_C, as_stream(stream1), as_stream(stream2));
 }
 
+int rode_hip_spmm_clear_rows(int M, int n, int elem_bytes, const int* d_row_offsets, void* d_C, void* stream)
+{
+    if (M < 0 || n <= 0 || (elem_bytes != 4 && elem_bytes != 8) || ((size_t)n * elem_bytes) % 16 != 0)
+        return hipErrorInvalidValue;
+    if (M == 0) return hipSuccess;
+    if (!d_row_offsets || !d_C || !aligned16(d_C)) return hipErrorInvalidValue;
+    return rode::spmm_clear_rows_launch(M, (size_t)n * elem_bytes, d_row_offsets, d_C, as_stream(stream));
+}
+
 int rode_hip_spmm_f64(int m1, int m2, int k, int n, const double* d_values, const int* d_column_indices,
                       const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
                       const int* d_row_seg_st_offsets, const double* d_B, double* d_C, void* stream1, void* stream2)

@@ -229,6 +229,24 @@ spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const i
     }
 }
 
+// Zeroes exactly the rows of C that the two SpMM kernels do not overwrite: rows whose
+// aligned length N = len + (start & 3) is >= 32 are accumulated into, rows with N == 0
+// belong to no work item; rows with 0 < N < 32 are stored by the residue kernel and
+// are left alone.  16 lanes x 16 bytes per step and row.
+__global__ void __launch_bounds__(kWgThreads)
+spmm_clear_rows_kernel(int M, size_t row_bytes, const int* __restrict__ row_ptr, char* __restrict__ C)
+{
+    constexpr int kLanes = 16, kRowsPerWg = kWgThreads / kLanes;
+    const int row = xcd_logical_block(blockIdx.x, gridDim.x) * kRowsPerWg + threadIdx.x / kLanes;
+    if (row >= M) return;
+    const int s = row_ptr[row], e = row_ptr[row + 1];
+    const int N = e - s + (s & (kVecLen - 1));
+    if (N > 0 && N < kBlockItems) return;
+    char* dst = C + (size_t)row * row_bytes;
+    for (size_t b = (threadIdx.x % kLanes) * 16; b < row_bytes; b += kLanes * 16)
+        *reinterpret_cast<uint4*>(dst + b) = make_uint4(0, 0, 0, 0);
+}
+
 inline int grid_for_waves(long long nwaves)
 {
     long long wgs = (nwaves + kWavesPerWg - 1) / kWavesPerWg;
@@ -287,6 +305,15 @@ hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* 
     }
     if (best == 64) return launch_edge<T, 64>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
     return launch_edge<T, 32>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, s1, s2);
+}
+
+hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, void* C, hipStream_t stream)
+{
+    if (M <= 0) return hipSuccess;
+    long long wgs = ((long long)M + 15) / 16;
+    wgs = (wgs + kXcds - 1) / kXcds * kXcds;
+    spmm_clear_rows_kernel<<<(int)wgs, kWgThreads, 0, stream>>>(M, row_bytes, row_ptr, static_cast<char*>(C));
+    return hipGetLastError();
 }
 
 template hipError_t spmm_launch<float>(int, int, int, const int*, const int*, const int*, const int*, const int*,

@@ -160,14 +160,20 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     n = dense_matrix.size(1)
     vec = _VEC[dense_matrix.dtype]
     _check(n > 0 and n % vec == 0, f"dense_matrix cols must be a positive multiple of {vec}")
+    lib = _lib.load()
     if out is None:
-        out = torch.zeros((m, n), dtype=out_dtype, device=values.device)
+        if m1 == 0 and m2 == 0:
+            return torch.zeros((m, n), dtype=out_dtype, device=values.device)
+        # only the rows the kernels add to (or skip) need clearing, the others are overwritten
+        out = torch.empty((m, n), dtype=out_dtype, device=values.device)
+        with torch.cuda.device(values.device):
+            _lib.check(lib.rode_hip_spmm_clear_rows(m, n, out.element_size(), row_offsets.data_ptr(), out.data_ptr(),
+                                                    _stream_handle(values.device)), "rode_hip_spmm_clear_rows")
     else:
         _check_input(out, "out")
         _check(out.dtype == out_dtype and tuple(out.shape) == (m, n), f"out must be {out_dtype} of shape (m, n)")
     if m1 == 0 and m2 == 0:
         return out
-    lib = _lib.load()
     fn = {torch.float32: lib.rode_hip_spmm_f32, torch.float16: lib.rode_hip_spmm_f16,
           torch.float64: lib.rode_hip_spmm_f64}[dense_matrix.dtype]
     with torch.cuda.device(values.device):

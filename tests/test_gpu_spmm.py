@@ -350,3 +350,35 @@ def test_dense_operand_beyond_2_gib():
     lhs[:, 0] = 1
     out = rode_sddmm(csr, lhs, B).cpu().numpy()
     np.testing.assert_array_equal(out, (col % 1000).astype(np.float32))
+
+
+def test_clear_rows_prepares_exactly_what_spmm_does_not_overwrite():
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import _lib, rode_sddmm_hip
+    lib = _lib.load()
+    rng = np.random.default_rng(13)
+    m, k, n = 900, 800, 96
+    rp, col, val = random_csr(rng, m, k, 30, long_rows=4, long_len=700, empty_frac=0.2)
+    csr = make_csr(rp, col, val, m, k, 32)
+    C = torch.full((m, n), float("nan"), device=DEV)
+    assert lib.rode_hip_spmm_clear_rows(m, n, 4, csr.row_offsets.data_ptr(), C.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    aligned = np.diff(rp) + rp[:-1] % 4
+    cleared = (aligned >= 32) | (aligned == 0)
+    got = C.cpu().numpy()
+    assert (got[cleared] == 0).all() and np.isnan(got[~cleared]).all()
+    # SpMM on the prepared buffer == SpMM on a fully zeroed one
+    B = torch.from_numpy(rng.standard_normal((k, n)).astype(np.float32)).to(DEV)
+    args = (csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2, csr.row_offsets,
+            csr.column_indices, csr.values, m, k, B)
+    a = rode_sddmm_hip.spmm_forward(*args, out=C)
+    b = rode_sddmm_hip.spmm_forward(*args, out=torch.zeros(m, n, device=DEV))
+    assert torch.isfinite(a).all() and (a - b).abs().max().item() <= 1e-5 * b.abs().max().item()
+    # fp64 element size, bad arguments
+    C64 = torch.full((m, 6), float("nan"), dtype=torch.float64, device=DEV)
+    assert lib.rode_hip_spmm_clear_rows(m, 6, 8, csr.row_offsets.data_ptr(), C64.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert (C64[torch.from_numpy(cleared).to(DEV)] == 0).all()
+    assert lib.rode_hip_spmm_clear_rows(m, 6, 4, csr.row_offsets.data_ptr(), C64.data_ptr(), None) != 0  # 24-byte rows
+    assert lib.rode_hip_spmm_clear_rows(m, 8, 2, csr.row_offsets.data_ptr(), C64.data_ptr(), None) != 0
