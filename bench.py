@@ -50,21 +50,24 @@ def parse_args():
     return p.parse_args()
 
 
-def work_split(row_ptr, col, ncols):
+def work_split(row_ptr, col, ncols, owned_slots=0):
     """Which nonzeros the residue kernels own (tail rule of RoDeSpmm.cu:71-82) and how
-    many distinct dense rows each kernel family touches."""
+    many distinct dense rows each kernel family touches.  ``owned_slots``: rows of
+    32..owned_slots aligned slots are summed, tail included, by the SpMM block kernel."""
     rp = row_ptr.astype(np.int64)
     s, e = rp[:-1], rp[1:]
     pad = s % 4
     N = e - s + pad
     tail_first = np.where(N >= 32, s - pad + N // 32 * 32, s)
+    tail_first = np.where((N >= 32) & (N <= owned_slots), e, tail_first)
     in_res = np.arange(rp[-1], dtype=np.int64) >= np.repeat(tail_first, e - s)
     nnz_res = int(in_res.sum())
     distinct_res = int((np.bincount(col[in_res], minlength=ncols) > 0).sum())
     distinct_blk = int((np.bincount(col[~in_res], minlength=ncols) > 0).sum())
     rows_blk = int((N >= 32).sum())
+    rows_res = int((((N % 32) != 0) & (N > 0) & ~((N >= 32) & (N <= owned_slots))).sum())
     return {"nnz_res": nnz_res, "nnz_blk": int(rp[-1]) - nnz_res, "distinct_res": distinct_res,
-            "distinct_blk": distinct_blk, "rows_blk": rows_blk}
+            "distinct_blk": distinct_blk, "rows_blk": rows_blk, "rows_res": rows_res}
 
 
 def algorithmic_bytes(kernel, split, m1, m2, k, elem):
@@ -216,7 +219,11 @@ def main():
         kernels["spmm_block"] = event_time(lambda: spmm(csr.m1, 0), reps)
         kernels["sddmm_block"] = event_time(lambda: sddmm(csr.m1, 0), reps)
     if csr.m2 > 0:
-        kernels["spmm_residue"] = event_time(lambda: spmm(0, csr.m2), reps)
+        # The SpMM residue kernel skips the rows its block kernel sums whole, which only
+        # happens when both are launched by one call: time the pair and subtract (the two
+        # kernels run back to back on one stream).
+        both = event_time(lambda: spmm(csr.m1, csr.m2), reps)
+        kernels["spmm_residue"] = max(both - kernels.get("spmm_block", 0.0), 1e-4)
         kernels["sddmm_residue"] = event_time(lambda: sddmm(0, csr.m2), reps)
     spmm_ms = event_time(lambda: (clear_c(), spmm(csr.m1, csr.m2)), reps)
     sddmm_ms = event_time(lambda: sddmm(csr.m1, csr.m2), reps)
@@ -228,10 +235,16 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    split = work_split(row_ptr, col, n)
+    # the SpMM block kernel sums rows of 32..1024 slots whole when there are >= 16384 segments
+    split_sddmm = work_split(row_ptr, col, n)
+    split_spmm = work_split(row_ptr, col, n, 1024 if csr.m1 >= 16384 else 0)
     per_kernel = {}
     for name, ms in kernels.items():
-        ab = algorithmic_bytes(name, split, csr.m1, csr.m2, k, elem)
+        split = split_spmm if name.startswith("spmm") else split_sddmm
+        m2_eff = csr.m2
+        if name == "spmm_residue":
+            m2_eff = split["rows_res"]
+        ab = algorithmic_bytes(name, split, csr.m1, m2_eff, k, elem)
         knnz = split["nnz_blk"] if name.endswith("block") else split["nnz_res"]
         per_kernel[name] = {"ms": round(ms, 4), "algorithmic_bytes": ab,
                             "algorithmic_GBs": round(ab / ms / 1e6, 1),

@@ -12,7 +12,10 @@
 //   * block kernel: one wave per block segment; its lane groups take
 //     interleaved slot quads, the partial rows are combined with a butterfly
 //     over the groups and added to C with hardware fp32 atomics (always, as in
-//     RoDeSpmm.cu:464-474: a long row has several segments and usually a residue);
+//     RoDeSpmm.cu:464-474: a long row has several segments and usually a residue).
+//     Rows of 32..1024 slots are an exception in the execution, not in the result:
+//     the wave of the row's first segment sums the whole row, tail included, and
+//     adds it to C once; the row's other work items return at once;
 //   * residue kernel: one group of LPR lanes per residue row, 64 / LPR rows per
 //     wave (short rows are latency-bound and need many rows in flight); rows
 //     shorter than 32 slots are stored with plain 128-bit stores, tails of
@@ -30,6 +33,14 @@
 namespace rode {
 
 namespace {
+
+// Rows of at most `owned_slots` aligned slots (and at least 32, i.e. rows that have block
+// segments) are summed by a single wave of the block kernel.  The launcher passes 1024
+// when there are enough block segments to keep every CU busy anyway, else 0 (every
+// work item on its own wave: small matrices need the parallelism more than they
+// mind the extra atomics).
+constexpr int kOwnedRowSlots = 1024;
+constexpr int kOwnedMinSegments = 16384;
 
 template <typename T, int TN>
 struct SpmmShape {
@@ -100,7 +111,7 @@ __device__ __forceinline__ void store_row(double* dst, const double (&acc)[VEC])
 // identical at RoDeSpmm.cu:210-234).
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_rows, const int* __restrict__ st_off,
                   const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                   typename DenseVec<T>::Acc* __restrict__ C)
@@ -115,11 +126,23 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
     if (seg >= m1) return;
 
     const int row = block_rows[seg];
-    const int start = st_off[seg];
-    const int end = min(row_ptr[row + 1], st_off[seg + 1]);
-    const int mask = start & (kVecLen - 1);
-    const int base = start - mask;
-    const int cnt = (end - start + mask) / kBlockItems * kBlockItems;
+    const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
+    int mask, base, cnt;
+    if (row_end - row_start + (row_start & (kVecLen - 1)) <= owned_slots) {
+        // A moderately long row is summed by ONE wave, the one of its first segment:
+        // all its segments and its tail, one update of C instead of one per work item.
+        // The residue kernel skips such rows by the same test.
+        if (seg > 0 && block_rows[seg - 1] == row) return;
+        mask = row_start & (kVecLen - 1);
+        base = row_start - mask;
+        cnt = row_end - base;
+    } else {
+        const int start = st_off[seg];
+        const int end = min(row_end, st_off[seg + 1]);
+        mask = start & (kVecLen - 1);
+        base = start - mask;
+        cnt = (end - start + mask) / kBlockItems * kBlockItems;
+    }
 
     const int ls = lane % LPR, group = lane / LPR;
     const int tile = blockIdx.y * TN;
@@ -136,13 +159,15 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
 
     for (int off = 0; off < cnt; off += kWave) {
         const int slot = off + lane;
-        const int live = min(cnt - off, kWave); // 64, or 32 on a trailing half step
+        const int live = min(cnt - off, kWave); // 64, or less on the last step
         int c = 0;
         A v = A(0);
-        if (lane < live) {
-            const bool head = slot < mask; // previous row's slots
-            c = col[base + (head ? mask : slot)];
-            v = head ? A(0) : val[base + slot];
+        if (lane < ((live + 3) & ~3)) {
+            // slots of the previous row (head) and slots past the end (last quad) are
+            // neutralised: value 0, column of a real slot
+            const bool head = slot < mask, past = slot >= cnt;
+            c = col[base + (head ? mask : (past ? cnt - 1 : slot))];
+            v = (head || past) ? A(0) : val[base + slot];
         }
         my_c[lane] = c;
         my_v[lane] = v;
@@ -150,7 +175,7 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
         if (live == kWave)
             spmm_gather<T, TN, 16 / G, true>(b_lane, (size_t)n, acc, my_c, my_v, group, G, 16);
         else
-            spmm_gather<T, TN, 16 / G, false>(b_lane, (size_t)n, acc, my_c, my_v, group, G, live / 4);
+            spmm_gather<T, TN, 16 / G, false>(b_lane, (size_t)n, acc, my_c, my_v, group, G, (live + 3) / 4);
         wave_lds_sync();
     }
 
@@ -168,7 +193,7 @@ spmm_block_kernel(int m1, int n, const int* __restrict__ block_rows, const int* 
 // group walks its row's slot quads one after the other, no cross-lane reduction.
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
+spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
                     const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
                     const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C)
 {
@@ -191,6 +216,7 @@ spmm_residue_kernel(int m2, int n, const int* __restrict__ residue_rows, const i
     int first = s, cnt = e - s;
     const bool accumulate = N >= kBlockItems; // the row also has block segments
     if (accumulate) {
+        if (N <= owned_slots) return; // summed entirely, tail included, by the block kernel
         first = (s - pad) + N / kBlockItems * kBlockItems;
         cnt = N % kBlockItems;
     }
@@ -260,14 +286,17 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
                   typename DenseVec<T>::Acc* C, hipStream_t s1, hipStream_t s2)
 {
     const int tiles = (n + TN - 1) / TN;
+    const int owned_slots = m1 >= kOwnedMinSegments ? kOwnedRowSlots : 0;
     if (m1 > 0) {
         dim3 grid(grid_for_waves(m1), tiles);
-        spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_rows, st_off, row_ptr, col, val, B, C);
+        spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, owned_slots, block_rows, st_off, row_ptr, col,
+                                                                    val, B, C);
     }
     if (m2 > 0) {
         constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
         dim3 grid(grid_for_waves(((long long)m2 + RPW - 1) / RPW), tiles);
-        spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, residue_rows, row_ptr, col, val, B, C);
+        spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, residue_rows, row_ptr, col, val,
+                                                                      B, C);
     }
     return hipGetLastError();
 }
