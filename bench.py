@@ -116,7 +116,9 @@ def main():
     setup_s = time.time() - t0
 
     stream = torch.cuda.current_stream().cuda_stream
-    spmm_fn = lib.rode_hip_spmm_f32 if args.dtype == "f32" else lib.rode_hip_spmm_f16
+    def spmm_fn(*a):  # the whole decomposition is passed, and the library is told so
+        return lib.rode_hip_spmm_ex(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS, *a)
+
     sddmm_fn = lib.rode_hip_sddmm_f32 if args.dtype == "f32" else lib.rode_hip_sddmm_f16
 
     main_stream = torch.cuda.current_stream()
@@ -216,7 +218,7 @@ def main():
     del p_blk, p_st, p_res, p_ws
     kernels = {}
     if csr.m1 > 0:
-        kernels["spmm_block"] = event_time(lambda: spmm(csr.m1, 0), reps)
+        kernels["spmm_block"] = event_time(lambda: spmm(csr.m1, 0), reps)  # incl. whole rows of 32..1024 slots
         kernels["sddmm_block"] = event_time(lambda: sddmm(csr.m1, 0), reps)
     if csr.m2 > 0:
         # The SpMM residue kernel skips the rows its block kernel sums whole, which only

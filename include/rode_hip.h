@@ -79,6 +79,25 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
                       void* stream2);
 
 /*
+ * SpMM with a promise.  dtype selects the element type of B (RODE_DENSE_F32: fp32 values
+ * and C; RODE_DENSE_F16: fp32 values and C, fp16 B; RODE_DENSE_F64: fp64 values, B, C);
+ * flags = 0 behaves exactly like the typed functions above.  RODE_SPMM_WHOLE_LISTS
+ * promises that row_indices1 / row_seg_st_offsets / row_indices2 are the COMPLETE
+ * decomposition of the matrix (not a slice of it): a row of 32..1024 aligned slots may
+ * then be summed - all its segments and its tail - by one wavefront with a single
+ * update of C instead of one atomic update per work item.  Same results; no counterpart
+ * in the reference.
+ */
+#define RODE_DENSE_F32 0
+#define RODE_DENSE_F16 1
+#define RODE_DENSE_F64 2
+#define RODE_SPMM_WHOLE_LISTS 1
+int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
+                     const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
+                     const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
+                     void* stream1, void* stream2);
+
+/*
  * Prepares an uninitialised C[M x n] for one of the SpMM calls: zeroes exactly the rows
  * that SpMM adds to (aligned length >= 32) or never touches (rows in no list) and
  * leaves alone the rows it stores.  A cheaper replacement for clearing all of C; the

@@ -21,12 +21,16 @@ SIGNATURES = {
     "rode_hip_spmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 10),
     "rode_hip_spmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 10),
     "rode_hip_spmm_f64": (c_int, [c_int] * 4 + [c_void_p] * 10),
+    "rode_hip_spmm_ex": (c_int, [c_int] * 6 + [c_void_p] * 10),
     "rode_hip_spmm_clear_rows": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "rode_hip_sddmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 11),
     "rode_hip_sddmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 11),
     "rode_hip_csr_softmax_f32": (c_int, [c_int, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p]),
     "rode_hip_csr_softmax_backward_f32": (c_int, [c_int] + [c_void_p] * 4 + [ctypes.c_float, c_void_p]),
 }
+
+DENSE_CODE = {"f32": 0, "f16": 1, "f64": 2}  # RODE_DENSE_* of include/rode_hip.h
+SPMM_WHOLE_LISTS = 1
 
 _lib = None
 

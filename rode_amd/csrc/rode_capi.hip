@@ -37,16 +37,40 @@ int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const i
                                    d_residue_r_ind, d_n_blk, d_n_res, d_workspace, capacity_blocks, as_stream(stream));
 }
 
+int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
+                     const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
+                     const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
+                     void* stream1, void* stream2)
+{
+    (void)k;
+    if (m1 < 0 || m2 < 0 || (flags & ~RODE_SPMM_WHOLE_LISTS)) return hipErrorInvalidValue;
+    if (m1 == 0 && m2 == 0) return hipSuccess;
+    if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
+    const bool whole = flags & RODE_SPMM_WHOLE_LISTS;
+    hipStream_t s1 = as_stream(stream1), s2 = as_stream(stream2);
+    switch (dtype) {
+    case RODE_DENSE_F32:
+        return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
+                                        d_column_indices, static_cast<const float*>(d_values),
+                                        static_cast<const float*>(d_B), static_cast<float*>(d_C), whole, s1, s2);
+    case RODE_DENSE_F16:
+        return rode::spmm_launch<__half>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets,
+                                         d_row_offsets, d_column_indices, static_cast<const float*>(d_values),
+                                         static_cast<const __half*>(d_B), static_cast<float*>(d_C), whole, s1, s2);
+    case RODE_DENSE_F64:
+        return rode::spmm_launch<double>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets,
+                                         d_row_offsets, d_column_indices, static_cast<const double*>(d_values),
+                                         static_cast<const double*>(d_B), static_cast<double*>(d_C), whole, s1, s2);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
                       const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
                       const int* d_row_seg_st_offsets, const float* d_B, float* d_C, void* stream1, void* stream2)
 {
-    (void)k;
-    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
-    if (m1 == 0 && m2 == 0) return hipSuccess;
-    if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
-    return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
-                                    d_column_indices, d_values, d_B, d_C, as_stream(stream1), as_stream(stream2));
+    return rode_hip_spmm_ex(RODE_DENSE_F32, 0, m1, m2, k, n, d_values, d_column_indices, d_row_offsets, d_row_indices1,
+                            d_row_indices2, d_row_seg_st_offsets, d_B, d_C, stream1, stream2);
 }
 
 int rode_hip_spmm_clear_rows(int M, int n, int elem_bytes, const int* d_row_offsets, void* d_C, void* stream)
@@ -62,12 +86,8 @@ int rode_hip_spmm_f64(int m1, int m2, int k, int n, const double* d_values, cons
                       const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
                       const int* d_row_seg_st_offsets, const double* d_B, double* d_C, void* stream1, void* stream2)
 {
-    (void)k;
-    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
-    if (m1 == 0 && m2 == 0) return hipSuccess;
-    if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
-    return rode::spmm_launch<double>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
-                                     d_column_indices, d_values, d_B, d_C, as_stream(stream1), as_stream(stream2));
+    return rode_hip_spmm_ex(RODE_DENSE_F64, 0, m1, m2, k, n, d_values, d_column_indices, d_row_offsets, d_row_indices1,
+                            d_row_indices2, d_row_seg_st_offsets, d_B, d_C, stream1, stream2);
 }
 
 int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
@@ -75,13 +95,8 @@ int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const
                       const int* d_row_seg_st_offsets, const void* d_B_half, float* d_C, void* stream1,
                       void* stream2)
 {
-    (void)k;
-    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
-    if (m1 == 0 && m2 == 0) return hipSuccess;
-    if (!aligned16(d_B_half) || !aligned16(d_C)) return hipErrorInvalidValue;
-    return rode::spmm_launch<__half>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
-                                     d_column_indices, d_values, static_cast<const __half*>(d_B_half), d_C,
-                                     as_stream(stream1), as_stream(stream2));
+    return rode_hip_spmm_ex(RODE_DENSE_F16, 0, m1, m2, k, n, d_values, d_column_indices, d_row_offsets, d_row_indices1,
+                            d_row_indices2, d_row_seg_st_offsets, d_B_half, d_C, stream1, stream2);
 }
 
 int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,

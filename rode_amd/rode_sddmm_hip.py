@@ -135,13 +135,14 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
 
 
 def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, k,
-                 dense_matrix, out=None):
+                 dense_matrix, out=None, whole_lists=True):
     """C = A_csr @ dense_matrix through ``rode_hip_spmm_f32`` / ``_f16``
     (host API ``RoDe_SpMM/RoDeSpmm.h:4-8``).  ``dense_matrix`` is (k, n) with n a
     multiple of 4 (8 for fp16, 2 for fp64), fp32 / fp16 (fp32 ``values``) or fp64 (fp64 ``values``); the
     result is a new zero-initialised (m, n) tensor of the dtype of ``values``, or
     ``out`` accumulated in place the way the reference kernels do (long rows add,
-    short rows overwrite)."""
+    short rows overwrite).  ``whole_lists`` promises that the index tensors are the
+    complete decomposition (always true for a ``RoDeCSR``); pass False for a slice."""
     for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
                     (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
                     (values, "values"), (dense_matrix, "dense_matrix")):
@@ -174,12 +175,12 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
         _check(out.dtype == out_dtype and tuple(out.shape) == (m, n), f"out must be {out_dtype} of shape (m, n)")
     if m1 == 0 and m2 == 0:
         return out
-    fn = {torch.float32: lib.rode_hip_spmm_f32, torch.float16: lib.rode_hip_spmm_f16,
-          torch.float64: lib.rode_hip_spmm_f64}[dense_matrix.dtype]
+    dtype = {torch.float32: 0, torch.float16: 1, torch.float64: 2}[dense_matrix.dtype]  # RODE_DENSE_*
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
-        code = fn(m1, m2, k, n, values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
-                  block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
-                  dense_matrix.data_ptr(), out.data_ptr(), s, s)
-    _lib.check(code, "rode_hip_spmm")
+        code = lib.rode_hip_spmm_ex(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
+                                    values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
+                                    block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
+                                    dense_matrix.data_ptr(), out.data_ptr(), s, s)
+    _lib.check(code, "rode_hip_spmm_ex")
     return out

@@ -382,3 +382,46 @@ def test_clear_rows_prepares_exactly_what_spmm_does_not_overwrite():
     assert (C64[torch.from_numpy(cleared).to(DEV)] == 0).all()
     assert lib.rode_hip_spmm_clear_rows(m, 6, 4, csr.row_offsets.data_ptr(), C64.data_ptr(), None) != 0  # 24-byte rows
     assert lib.rode_hip_spmm_clear_rows(m, 8, 2, csr.row_offsets.data_ptr(), C64.data_ptr(), None) != 0
+
+
+@pytest.mark.parametrize("seg,half", [(32, False), (512, False), (512, True)])
+def test_whole_row_mode_and_split_calls(seg, half):
+    """With >= 16384 block segments and the whole-lists promise (what the Python op
+    passes), rows of 32..1024 slots are summed by one wave, tail included; rows just
+    outside that range, unaligned starts and empty rows sit next to them here.  The
+    typed entry points make no such promise: a caller who feeds the two lists in
+    separate calls, or the block list in two halves, must get the same matrix."""
+    import oracle
+    from gpu_common import DEV, TOL_F16, TOL_F32, make_csr, round_half, run_spmm
+    from helpers import spmm_row_l1_error
+    from rode_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(seg)
+    m, k, n = 24000, 3000, 64
+    lens = rng.choice([0, 1, 5, 31, 32, 33, 63, 64, 100, 500, 1000, 1020, 1021, 1024, 1025, 1056, 1500], size=m,
+                      p=[.05, .05, .1, .05, .05, .05, .05, .05, .2, .1, .05, .03, .03, .03, .03, .03, .05])
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(k, size=l, replace=False)) for l in lens]).astype(np.int32)
+    val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    csr = make_csr(rp, col, val, m, k, 32, seg)
+    assert csr.m1 >= 16384
+    ref = oracle.spmm_f64(rp, col, val, round_half(B) if half else B)
+    tol = TOL_F16 if half else TOL_F32
+    assert spmm_row_l1_error(run_spmm(csr, B, half), ref) <= tol
+    if half:
+        return
+    dB = torch.from_numpy(B).to(DEV)
+
+    def typed(m1, m2, blk_ptr, st_ptr, C):
+        _lib.check(lib.rode_hip_spmm_f32(m1, m2, k, n, csr.values.data_ptr(), csr.column_indices.data_ptr(),
+                                         csr.row_offsets.data_ptr(), blk_ptr, csr.residue_indices.data_ptr(), st_ptr,
+                                         dB.data_ptr(), C.data_ptr(), None, None), "spmm")
+
+    C = torch.zeros(m, n, device=DEV)
+    half_m1 = csr.m1 // 2  # very likely inside a row
+    typed(half_m1, 0, csr.block_indices.data_ptr(), csr.st_offsets.data_ptr(), C)
+    typed(csr.m1 - half_m1, 0, csr.block_indices.data_ptr() + 4 * half_m1, csr.st_offsets.data_ptr() + 4 * half_m1, C)
+    typed(0, csr.m2, csr.block_indices.data_ptr(), csr.st_offsets.data_ptr(), C)
+    torch.cuda.synchronize()
+    assert spmm_row_l1_error(C.cpu().numpy(), ref) <= tol
