@@ -257,6 +257,8 @@ spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ resi
     }
 }
 
+constexpr int kClearRowsPerGroup = 8;
+
 // Zeroes exactly the rows of C that the two SpMM kernels do not overwrite: rows whose
 // aligned length N = len + (start & 3) is >= 32 are accumulated into, rows with N == 0
 // belong to no work item; rows with 0 < N < 32 are stored by the residue kernel and
@@ -264,15 +266,25 @@ spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ resi
 __global__ void __launch_bounds__(kWgThreads)
 spmm_clear_rows_kernel(int M, size_t row_bytes, const int* __restrict__ row_ptr, char* __restrict__ C)
 {
-    constexpr int kLanes = 16, kRowsPerWg = kWgThreads / kLanes;
-    const int row = xcd_logical_block(blockIdx.x, gridDim.x) * kRowsPerWg + threadIdx.x / kLanes;
-    if (row >= M) return;
-    const int s = row_ptr[row], e = row_ptr[row + 1];
-    const int N = e - s + (s & (kVecLen - 1));
-    if (N > 0 && N < kBlockItems) return;
-    char* dst = C + (size_t)row * row_bytes;
-    for (size_t b = (threadIdx.x % kLanes) * 16; b < row_bytes; b += kLanes * 16)
-        *reinterpret_cast<uint4*>(dst + b) = make_uint4(0, 0, 0, 0);
+    constexpr int kLanes = 16, kGroups = kWgThreads / kLanes;
+    const int group = threadIdx.x / kLanes, lane = threadIdx.x % kLanes;
+    const int first = xcd_logical_block(blockIdx.x, gridDim.x) * (kGroups * kClearRowsPerGroup);
+    // batch b of a workgroup covers kGroups consecutive rows, one per lane group
+    int s[kClearRowsPerGroup], e[kClearRowsPerGroup];
+#pragma unroll
+    for (int b = 0; b < kClearRowsPerGroup; ++b) {
+        const int row = first + b * kGroups + group;
+        s[b] = row < M ? row_ptr[row] : 1;
+        e[b] = row < M ? row_ptr[row + 1] : 2; // N = 2: a row that is left alone
+    }
+#pragma unroll
+    for (int b = 0; b < kClearRowsPerGroup; ++b) {
+        const int N = e[b] - s[b] + (s[b] & (kVecLen - 1));
+        if (N > 0 && N < kBlockItems) continue;
+        char* dst = C + (size_t)(first + b * kGroups + group) * row_bytes;
+        for (size_t off = lane * 16; off < row_bytes; off += kLanes * 16)
+            *reinterpret_cast<uint4*>(dst + off) = make_uint4(0, 0, 0, 0);
+    }
 }
 
 inline int grid_for_waves(long long nwaves)
@@ -346,7 +358,8 @@ hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* 
 hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, void* C, hipStream_t stream)
 {
     if (M <= 0) return hipSuccess;
-    long long wgs = ((long long)M + 15) / 16;
+    constexpr int kRowsPerWg = kWgThreads / 16 * kClearRowsPerGroup;
+    long long wgs = ((long long)M + kRowsPerWg - 1) / kRowsPerWg;
     wgs = (wgs + kXcds - 1) / kXcds * kXcds;
     spmm_clear_rows_kernel<<<(int)wgs, kWgThreads, 0, stream>>>(M, row_bytes, row_ptr, static_cast<char*>(C));
     return hipGetLastError();
