@@ -230,7 +230,9 @@ inline int grid_for_waves(long long nwaves)
 {
     long long wgs = (nwaves + kWavesPerWg - 1) / kWavesPerWg;
     wgs = (wgs + kXcds - 1) / kXcds * kXcds; // xcd_logical_block needs a multiple of kXcds
-    return (int)wgs;
+    // a launch dimension holds fewer than 2^32 threads; more work items than that (over
+    // 16 M workgroups) are refused instead of being launched wrongly
+    return wgs * kWgThreads < (1ll << 32) ? (int)wgs : -1;
 }
 
 template <typename T, int KT, int NS, bool EDGE>
@@ -238,13 +240,15 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
                   const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
                   hipStream_t s1, hipStream_t s2)
 {
+    constexpr int RPW = kWave / SddmmShape<T, KT>::kLpr;
+    const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
+    if (g1 < 0 || g2 < 0) return hipErrorInvalidConfiguration;
     if (m1 > 0) {
-        sddmm_block_kernel<T, KT, NS, EDGE><<<grid_for_waves(m1), kWgThreads, 0, s1>>>(
+        sddmm_block_kernel<T, KT, NS, EDGE><<<g1, kWgThreads, 0, s1>>>(
             m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
     }
     if (m2 > 0) {
-        constexpr int RPW = kWave / SddmmShape<T, KT>::kLpr;
-        sddmm_residue_kernel<T, KT, NS, EDGE><<<grid_for_waves(((long long)m2 + RPW - 1) / RPW), kWgThreads, 0, s2>>>(
+        sddmm_residue_kernel<T, KT, NS, EDGE><<<g2, kWgThreads, 0, s2>>>(
             m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out);
     }
     return hipGetLastError();

@@ -58,13 +58,15 @@ csr_softmax_backward_kernel(int M, const int* __restrict__ row_ptr, const float*
 inline int grid_for_rows(int M)
 {
     long long wgs = ((long long)M + kWavesPerWg - 1) / kWavesPerWg;
-    return (int)((wgs + kXcds - 1) / kXcds * kXcds);
+    wgs = (wgs + kXcds - 1) / kXcds * kXcds;
+    return wgs * kWgThreads < (1ll << 32) ? (int)wgs : -1; // a launch dimension holds fewer than 2^32 threads
 }
 
 } // namespace
 
 hipError_t csr_softmax_launch(int M, const int* row_ptr, const float* in, float* out, float scale, hipStream_t stream)
 {
+    if (grid_for_rows(M) < 0) return hipErrorInvalidConfiguration;
     if (M > 0) csr_softmax_kernel<<<grid_for_rows(M), kWgThreads, 0, stream>>>(M, row_ptr, in, out, scale);
     return hipGetLastError();
 }
@@ -72,6 +74,7 @@ hipError_t csr_softmax_launch(int M, const int* row_ptr, const float* in, float*
 hipError_t csr_softmax_backward_launch(int M, const int* row_ptr, const float* p, const float* dp, float* ds,
                                        float scale, hipStream_t stream)
 {
+    if (grid_for_rows(M) < 0) return hipErrorInvalidConfiguration;
     if (M > 0) csr_softmax_backward_kernel<<<grid_for_rows(M), kWgThreads, 0, stream>>>(M, row_ptr, p, dp, ds, scale);
     return hipGetLastError();
 }

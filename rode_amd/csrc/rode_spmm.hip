@@ -291,7 +291,9 @@ inline int grid_for_waves(long long nwaves)
 {
     long long wgs = (nwaves + kWavesPerWg - 1) / kWavesPerWg;
     wgs = (wgs + kXcds - 1) / kXcds * kXcds; // xcd_logical_block needs a multiple of kXcds
-    return (int)wgs;
+    // a launch dimension holds fewer than 2^32 threads; more work items than that (over
+    // 16 M workgroups) are refused instead of being launched wrongly
+    return wgs * kWgThreads < (1ll << 32) ? (int)wgs : -1;
 }
 
 template <typename T, int TN, bool EDGE>
@@ -301,14 +303,16 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
 {
     const int tiles = (n + TN - 1) / TN;
     const int owned_slots = whole_lists && m1 >= kOwnedMinSegments ? kOwnedRowSlots : 0;
+    constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
+    const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
+    if (g1 < 0 || g2 < 0 || tiles > 65535) return hipErrorInvalidConfiguration;
     if (m1 > 0) {
-        dim3 grid(grid_for_waves(m1), tiles);
+        dim3 grid(g1, tiles);
         spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, owned_slots, block_rows, st_off, row_ptr, col,
                                                                     val, B, C);
     }
     if (m2 > 0) {
-        constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
-        dim3 grid(grid_for_waves(((long long)m2 + RPW - 1) / RPW), tiles);
+        dim3 grid(g2, tiles);
         spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, residue_rows, row_ptr, col, val,
                                                                       B, C);
     }
@@ -361,6 +365,7 @@ hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, v
     constexpr int kRowsPerWg = kWgThreads / 16 * kClearRowsPerGroup;
     long long wgs = ((long long)M + kRowsPerWg - 1) / kRowsPerWg;
     wgs = (wgs + kXcds - 1) / kXcds * kXcds;
+    if (wgs * kWgThreads >= (1ll << 32)) return hipErrorInvalidConfiguration;
     spmm_clear_rows_kernel<<<(int)wgs, kWgThreads, 0, stream>>>(M, row_bytes, row_ptr, static_cast<char*>(C));
     return hipGetLastError();
 }
