@@ -4,16 +4,17 @@
 // (RoDe_SDDMM/RoDeSddmm.cu:15-203) and SDDMMKernel4Residue (:206-494); the
 // execution shape is written for 64-lane wavefronts:
 //
-//   * a "unit" is 32 consecutive nonzero slots handled by one 32-lane half of a
-//     wave: lane e of the half owns slot e (its column index, its value, its
-//     output), so sparse loads and the final store are fully coalesced;
-//   * inside a half, groups of LPR = K / (elements per 128-bit load) lanes read
-//     one dense rhs row per load instruction, LPR rows per group per unit;
+//   * block kernel: a "unit" is 32 consecutive nonzero slots handled by one 32-lane
+//     half of a wave: lane e of the half owns slot e (its column index, its value,
+//     its output), so sparse loads and the final store are fully coalesced;
+//   * inside a half, groups of LPR = KT / (elements per 128-bit load) lanes read one
+//     dense rhs row (KT = 32, 64 or 128 elements of it at a time; K up to 4 such
+//     slabs) per load instruction, LPR rows per group per unit;
 //   * the K-slices of four rows at a time are combined with a transpose-reduce
 //     (DPP quad_perm for xor 1/2, ds_swizzle for xor 4/8/16) that leaves the dot
 //     product of slot e in lane e;
-//   * block kernel: one wave walks one block segment, 64 slots per step, the
-//     lhs row slice stays in registers for the whole segment;
+//   * one wave walks one block segment, 64 slots per step, the lhs row slice stays
+//     in registers for the whole segment;
 //   * residue kernel: each group of LPR lanes takes one residue row (< 32 slots),
 //     so a wave works on 64 / LPR rows at once (2 at K=128 fp32, 8 at K=32):
 //     short rows are latency-bound and need many rows in flight per wave.
