@@ -44,6 +44,11 @@ class RoDeCSR:
         self.nnz = values.numel()
         self.device = torch.device(device)
         self.config = dict(config) if config is not None else dict(self.CONFIGS.get(k, self.DEFAULT_CONFIG))
+        cfg = self.config
+        if cfg.get("k_block") != 32 or cfg.get("vec_len") != 4 or cfg.get("seg_length", 0) <= 0 \
+                or cfg["seg_length"] % 32 != 0:
+            # the kernels process 32-slot chunks from 4-aligned offsets, as the reference's do
+            raise ValueError(f"config must have k_block=32, vec_len=4 and seg_length a positive multiple of 32, got {cfg}")
 
         self.row_offsets_cpu = row_offsets.to(dtype=torch.int32, device="cpu").contiguous()
         self.column_indices = column_indices.to(dtype=torch.int32, device=self.device).contiguous()

@@ -21,6 +21,10 @@ def test_errors_raised_before_any_device_work():
         RoDeCSR(rp, torch.zeros(4, dtype=torch.int32), torch.zeros(4), "cpu", 2, 4, k=50)
     with pytest.raises(ValueError, match="k must be"):
         RoDeCSR(rp, torch.zeros(4, dtype=torch.int32), torch.zeros(4), "cpu", 2, 4, k=1024)
+    for bad in ({"seg_length": 48, "k_block": 32, "vec_len": 4}, {"seg_length": 512, "k_block": 16, "vec_len": 4},
+                {"seg_length": 512, "k_block": 32, "vec_len": 2}, {"seg_length": 0, "k_block": 32, "vec_len": 4}):
+        with pytest.raises(ValueError, match="config must have"):
+            RoDeCSR(rp, torch.zeros(4, dtype=torch.int32), torch.zeros(4), "cpu", 2, 4, k=32, config=bad)
     with pytest.raises(RuntimeError, match="int32"):
         rode_sddmm_hip.preprocess(rp.long(), 4, 512, 32, 4)
     with pytest.raises(RuntimeError, match="CUDA tensor"):
