@@ -308,6 +308,9 @@ def main():
         good = np.add.reduceat(scale, starts) / row_l1 <= 100.0
         sddmm_err = float(row_err[good].max(initial=0.0))
         sddmm_strict = float(np.max(np.abs(o_gpu - o64) / np.maximum(scale, 1e-30)))
+        # the reference tests' own rule against its fp32 CPU loop: abs AND rel error above 1e-3
+        diff = np.abs(o_gpu - o_ref)
+        ref_rule_errors = int(((diff > 1e-3) & (diff / (np.abs(o_ref) + 1e-6) > 1e-3)).sum())
         # GPU row decomposition against the CPU routine, for the segment length in use and for
         # both parameter sets of the reference, (512,32,4) and (32,32,4); the CPU time is reported
         bit_exact, t_pre = True, 0.0
@@ -331,6 +334,7 @@ def main():
                              "value": round(2 * (2.0 * cnt * k) / (mt_spmm + mt_sddmm) / 1e9, 3)},
                "parity_vs_gpu": {"spmm_rowL1_err": spmm_err, "sddmm_rowL1_err_cond_le_100": sddmm_err,
                                  "sddmm_err_over_term_magnitude": sddmm_strict,
+                                 "sddmm_reference_rule_errors": ref_rule_errors,
                                  "preprocess_bit_exact": bool(bit_exact)}}
 
     line = {
