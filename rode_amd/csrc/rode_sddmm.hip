@@ -109,6 +109,8 @@ __device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int ro
     }
 }
 
+constexpr int kMergeSlots = 128;
+
 // One wave per block segment.  Segment s covers the aligned slots
 // [base, base + cnt) with base = st_off[s] & ~3 and cnt = floor((len + mask) / 32) * 32
 // (RoDeSddmm.cu:35-54); the first `mask` slots belong to the previous row and are
@@ -125,12 +127,29 @@ sddmm_block_kernel(int m1, int k, const int* __restrict__ block_rows, const int*
     const int seg = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (seg >= m1) return;
 
+    // Consecutive segments of one row whose starts fall into the same window of
+    // kMergeSlots slots are handled by the wave of the first of them, so a decomposition
+    // with short segments (32 in the reference's K=128 parameter set) still fills whole
+    // 64-slot steps and loads the lhs row once.  Segments of kMergeSlots or more are
+    // unaffected.  (Outputs are pure functions of the inputs, so this is safe even when a
+    // caller passes a slice of the lists: the worst case is an output computed twice.)
     const int row = block_rows[seg];
     const int start = st_off[seg];
-    const int end = min(row_ptr[row + 1], st_off[seg + 1]);
+    const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
+    const int row_base = row_start - (row_start & (kVecLen - 1));
+    const int window = (start - row_base) / kMergeSlots;
+    if (seg > 0 && block_rows[seg - 1] == row && (st_off[seg - 1] - row_base) / kMergeSlots == window) return;
+    const int probe = seg + 1 + lane; // the next leader: first later segment of another row or window
+    const bool follower = probe < m1 && block_rows[probe] == row && (st_off[probe] - row_base) / kMergeSlots == window;
+    const unsigned long long not_follower = ~__ballot(follower);
+    const int next = seg + 1 + (not_follower ? __builtin_ctzll(not_follower) : kWave);
+    // end of the row's block part, or the start of the next leader if that comes first
+    // (st_off[m1] exists: the sentinel, or the next segment when the lists are a slice)
+    const int block_end = row_base + (row_end - row_base) / kBlockItems * kBlockItems;
+    const int end = min(block_end, st_off[next]);
     const int mask = start & (kVecLen - 1);
     const int base = start - mask;
-    const int cnt = (end - start + mask) / kBlockItems * kBlockItems;
+    const int cnt = end - base;
 
     float a[NS][S::kVec];
     load_lhs_slice<T, KT, NS, EDGE>(lhs, row, k, lane, a);

@@ -43,6 +43,7 @@ namespace {
 // atomics).
 constexpr int kOwnedRowSlots = 1024;
 constexpr int kOwnedMinSegments = 16384;
+constexpr int kMergeSlots = 512; // under the same promise, short segments of a longer row are merged up to this many slots
 
 template <typename T, int TN>
 struct SpmmShape {
@@ -138,6 +139,27 @@ spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_
         mask = row_start & (kVecLen - 1);
         base = row_start - mask;
         cnt = row_end - base;
+    } else if (owned_slots > 0) {
+        // Long row, complete lists: consecutive segments of the row whose starts fall into the
+        // same window of kMergeSlots slots are summed by the wave of the first of them (the
+        // "leader"), so a decomposition with short segments (the reference's 32) does not
+        // multiply the atomic updates of C.  With segments of kMergeSlots or more every
+        // segment is its own leader and nothing changes.
+        const int start = st_off[seg];
+        const int row_base = row_start - (row_start & (kVecLen - 1));
+        const int window = (start - row_base) / kMergeSlots;
+        if (seg > 0 && block_rows[seg - 1] == row && (st_off[seg - 1] - row_base) / kMergeSlots == window) return;
+        // the next leader is the first later segment of another row or another window
+        const int probe = seg + 1 + lane;
+        const bool follower = probe < m1 && block_rows[probe] == row && (st_off[probe] - row_base) / kMergeSlots == window;
+        const unsigned long long not_follower = ~__ballot(follower); // 64 lanes cover kMergeSlots / 32 = 16 segments
+        const int followers = not_follower ? __builtin_ctzll(not_follower) : kWave;
+        const int next = seg + 1 + followers;
+        const int block_end = row_base + (row_end - row_base) / kBlockItems * kBlockItems; // end of the row's block part
+        const int end = min(block_end, st_off[next]); // another row's start (or the sentinel) lies past block_end
+        mask = start & (kVecLen - 1);
+        base = start - mask;
+        cnt = end - base;
     } else {
         const int start = st_off[seg];
         const int end = min(row_end, st_off[seg + 1]);
