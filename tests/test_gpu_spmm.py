@@ -384,7 +384,7 @@ def test_clear_rows_prepares_exactly_what_spmm_does_not_overwrite():
     assert lib.rode_hip_spmm_clear_rows(m, 8, 2, csr.row_offsets.data_ptr(), C64.data_ptr(), None) != 0
 
 
-@pytest.mark.parametrize("seg,half", [(32, False), (512, False), (512, True)])
+@pytest.mark.parametrize("seg,half", [(32, False), (96, False), (512, False), (512, True), (160, True)])
 def test_whole_row_mode_and_split_calls(seg, half):
     """With >= 16384 block segments and the whole-lists promise (what the Python op
     passes), rows of 32..1024 slots are summed by one wave, tail included; rows just
@@ -400,6 +400,7 @@ def test_whole_row_mode_and_split_calls(seg, half):
     m, k, n = 24000, 3000, 64
     lens = rng.choice([0, 1, 5, 31, 32, 33, 63, 64, 100, 500, 1000, 1020, 1021, 1024, 1025, 1056, 1500], size=m,
                       p=[.05, .05, .1, .05, .05, .05, .05, .05, .2, .1, .05, .03, .03, .03, .03, .03, .05])
+    lens[::4000] = [2999, 2500, 2048, 1999, 2990, 1600]  # several merge windows per row (k = 3000 columns)
     rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     col = np.concatenate([np.sort(rng.choice(k, size=l, replace=False)) for l in lens]).astype(np.int32)
     val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
