@@ -413,6 +413,12 @@ def test_whole_row_mode_and_split_calls(seg, half):
     if half:
         return
     dB = torch.from_numpy(B).to(DEV)
+    if seg == 96:  # the fp64 instantiation through the same promise
+        from rode_amd import rode_sddmm_hip
+        C64 = rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                          csr.row_offsets, csr.column_indices, csr.values.double(), m, k,
+                                          dB.double()).cpu().numpy()
+        assert spmm_row_l1_error(C64, ref) <= 1e-12
 
     def typed(m1, m2, blk_ptr, st_ptr, C):
         _lib.check(lib.rode_hip_spmm_f32(m1, m2, k, n, csr.values.data_ptr(), csr.column_indices.data_ptr(),
