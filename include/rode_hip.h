@@ -62,6 +62,26 @@ int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const i
                         int capacity_blocks, void* d_workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * rode_hip_preprocess() without a workspace argument and without any allocation, for
+ * callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its GPU
+ * routine allocates and frees CUB scratch on every call, _preprocess.cu:331-335).
+ * Same arguments, same kernels and byte-identical results; the scan scratch is a fixed
+ * array inside the library (16.1 MiB of device memory per GPU, held until the process
+ * ends), so M is limited to RODE_HIP_STATIC_MAX_ROWS: a larger M returns
+ * hipErrorOutOfMemory (2) before anything is launched.  The first call on a device looks
+ * up the array's address (no allocation; make that call outside stream capture).  Every
+ * call on one GPU uses that GPU's one array: calls that overlap in time on the same GPU
+ * (different streams or host threads) race; calls queued on one stream do not.  Nothing in
+ * the array has to be cleared between calls: every entry a call reads was written by
+ * the same call.
+ */
+#define RODE_HIP_STATIC_MAX_ROWS 4194304
+int rode_hip_preprocess_static(int seg_length, int k_block, int vec_len, int M, const int* d_row_ptr,
+                               int* d_block_r_ind, int* d_st_off, int* d_residue_r_ind, int* d_n_blk, int* d_n_res,
+                               int capacity_blocks, void* stream);
+
+/*
  * SpMM  C[M x n] += A_csr[M x k] * B[k x n]  (fp32 values, fp32 or fp16 dense B,
  * fp32 accumulate and output).
  * Replaces RoDeSpmm_n32 / RoDeSpmm_n128 (fp32), RoDe_SpMM/RoDeSpmm.h:4-8,

@@ -18,6 +18,7 @@ SIGNATURES = {
     "rode_hip_error_string": (ctypes.c_char_p, [c_int]),
     "rode_hip_preprocess_workspace_bytes": (c_size_t, [c_int]),
     "rode_hip_preprocess": (c_int, [c_int] * 4 + [c_void_p] * 6 + [c_int, c_void_p, c_size_t, c_void_p]),
+    "rode_hip_preprocess_static": (c_int, [c_int] * 4 + [c_void_p] * 6 + [c_int, c_void_p]),
     "rode_hip_spmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 10),
     "rode_hip_spmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 10),
     "rode_hip_spmm_f64": (c_int, [c_int] * 4 + [c_void_p] * 10),

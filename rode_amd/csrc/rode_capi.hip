@@ -8,6 +8,8 @@
 
 #include <cstdio>
 
+static_assert(RODE_HIP_STATIC_MAX_ROWS == rode::kPreprocessStaticMaxRows, "header and library disagree");
+
 namespace {
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
@@ -35,6 +37,21 @@ int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const i
         return hipErrorInvalidValue;
     return rode::preprocess_launch(seg_length, k_block, vec_len, M, d_row_ptr, d_block_r_ind, d_st_off,
                                    d_residue_r_ind, d_n_blk, d_n_res, d_workspace, capacity_blocks, as_stream(stream));
+}
+
+int rode_hip_preprocess_static(int seg_length, int k_block, int vec_len, int M, const int* d_row_ptr,
+                               int* d_block_r_ind, int* d_st_off, int* d_residue_r_ind, int* d_n_blk, int* d_n_res,
+                               int capacity_blocks, void* stream)
+{
+    if (seg_length <= 0 || k_block <= 0 || vec_len <= 0 || M < 0 || capacity_blocks < 0) return hipErrorInvalidValue;
+    if (!d_row_ptr || !d_block_r_ind || !d_st_off || !d_residue_r_ind || !d_n_blk || !d_n_res)
+        return hipErrorInvalidValue;
+    if (M > RODE_HIP_STATIC_MAX_ROWS) return hipErrorOutOfMemory; // the fixed scratch cannot hold the scan of more rows
+    void* ws = nullptr;
+    const hipError_t e = rode::preprocess_static_workspace(&ws);
+    if (e != hipSuccess) return e;
+    return rode::preprocess_launch(seg_length, k_block, vec_len, M, d_row_ptr, d_block_r_ind, d_st_off,
+                                   d_residue_r_ind, d_n_blk, d_n_res, ws, capacity_blocks, as_stream(stream));
 }
 
 int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,

@@ -8,6 +8,11 @@ namespace rode {
 
 size_t preprocess_workspace_bytes(int M);
 
+// Largest matrix the allocation-free preprocessing entry point takes (RODE_HIP_STATIC_MAX_ROWS).
+constexpr int kPreprocessStaticMaxRows = 4 * 1024 * 1024;
+// Device address of the current GPU's static preprocessing scratch.
+hipError_t preprocess_static_workspace(void** ptr);
+
 hipError_t preprocess_launch(int seg, int kblock, int veclen, int M, const int* row_ptr, int* block_r_ind,
                              int* st_off, int* residue_r_ind, int* n_blk, int* n_res, void* workspace,
                              int capacity_blocks, hipStream_t stream);

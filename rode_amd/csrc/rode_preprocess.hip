@@ -12,12 +12,26 @@
 #include "rode_device.hpp"
 #include "rode_internal.hpp"
 
+#include <mutex>
+
 namespace rode {
 
 namespace {
 
 constexpr int kRowsPerThread = 4;
 constexpr int kTileRows = kWgThreads * kRowsPerThread; // rows scanned by one workgroup
+
+// Scratch layout: [tile_sum | tile_prefix | row_blk_prefix], the 8-byte arrays first.
+constexpr size_t workspace_bytes_for(size_t rows)
+{
+    return (2 * ((rows + kTileRows - 1) / kTileRows) + 2) * sizeof(unsigned long long) + (rows + 2) * sizeof(int);
+}
+
+// Scratch of the allocation-free entry point: one copy per GPU, held until the process
+// ends (16.1 MiB).  In host code this name is only a handle for hipGetSymbolAddress; the
+// kernels receive the address that call returns.
+constexpr size_t kStaticScratchBytes = (workspace_bytes_for(kPreprocessStaticMaxRows) + 255) / 256 * 256;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // Per-row counts in closed form.  With p = s % vec_len and N = len + p the
 // sequential routine peels t = (N-1)/seg whole segments until 1 <= N' <= seg is
@@ -159,11 +173,28 @@ fill_segments_kernel(int seg, int veclen, int M, int capacity, const int* __rest
 
 } // namespace
 
-size_t preprocess_workspace_bytes(int M)
+size_t preprocess_workspace_bytes(int M) { return workspace_bytes_for((size_t)(M > 0 ? M : 0)); }
+
+// Device address of this GPU's copy of `scratch`, looked up once per device.
+hipError_t preprocess_static_workspace(void** ptr)
 {
-    const size_t ntiles = ((size_t)(M > 0 ? M : 0) + kTileRows - 1) / kTileRows;
-    // [tile_sum | tile_prefix | row_blk_prefix], 8-byte arrays first
-    return (2 * ntiles + 2) * sizeof(unsigned long long) + ((size_t)(M > 0 ? M : 0) + 2) * sizeof(int);
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* per_device[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!per_device[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        per_device[dev] = p;
+    }
+    *ptr = per_device[dev];
+    return hipSuccess;
 }
 
 hipError_t preprocess_launch(int seg, int kblock, int veclen, int M, const int* row_ptr, int* block_r_ind,

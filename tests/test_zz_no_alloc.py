@@ -1,0 +1,62 @@
+"""The allocation-free preprocessing entry point (rode_hip_preprocess_static) against
+rode_hip_preprocess with a caller workspace: byte-identical arrays and counts, on two
+calls in a row, the second on a smaller matrix (the fixed scratch keeps the first call's
+contents)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(lib, entry, rp, seg, dev):
+    m = len(rp) - 1
+    nnz = int(rp[-1])
+    cap = (nnz + 3 * m) // seg + m
+    d_rp = torch.from_numpy(rp).to(dev)
+    blk = torch.full((cap + 1,), -1, dtype=torch.int32, device=dev)
+    st = torch.full((cap + 2,), -1, dtype=torch.int32, device=dev)
+    res = torch.full((max(m, 1),), -1, dtype=torch.int32, device=dev)
+    cnt = torch.full((2,), -1, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    if entry == "static":
+        code = lib.rode_hip_preprocess_static(seg, 32, 4, m, d_rp.data_ptr(), blk.data_ptr(), st.data_ptr(),
+                                              res.data_ptr(), cnt.data_ptr(), cnt.data_ptr() + 4, cap, stream)
+    else:
+        nbytes = lib.rode_hip_preprocess_workspace_bytes(m)
+        ws = torch.empty((nbytes + 7) // 8, dtype=torch.int64, device=dev)
+        code = lib.rode_hip_preprocess(seg, 32, 4, m, d_rp.data_ptr(), blk.data_ptr(), st.data_ptr(), res.data_ptr(),
+                                       cnt.data_ptr(), cnt.data_ptr() + 4, cap, ws.data_ptr(), nbytes, stream)
+    assert code == 0, (entry, code)
+    torch.cuda.synchronize()
+    return blk.cpu().numpy(), st.cpu().numpy(), res.cpu().numpy(), cnt.cpu().numpy()
+
+
+def test_static_scratch_entry_point_matches_workspace_entry_point():
+    from helpers import random_row_ptr
+    from rode_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(11)
+    big = random_row_ptr(rng, 700_000, 9, long_rows=30, long_len=60_000)
+    small = random_row_ptr(rng, 5_000, 40, long_rows=3, long_len=4_000) + 2  # unaligned starts
+    for rp, seg in ((big, 512), (small, 32), (big, 32), (np.zeros(1, np.int32), 512)):
+        print("static preprocessing: rows", len(rp) - 1, "nnz", int(rp[-1]), "seg", seg, flush=True)
+        want = _run(lib, "workspace", rp, seg, dev)
+        got = _run(lib, "static", rp, seg, dev)
+        for a, b, name in zip(got, want, ("block_r_ind", "st_off", "residue_r_ind", "counts")):
+            assert a.tobytes() == b.tobytes(), f"{name} differs (rows {len(rp) - 1}, seg {seg})"
+        assert got[3][0] > 0 or len(rp) == 1
+
+
+def test_static_scratch_entry_point_rejects_what_it_cannot_hold():
+    from rode_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    one = torch.zeros(8, dtype=torch.int32, device=dev)
+    p = one.data_ptr()
+    too_many = 4194304 + 1  # RODE_HIP_STATIC_MAX_ROWS + 1: refused before any launch, so the short arrays are never read
+    assert lib.rode_hip_preprocess_static(512, 32, 4, too_many, p, p, p, p, p, p + 4, 16, None) == 2
+    assert b"memory" in lib.rode_hip_error_string(2).lower()
+    assert lib.rode_hip_preprocess_static(0, 32, 4, 4, p, p, p, p, p, p + 4, 16, None) == 1
+    assert lib.rode_hip_preprocess_static(512, 32, 4, 4, None, p, p, p, p, p + 4, 16, None) == 1
