@@ -25,6 +25,19 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+TOL = {"f32": 1e-4, "f16": 2e-3}  # max over rows of |err|_inf / |ref row|_1
+
+
+def kernel_sources_fingerprint():
+    """Hash of the SpMM / SDDMM kernel sources.  Every entry of profiles/traffic.json
+    carries the fingerprint of the sources it was measured on; an entry measured on other
+    sources is not reported."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in ("rode_device.hpp", "rode_spmm.hip", "rode_sddmm.hip"):
+        with open(os.path.join(ROOT, "rode_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def parse_args():
@@ -134,6 +147,22 @@ def main():
         if side is not None:
             main_stream.wait_stream(side)
 
+    def spmm_only(flag):  # one kernel of the pair, every other decision as in the full call
+        _lib.check(lib.rode_hip_spmm_ex(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS | flag, csr.m1, csr.m2, n, k,
+                                        csr.values.data_ptr(), csr.column_indices.data_ptr(),
+                                        csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(),
+                                        csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(), B.data_ptr(),
+                                        C.data_ptr(), stream, stream), "spmm")
+
+    def spmm_reference_contract():
+        # what a caller of the reference-signature API does (RoDeSpmm.cu:492-509): memset all of C,
+        # then the typed entry point, which is promised nothing about the lists
+        C.zero_()
+        fn = {"f32": lib.rode_hip_spmm_f32, "f16": lib.rode_hip_spmm_f16}[args.dtype]
+        _lib.check(fn(csr.m1, csr.m2, n, k, csr.values.data_ptr(), csr.column_indices.data_ptr(),
+                      csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
+                      csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, stream), "spmm")
+
     def spmm(m1, m2):
         s2 = fork()
         _lib.check(spmm_fn(m1, m2, n, k, csr.values.data_ptr(), csr.column_indices.data_ptr(),
@@ -218,17 +247,14 @@ def main():
     del p_blk, p_st, p_res, p_ws
     kernels = {}
     if csr.m1 > 0:
-        kernels["spmm_block"] = event_time(lambda: spmm(csr.m1, 0), reps)  # incl. whole rows of 32..1024 slots
+        kernels["spmm_block"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_BLOCK), reps)  # incl. rows summed whole
         kernels["sddmm_block"] = event_time(lambda: sddmm(csr.m1, 0), reps)
     if csr.m2 > 0:
-        # The SpMM residue kernel skips the rows its block kernel sums whole, which only
-        # happens when both are launched by one call: time the pair and subtract (the two
-        # kernels run back to back on one stream).
-        both = event_time(lambda: spmm(csr.m1, csr.m2), reps)
-        kernels["spmm_residue"] = max(both - kernels.get("spmm_block", 0.0), 1e-4)
+        kernels["spmm_residue"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_RESIDUE), reps)
         kernels["sddmm_residue"] = event_time(lambda: sddmm(0, csr.m2), reps)
     spmm_ms = event_time(lambda: (clear_c(), spmm(csr.m1, csr.m2)), reps)
     sddmm_ms = event_time(lambda: sddmm(csr.m1, csr.m2), reps)
+    spmm_contract_ms = event_time(spmm_reference_contract, reps)
 
     if args.calibrate:
         src = torch.ones(64 * 2**20, device=dev)  # 256 MiB read + 256 MiB written by one elementwise copy kernel
@@ -253,14 +279,18 @@ def main():
                             "gather_model_GBs": round((knnz * (8 + k * elem)) / ms / 1e6, 1),
                             "GFLOPs": round(2.0 * knnz * k / ms / 1e6, 1)}
     dominant = max(kernels, key=kernels.get)
-    traffic = None
+    traffic, traffic_note = None, "no counter run of this workload under profiles/"
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
-        key = f"{args.workload}/k{k}/{args.dtype}/{dominant}"
-        traffic = json.load(open(tpath)).get(key)
+        entry = json.load(open(tpath)).get(f"{args.workload}/k{k}/{args.dtype}/seg{csr.config['seg_length']}/{dominant}")
+        if entry is not None and entry.get("sources") == kernel_sources_fingerprint():
+            traffic, traffic_note = entry["bytes"], entry.get("kernel")
+        elif entry is not None:
+            traffic_note = "stale: the counter run under profiles/ was made on other kernel sources"
     dom = per_kernel[dominant]
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": dom["algorithmic_GBs"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(dom["algorithmic_GBs"] / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "traffic_source": traffic_note,
                 "gather_model_frac": round(dom["gather_model_GBs"] / HBM_PEAK_GBS, 4)}
 
     # ---- CPU baseline: the oracle on a bounded sample of the same matrix --------
@@ -307,6 +337,11 @@ def main():
         row_err = np.maximum.reduceat(np.abs(o_gpu - o64), starts) / row_l1
         good = np.add.reduceat(scale, starts) / row_l1 <= 100.0
         sddmm_err = float(row_err[good].max(initial=0.0))
+        sddmm_err_all = float(row_err.max(initial=0.0))
+        # the excluded rows: what the reference's own fp32 CPU loop (main.cu:65-91) gets on them
+        cpu_row_err = np.maximum.reduceat(np.abs(o_ref - o64), starts) / row_l1
+        cpu_err_bad = float(cpu_row_err[~good].max(initial=0.0))
+        gpu_err_bad = float(row_err[~good].max(initial=0.0))
         sddmm_strict = float(np.max(np.abs(o_gpu - o64) / np.maximum(scale, 1e-30)))
         # the reference tests' own rule against its fp32 CPU loop: abs AND rel error above 1e-3
         diff = np.abs(o_gpu - o_ref)
@@ -332,10 +367,35 @@ def main():
                "preprocess_ms": round(t_pre * 1e3, 2),
                "all_cores": {"cores": threads,
                              "value": round(2 * (2.0 * cnt * k) / (mt_spmm + mt_sddmm) / 1e9, 3)},
-               "parity_vs_gpu": {"spmm_rowL1_err": spmm_err, "sddmm_rowL1_err_cond_le_100": sddmm_err,
+               "parity_vs_gpu": {"tolerance": TOL[args.dtype], "rows_checked": int(len(nonempty)),
+                                 "spmm_rowL1_err": spmm_err,
+                                 "sddmm_rowL1_err_all_rows": sddmm_err_all,
+                                 "sddmm_rowL1_err_cond_le_100": sddmm_err,
+                                 "sddmm_rows_cond_gt_100": int((~good).sum()),
+                                 "sddmm_rowL1_err_on_those_rows": {"gpu": gpu_err_bad, "reference_cpu_fp32_loop": cpu_err_bad,
+                                                                   "gpu_over_cpu": round(gpu_err_bad / cpu_err_bad, 3)
+                                                                   if cpu_err_bad > 0 else None},
                                  "sddmm_err_over_term_magnitude": sddmm_strict,
                                  "sddmm_reference_rule_errors": ref_rule_errors,
                                  "preprocess_bit_exact": bool(bit_exact)}}
+        # the gate: a wrong result must not leave a headline number behind
+        tol = TOL[args.dtype]
+        failures = []
+        if not bit_exact:
+            failures.append("preprocessing differs from the CPU routine")
+        if spmm_err > tol:
+            failures.append(f"SpMM row-L1 error {spmm_err:.3g} > {tol}")
+        if sddmm_err > tol:
+            failures.append(f"SDDMM row-L1 error {sddmm_err:.3g} > {tol} on rows with condition <= 100")
+        if gpu_err_bad > max(2.0 * cpu_err_bad, tol):
+            failures.append(f"SDDMM error {gpu_err_bad:.3g} on ill-conditioned rows exceeds twice the reference CPU loop's "
+                            f"{cpu_err_bad:.3g}")
+        if sddmm_strict > (2e-6 if args.dtype == "f32" else 2e-3):
+            failures.append(f"SDDMM per-element error {sddmm_strict:.3g} of the summed terms' magnitude")
+        if args.dtype == "f32" and ref_rule_errors:
+            failures.append(f"{ref_rule_errors} outputs fail the reference tests' rule")
+        cpu["parity_vs_gpu"]["passed"] = not failures
+        cpu["parity_vs_gpu"]["failures"] = failures
 
     line = {
         "metric": "SpMM & SDDMM GFLOP/s (2*nnz*K/t)", "value": round(gflops, 1), "unit": "GFLOP/s",
@@ -347,7 +407,10 @@ def main():
                                   else "step = clear C rows + SpMM + SDDMM"),
                    "rows": m, "cols": n, "nnz": nnz, "K": k, "seg_length": csr.config["seg_length"],
                    "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale},
-        "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C"},
+        "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C",
+                 "reference_contract_ms": round(spmm_contract_ms, 4),
+                 "reference_contract": "memset of all of C + the typed entry point without the whole-lists promise "
+                                       "(RoDeSpmm.cu:492-509 semantics)"},
         "sddmm": {"ms": round(sddmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / sddmm_ms / 1e6, 1)},
         "kernels": per_kernel,
         "preprocess": {"ms": round(preprocess_ms, 4), "rows_per_s": round(m / preprocess_ms * 1e3),
@@ -357,6 +420,9 @@ def main():
         "setup_s": round(setup_s, 1),
     }
     print(json.dumps(line))
+    if cpu is not None and not cpu["parity_vs_gpu"]["passed"]:
+        print("bench.py: PARITY FAILED: " + "; ".join(cpu["parity_vs_gpu"]["failures"]), file=sys.stderr)
+        sys.exit(1)
 
 
 if __name__ == "__main__":

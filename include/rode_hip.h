@@ -62,6 +62,20 @@ int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const i
                         int capacity_blocks, void* d_workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The same decomposition for a caller that holds the row pointer in HOST memory and wants
+ * HOST arrays back.  Replaces the CPU routines RoDe_preprocess_cpu,
+ * Preprocess_opt/_preprocess.cu:340-373, and RoDe_preprocess, RoDe_SDDMM/main.cu:114-163
+ * (argument order here: seg_length, k_block, vec_len; main.cu has vec_len before k_block).
+ * Every pointer is host memory; h_block_r_ind needs n_blk entries, h_st_off n_blk + 1
+ * (sentinel), h_residue_r_ind n_res; (nnz + (vec_len-1)*M)/seg_length + M (+1) and M always
+ * suffice.  Unlike everything else in this header the call allocates (and frees) device
+ * memory, copies, runs the kernels of rode_hip_preprocess on the default stream of the
+ * current device and waits for them.
+ */
+int rode_hip_preprocess_host(int seg_length, int k_block, int vec_len, int M, const int* h_row_ptr,
+                             int* h_block_r_ind, int* h_st_off, int* h_residue_r_ind, int* h_n_blk, int* h_n_res);
+
+/*
  * rode_hip_preprocess() without a workspace argument and without any allocation, for
  * callers that cannot allocate device memory: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its GPU
@@ -91,7 +105,12 @@ int rode_hip_preprocess_static(int seg_length, int k_block, int vec_len, int M, 
  * atomics, short rows are stored, rows without nonzeros are not touched.
  * n: any positive multiple of 4 (the reference needs a multiple of its 32- or
  * 64-wide tile and does not guard the edge); multiples of 32 take the unguarded
- * fast path.  The decomposition must have been made with k_block 32, vec_len 4.
+ * fast path.  The decomposition must have been made with k_block 32, vec_len 4 and a
+ * seg_length that is a positive multiple of 32 (rode_hip_preprocess itself accepts any
+ * parameters).  This holds for every SpMM and SDDMM entry point below.  With lists made
+ * for another seg_length the kernels still stay inside the arrays and inside each row,
+ * but - like the reference's kernels - they leave some nonzeros of a row out, and which
+ * ones may differ between entry points.
  */
 int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,
                       const int* d_row_offsets, const int* d_row_indices1, const int* d_row_indices2,
@@ -112,6 +131,12 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
 #define RODE_DENSE_F16 1
 #define RODE_DENSE_F64 2
 #define RODE_SPMM_WHOLE_LISTS 1
+/* Launch only the block-segment kernel / only the residue kernel of the pair, with every
+ * other decision (which rows a single wavefront sums whole) taken as if both were
+ * launched: for measuring one kernel, and for callers that order the two themselves.
+ * m1, m2 and all lists are passed as for a normal call. */
+#define RODE_SPMM_ONLY_BLOCK 2
+#define RODE_SPMM_ONLY_RESIDUE 4
 int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                      const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                      const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,

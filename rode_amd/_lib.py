@@ -18,6 +18,7 @@ SIGNATURES = {
     "rode_hip_error_string": (ctypes.c_char_p, [c_int]),
     "rode_hip_preprocess_workspace_bytes": (c_size_t, [c_int]),
     "rode_hip_preprocess": (c_int, [c_int] * 4 + [c_void_p] * 6 + [c_int, c_void_p, c_size_t, c_void_p]),
+    "rode_hip_preprocess_host": (c_int, [c_int] * 4 + [c_void_p] * 6),
     "rode_hip_preprocess_static": (c_int, [c_int] * 4 + [c_void_p] * 6 + [c_int, c_void_p]),
     "rode_hip_spmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 10),
     "rode_hip_spmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 10),
@@ -31,7 +32,7 @@ SIGNATURES = {
 }
 
 DENSE_CODE = {"f32": 0, "f16": 1, "f64": 2}  # RODE_DENSE_* of include/rode_hip.h
-SPMM_WHOLE_LISTS = 1
+SPMM_WHOLE_LISTS, SPMM_ONLY_BLOCK, SPMM_ONLY_RESIDUE = 1, 2, 4  # RODE_SPMM_* flags
 
 _lib = None
 

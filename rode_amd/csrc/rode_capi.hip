@@ -54,30 +54,74 @@ int rode_hip_preprocess_static(int seg_length, int k_block, int vec_len, int M, 
                                    d_residue_r_ind, d_n_blk, d_n_res, ws, capacity_blocks, as_stream(stream));
 }
 
+int rode_hip_preprocess_host(int seg_length, int k_block, int vec_len, int M, const int* h_row_ptr,
+                             int* h_block_r_ind, int* h_st_off, int* h_residue_r_ind, int* h_n_blk, int* h_n_res)
+{
+    if (seg_length <= 0 || k_block <= 0 || vec_len <= 0 || M < 0) return hipErrorInvalidValue;
+    if (!h_row_ptr || !h_block_r_ind || !h_st_off || !h_residue_r_ind || !h_n_blk || !h_n_res)
+        return hipErrorInvalidValue;
+    const long long nnz = h_row_ptr[M];
+    const long long cap64 = (nnz + (long long)(vec_len - 1) * M) / seg_length + M;
+    if (nnz < 0 || cap64 > 0x7ffffff0ll) return hipErrorInvalidValue;
+    const int cap = (int)cap64;
+    const size_t ws_bytes = rode::preprocess_workspace_bytes(M);
+    // one device allocation: [workspace | row_ptr | block_r_ind | st_off | residue_r_ind | counts]
+    const size_t ws_slots = (ws_bytes + 3) / 4;
+    const size_t slots = ws_slots + (size_t)(M + 1) + (size_t)cap + 1 + (size_t)cap + 2 + (size_t)(M > 0 ? M : 1) + 2;
+    int* d = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&d), slots * sizeof(int));
+    if (e != hipSuccess) return e;
+    int* d_rp = d + ws_slots;
+    int* d_blk = d_rp + (M + 1);
+    int* d_st = d_blk + cap + 1;
+    int* d_res = d_st + cap + 2;
+    int* d_cnt = d_res + (M > 0 ? M : 1);
+    int cnt[2] = {0, 0};
+    e = hipMemcpy(d_rp, h_row_ptr, sizeof(int) * (size_t)(M + 1), hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+        e = rode::preprocess_launch(seg_length, k_block, vec_len, M, d_rp, d_blk, d_st, d_res, d_cnt, d_cnt + 1, d, cap,
+                                    nullptr);
+    if (e == hipSuccess) e = hipMemcpy(cnt, d_cnt, sizeof(cnt), hipMemcpyDeviceToHost); // waits for the kernels
+    if (e == hipSuccess && cnt[0] > 0)
+        e = hipMemcpy(h_block_r_ind, d_blk, sizeof(int) * (size_t)cnt[0], hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipMemcpy(h_st_off, d_st, sizeof(int) * ((size_t)cnt[0] + 1), hipMemcpyDeviceToHost);
+    if (e == hipSuccess && cnt[1] > 0)
+        e = hipMemcpy(h_residue_r_ind, d_res, sizeof(int) * (size_t)cnt[1], hipMemcpyDeviceToHost);
+    (void)hipFree(d);
+    if (e == hipSuccess) {
+        *h_n_blk = cnt[0];
+        *h_n_res = cnt[1];
+    }
+    return e;
+}
+
 int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                      const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                      const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
                      void* stream1, void* stream2)
 {
     (void)k;
-    if (m1 < 0 || m2 < 0 || (flags & ~RODE_SPMM_WHOLE_LISTS)) return hipErrorInvalidValue;
+    constexpr int kKnown = RODE_SPMM_WHOLE_LISTS | RODE_SPMM_ONLY_BLOCK | RODE_SPMM_ONLY_RESIDUE;
+    static_assert(RODE_SPMM_WHOLE_LISTS == rode::kSpmmWholeLists && RODE_SPMM_ONLY_BLOCK == rode::kSpmmOnlyBlock &&
+                      RODE_SPMM_ONLY_RESIDUE == rode::kSpmmOnlyResidue, "header and library disagree");
+    if (m1 < 0 || m2 < 0 || (flags & ~kKnown)) return hipErrorInvalidValue;
+    if ((flags & RODE_SPMM_ONLY_BLOCK) && (flags & RODE_SPMM_ONLY_RESIDUE)) return hipErrorInvalidValue;
     if (m1 == 0 && m2 == 0) return hipSuccess;
     if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
-    const bool whole = flags & RODE_SPMM_WHOLE_LISTS;
     hipStream_t s1 = as_stream(stream1), s2 = as_stream(stream2);
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
                                         d_column_indices, static_cast<const float*>(d_values),
-                                        static_cast<const float*>(d_B), static_cast<float*>(d_C), whole, s1, s2);
+                                        static_cast<const float*>(d_B), static_cast<float*>(d_C), flags, s1, s2);
     case RODE_DENSE_F16:
         return rode::spmm_launch<__half>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets,
                                          d_row_offsets, d_column_indices, static_cast<const float*>(d_values),
-                                         static_cast<const __half*>(d_B), static_cast<float*>(d_C), whole, s1, s2);
+                                         static_cast<const __half*>(d_B), static_cast<float*>(d_C), flags, s1, s2);
     case RODE_DENSE_F64:
         return rode::spmm_launch<double>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets,
                                          d_row_offsets, d_column_indices, static_cast<const double*>(d_values),
-                                         static_cast<const double*>(d_B), static_cast<double*>(d_C), whole, s1, s2);
+                                         static_cast<const double*>(d_B), static_cast<double*>(d_C), flags, s1, s2);
     default: return hipErrorInvalidValue;
     }
 }
@@ -227,6 +271,22 @@ void RoDeSDDMM_n128(int m1, int m2, int n, int k, const int* row_indices_block, 
                                       : rode_hip_sddmm_f32(m1, m2, n, k, row_indices_block, row_indices_residue,
                                                            st_offsets, row_offsets, column_indices, values,
                                                            lhs_matrix, rhs_matrix, out, stream1, stream2));
+}
+
+void RoDe_preprocess_cpu(int N_SEG, int blockX, int vecLen, int M, const int* row_ptr, int* block_r_ind, int* st_off,
+                         int* residue_r_ind, int& n_blk, int& n_res)
+{
+    n_blk = n_res = 0;
+    report("RoDe_preprocess_cpu", rode_hip_preprocess_host(N_SEG, blockX, vecLen, M, row_ptr, block_r_ind, st_off,
+                                                           residue_r_ind, &n_blk, &n_res));
+}
+
+void RoDe_preprocess(int SegmentLength, int vectorLen, int KBLOCK, int M, const int* row_ptr, int* block_r_ind,
+                     int* st_off, int* residue_r_ind, int& n_blk, int& n_res)
+{
+    n_blk = n_res = 0;
+    report("RoDe_preprocess", rode_hip_preprocess_host(SegmentLength, KBLOCK, vectorLen, M, row_ptr, block_r_ind, st_off,
+                                                       residue_r_ind, &n_blk, &n_res));
 }
 
 void RoDe_preprocess(int N_SEG, int blockX, int vecLen, int M, const int* row_ptr, int* block_r_ind, int* st_off,

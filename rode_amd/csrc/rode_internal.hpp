@@ -22,10 +22,13 @@ hipError_t preprocess_launch(int seg, int kblock, int veclen, int M, const int* 
 template <typename T> struct SpmmAcc { using type = float; };
 template <> struct SpmmAcc<double> { using type = double; };
 
+// flags: the RODE_SPMM_* bits of the C ABI
+constexpr int kSpmmWholeLists = 1, kSpmmOnlyBlock = 2, kSpmmOnlyResidue = 4;
+
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                        const int* row_ptr, const int* col, const typename SpmmAcc<T>::type* val, const T* B,
-                       typename SpmmAcc<T>::type* C, bool whole_lists, hipStream_t s1, hipStream_t s2);
+                       typename SpmmAcc<T>::type* C, int flags, hipStream_t s1, hipStream_t s2);
 
 hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, void* C, hipStream_t stream);
 

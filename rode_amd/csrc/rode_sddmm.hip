@@ -159,10 +159,16 @@ sddmm_block_kernel(int m1, int k, const int* __restrict__ block_rows, const int*
     for (int off = 0; off < cnt; off += kWave) {
         if (off + (lane & 32) < cnt) { // the upper half sits out a trailing 32-slot step
             const int slot = off + lane;
-            const int c = col[base + slot];
-            const float v = val[base + slot];
+            // cnt is a multiple of 32 for every decomposition the kernels are specified for
+            // (segment length a multiple of 32).  Lists made with another segment length must
+            // still never make a lane read or write beyond its row's block part: such lanes
+            // repeat the last slot and store nothing.
+            const bool live = slot < cnt;
+            const int idx = base + (live ? slot : cnt - 1);
+            const int c = col[idx];
+            const float v = val[idx];
             const float d = sddmm_unit<T, KT, NS, EDGE>(rhs_lane, a, c, k, lds_cols, lane);
-            if (slot >= mask) out[base + slot] = v * d;
+            if (slot >= mask && live) out[idx] = v * d;
         }
     }
 }

@@ -321,19 +321,19 @@ inline int grid_for_waves(long long nwaves)
 template <typename T, int TN, bool EDGE>
 hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                   const int* row_ptr, const int* col, const typename DenseVec<T>::Acc* val, const T* B,
-                  typename DenseVec<T>::Acc* C, bool whole_lists, hipStream_t s1, hipStream_t s2)
+                  typename DenseVec<T>::Acc* C, int flags, hipStream_t s1, hipStream_t s2)
 {
     const int tiles = (n + TN - 1) / TN;
-    const int owned_slots = whole_lists && m1 >= kOwnedMinSegments ? kOwnedRowSlots : 0;
+    const int owned_slots = (flags & kSpmmWholeLists) && m1 >= kOwnedMinSegments ? kOwnedRowSlots : 0;
     constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
     const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0 || tiles > 65535) return hipErrorInvalidConfiguration;
-    if (m1 > 0) {
+    if (m1 > 0 && !(flags & kSpmmOnlyResidue)) {
         dim3 grid(g1, tiles);
         spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, owned_slots, block_rows, st_off, row_ptr, col,
                                                                     val, B, C);
     }
-    if (m2 > 0) {
+    if (m2 > 0 && !(flags & kSpmmOnlyBlock)) {
         dim3 grid(g2, tiles);
         spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, residue_rows, row_ptr, col, val,
                                                                       B, C);
@@ -344,12 +344,12 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
 template <typename T, int TN>
 hipError_t launch_edge(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                        const int* row_ptr, const int* col, const typename DenseVec<T>::Acc* val, const T* B,
-                       typename DenseVec<T>::Acc* C, bool whole_lists, hipStream_t s1, hipStream_t s2)
+                       typename DenseVec<T>::Acc* C, int flags, hipStream_t s1, hipStream_t s2)
 {
     return n % TN ? launch<T, TN, true>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C,
-                                        whole_lists, s1, s2)
+                                        flags, s1, s2)
                   : launch<T, TN, false>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C,
-                                         whole_lists, s1, s2);
+                                         flags, s1, s2);
 }
 
 } // namespace
@@ -361,7 +361,7 @@ hipError_t launch_edge(int m1, int m2, int n, const int* block_rows, const int* 
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                        const int* row_ptr, const int* col, const typename SpmmAcc<T>::type* val, const T* B,
-                       typename SpmmAcc<T>::type* C, bool whole_lists, hipStream_t s1, hipStream_t s2)
+                       typename SpmmAcc<T>::type* C, int flags, hipStream_t s1, hipStream_t s2)
 {
     static_assert(std::is_same<typename SpmmAcc<T>::type, typename DenseVec<T>::Acc>::value, "accumulation type");
     if (n <= 0 || n % DenseVec<T>::kElems != 0) return hipErrorInvalidValue;
@@ -372,13 +372,13 @@ hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* 
     if (kMaxTile >= 128 && padded(128) <= padded(best)) best = 128;
     if constexpr (kMaxTile >= 128) {
         if (best == 128)
-            return launch_edge<T, 128>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, whole_lists,
+            return launch_edge<T, 128>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, flags,
                                        s1, s2);
     }
     if (best == 64)
-        return launch_edge<T, 64>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, whole_lists, s1,
+        return launch_edge<T, 64>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, flags, s1,
                                   s2);
-    return launch_edge<T, 32>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, whole_lists, s1, s2);
+    return launch_edge<T, 32>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, flags, s1, s2);
 }
 
 hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, void* C, hipStream_t stream)
@@ -393,10 +393,10 @@ hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, v
 }
 
 template hipError_t spmm_launch<float>(int, int, int, const int*, const int*, const int*, const int*, const int*,
-                                       const float*, const float*, float*, bool, hipStream_t, hipStream_t);
+                                       const float*, const float*, float*, int, hipStream_t, hipStream_t);
 template hipError_t spmm_launch<__half>(int, int, int, const int*, const int*, const int*, const int*, const int*,
-                                        const float*, const __half*, float*, bool, hipStream_t, hipStream_t);
+                                        const float*, const __half*, float*, int, hipStream_t, hipStream_t);
 template hipError_t spmm_launch<double>(int, int, int, const int*, const int*, const int*, const int*, const int*,
-                                        const double*, const double*, double*, bool, hipStream_t, hipStream_t);
+                                        const double*, const double*, double*, int, hipStream_t, hipStream_t);
 
 } // namespace rode

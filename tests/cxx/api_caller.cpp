@@ -97,6 +97,29 @@ int main(int argc, char** argv)
     int cnt[2];
     HIP_OK(hipMemcpy(cnt, d_cnt, sizeof(cnt), hipMemcpyDeviceToHost));
 
+    // the host-pointer twins (Preprocess_opt/_preprocess.cu:340 and main.cu:114-123 argument
+    // orders) must give the arrays of the device routine
+    bool twins_equal = true;
+    {
+        std::vector<int> g_blk(std::max(cnt[0], 1)), g_st(cnt[0] + 1), g_res(std::max(cnt[1], 1));
+        if (cnt[0]) HIP_OK(hipMemcpy(g_blk.data(), d_blk, sizeof(int) * cnt[0], hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(g_st.data(), d_st, sizeof(int) * (cnt[0] + 1), hipMemcpyDeviceToHost));
+        if (cnt[1]) HIP_OK(hipMemcpy(g_res.data(), d_res, sizeof(int) * cnt[1], hipMemcpyDeviceToHost));
+        for (int variant = 0; variant < 2; ++variant) {
+            std::vector<int> h_blk(cap, -1), h_st(cap + 1, -1), h_res(std::max(m, 1), -1);
+            int n_blk = -1, n_res = -1;
+            if (variant == 0)
+                RoDe_preprocess_cpu(seg, 32, 4, m, row_ptr.data(), h_blk.data(), h_st.data(), h_res.data(), n_blk, n_res);
+            else
+                RoDe_preprocess(seg, 4, 32, m, row_ptr.data(), h_blk.data(), h_st.data(), h_res.data(), n_blk, n_res);
+            twins_equal = twins_equal && n_blk == cnt[0] && n_res == cnt[1] &&
+                          std::equal(g_blk.begin(), g_blk.begin() + cnt[0], h_blk.begin()) &&
+                          std::equal(g_st.begin(), g_st.end(), h_st.begin()) &&
+                          std::equal(g_res.begin(), g_res.begin() + cnt[1], h_res.begin()) &&
+                          h_blk[cnt[0]] == -1 && h_st[cnt[0] + 1] == -1; // nothing written past the result
+        }
+    }
+
     hipStream_t s1, s2;
     HIP_OK(hipStreamCreate(&s1));
     HIP_OK(hipStreamCreate(&s2));
@@ -131,9 +154,10 @@ int main(int argc, char** argv)
             if (spmm_l1[r] > 0) spmm_err = std::max(spmm_err, diff / spmm_l1[r]);
             else if (diff != 0) spmm_err = 1.0;
         }
-    const bool passed = errors == 0 && spmm_err <= 1e-4;
+    const bool passed = errors == 0 && spmm_err <= 1e-4 && twins_equal;
     std::printf("{\"passed\": %s, \"nnz\": %d, \"n_blk\": %d, \"n_res\": %d, \"sddmm_errors\": %d, "
-                "\"sddmm_max_abs\": %.3e, \"spmm_rowL1_err\": %.3e}\n",
-                passed ? "true" : "false", nnz, cnt[0], cnt[1], errors, max_abs, spmm_err);
+                "\"sddmm_max_abs\": %.3e, \"spmm_rowL1_err\": %.3e, \"host_twins_equal\": %s}\n",
+                passed ? "true" : "false", nnz, cnt[0], cnt[1], errors, max_abs, spmm_err,
+                twins_equal ? "true" : "false");
     return passed ? 0 : 1;
 }

@@ -55,6 +55,48 @@ def coverage_counts(row_ptr, blk, st, res, kblock=32, veclen=4):
     return hits, owner
 
 
+def merged_block_ranges(row_ptr, blk, st, merge_slots, kblock=32, veclen=4):
+    """Host model of what the merging block kernels touch (sddmm_block_kernel with
+    merge_slots = 128; spmm_block_kernel under the whole-lists promise with 512, for rows
+    it does not sum whole): consecutive segments of a row whose starts fall into one window
+    of merge_slots slots are handled by the first of them.  Returns one tuple per leader:
+    (row, first index read, first index written, end) -- the kernel reads col/val in
+    [first read, end) and writes out in [first written, end)."""
+    rp = np.asarray(row_ptr, dtype=np.int64)
+    out = []
+    n = len(blk)
+    i = 0
+    while i < n:
+        r = int(blk[i])
+        row_base = int(rp[r]) - int(rp[r]) % veclen
+        window = (int(st[i]) - row_base) // merge_slots
+        j = i + 1
+        while j < n and int(blk[j]) == r and (int(st[j]) - row_base) // merge_slots == window:
+            j += 1
+        block_end = row_base + (int(rp[r + 1]) - row_base) // kblock * kblock
+        end = min(block_end, int(st[j]))
+        start = int(st[i])
+        base = start - start % veclen
+        if end > base:
+            out.append((r, base, start, end))
+        i = j
+    return out
+
+
+def residue_ranges(row_ptr, res, kblock=32, veclen=4):
+    """(row, first, end) of the slots each residue work item owns (RoDeSpmm.cu:71-82)."""
+    rp = np.asarray(row_ptr, dtype=np.int64)
+    out = []
+    for r in res:
+        s, e = int(rp[r]), int(rp[r + 1])
+        pad = s % veclen
+        N = e - s + pad
+        first = (s - pad) + N // kblock * kblock if N >= kblock else s
+        if e > first:
+            out.append((int(r), first, e))
+    return out
+
+
 def row_of_index(row_ptr):
     rp = np.asarray(row_ptr, dtype=np.int64)
     return np.repeat(np.arange(len(rp) - 1), np.diff(rp))

@@ -31,7 +31,9 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_reference_signature_entry_points_are_exported():
     out = subprocess.check_output(["nm", "-D", "--defined-only", "-C", _lib.LIB_PATH], text=True)
-    for name in ("RoDeSpmm_n32(", "RoDeSpmm_n128(", "RoDeSDDMM_n32(", "RoDeSDDMM_n128(", "RoDe_preprocess("):
+    for name in ("RoDeSpmm_n32(", "RoDeSpmm_n128(", "RoDeSDDMM_n32(", "RoDeSDDMM_n128(", "RoDe_preprocess(",
+                 "RoDe_preprocess_cpu(int, int, int, int, int const*, int*, int*, int*, int&, int&)",
+                 "RoDe_preprocess(int, int, int, int, int const*, int*, int*, int*, int&, int&)"):
         assert name in out, f"C++ entry point {name}...) missing"
 
 

@@ -21,3 +21,4 @@ def test_cxx_caller(args):
     res = json.loads(line)
     assert run.returncode == 0 and res["passed"], (res, run.stderr)
     assert res["sddmm_errors"] == 0 and res["spmm_rowL1_err"] <= 1e-4
+    assert res["host_twins_equal"], "RoDe_preprocess_cpu / host RoDe_preprocess differ from the device routine"

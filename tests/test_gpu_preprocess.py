@@ -143,3 +143,46 @@ def test_capacity_too_small_is_detected_not_overrun():
                                    cnt.data_ptr(), cnt.data_ptr() + 4, cap, ws.data_ptr(), nbytes, None) != 0
     assert lib.rode_hip_preprocess(32, 32, 4, 1000, d_rp.data_ptr(), blk.data_ptr(), st.data_ptr(), res.data_ptr(),
                                    cnt.data_ptr(), cnt.data_ptr() + 4, cap, ws.data_ptr(), 16, None) != 0
+
+
+def test_host_pointer_twins():
+    """RoDe_preprocess_cpu (Preprocess_opt/_preprocess.cu:340 order: seg, k_block, vec_len) and
+    the host overload of RoDe_preprocess (main.cu:114-123 order: seg, vec_len, k_block), called
+    through their mangled names with host arrays and int& counts, and the C-ABI function
+    beneath them."""
+    import ctypes
+    import oracle
+    from rode_amd import _lib
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    rng = np.random.default_rng(8)
+    rp = (np.concatenate([[0], rng.integers(0, 700, 30000)]).cumsum() + 1).astype(np.int32)
+    m = len(rp) - 1
+    for name, order in (("_Z19RoDe_preprocess_cpuiiiiPKiPiS1_S1_RiS2_", "seg_kb_vl"),
+                        ("_Z15RoDe_preprocessiiiiPKiPiS1_S1_RiS2_", "seg_vl_kb"), ("rode_hip_preprocess_host", "c")):
+        for seg in (512, 32):
+            oblk, ost, ores = oracle.preprocess(rp, seg)
+            cap = (int(rp[-1]) + 3 * m) // seg + m + 1
+            blk, st, res = np.full(cap, -1, np.int32), np.full(cap + 1, -1, np.int32), np.full(m, -1, np.int32)
+            nb, nr = ctypes.c_int(-1), ctypes.c_int(-1)
+            fn = getattr(lib, name)
+            fn.restype = ctypes.c_int if order == "c" else None
+            fn.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 6
+            a, b = (32, 4) if order != "seg_vl_kb" else (4, 32)
+            ret = fn(seg, a, b, m, rp.ctypes.data, blk.ctypes.data, st.ctypes.data, res.ctypes.data,
+                     ctypes.addressof(nb), ctypes.addressof(nr))
+            assert order != "c" or ret == 0
+            assert (nb.value, nr.value) == (len(oblk), len(ores)), name
+            assert blk[:nb.value].tobytes() == oblk.tobytes() and (blk[nb.value:] == -1).all()
+            assert st[:nb.value + 1].tobytes() == ost.tobytes() and (st[nb.value + 1:] == -1).all()
+            assert res[:nr.value].tobytes() == ores.tobytes() and (res[nr.value:] == -1).all()
+    # empty matrix, bad arguments
+    z = np.zeros(1, np.int32)
+    one = np.full(2, -1, np.int32)
+    nb, nr = ctypes.c_int(-1), ctypes.c_int(-1)
+    host = lib.rode_hip_preprocess_host
+    host.restype, host.argtypes = ctypes.c_int, [ctypes.c_int] * 4 + [ctypes.c_void_p] * 6
+    assert host(512, 32, 4, 0, z.ctypes.data, one.ctypes.data, one.ctypes.data, one.ctypes.data,
+                ctypes.addressof(nb), ctypes.addressof(nr)) == 0
+    assert (nb.value, nr.value) == (0, 0) and one[0] == 0
+    assert host(0, 32, 4, 0, z.ctypes.data, one.ctypes.data, one.ctypes.data, one.ctypes.data,
+                ctypes.addressof(nb), ctypes.addressof(nr)) != 0

@@ -302,3 +302,100 @@ def test_lists_passed_in_slices(seg):
     got = out.cpu().numpy()
     assert np.isfinite(got).all()
     assert np.max(np.abs(got - ref) / np.maximum(scale, 1e-30)) <= 2e-6
+
+
+@pytest.mark.parametrize("seg", [48, 80, 100])
+def test_lists_of_an_unsupported_segment_length_stay_in_bounds(seg):
+    """seg_length % 32 != 0 is outside the contract of the entry points (the Python class
+    refuses it), but the C ABI cannot tell how its lists were made.  The kernels must then
+    write exactly the entries that the host model of their index ranges lists
+    (helpers.merged_block_ranges / residue_ranges: inside the arrays, inside the row),
+    each with the right value, and nothing else -- canaries before out[0], after
+    out[nnz-1] and on every entry no work item owns must survive."""
+    import oracle
+    from gpu_common import DEV
+    from helpers import merged_block_ranges, random_csr, residue_ranges
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(seg)
+    m, n, k = 700, 900, 64
+    rp, col, val = random_csr(rng, m, n, 45, long_rows=6, long_len=850, empty_frac=0.1)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    nnz = len(val)
+    d_rp = torch.from_numpy(rp).to(DEV)
+    blk, st, res, m1, m2 = rode_sddmm_hip.preprocess_device(d_rp, nnz, seg, 32, 4)
+    oblk, ost, ores = oracle.preprocess(rp, seg)
+    assert blk.cpu().numpy()[:m1].tobytes() == oblk.tobytes() and st.cpu().numpy().tobytes() == ost.tobytes()
+    expect = np.zeros(nnz, bool)
+    for r, _, first, end in merged_block_ranges(rp, oblk, ost, 128):
+        expect[first:end] = True
+    for r, first, end in residue_ranges(rp, ores):
+        expect[first:end] = True
+    assert expect.sum() > 0
+    pad = 256
+    dcol = torch.zeros(nnz + 2 * pad, dtype=torch.int32, device=DEV)   # col / val with margins, so that a stray
+    dval = torch.zeros(nnz + 2 * pad, dtype=torch.float32, device=DEV)  # read would be harmless and a stray write visible
+    dcol[pad:pad + nnz] = torch.from_numpy(col).to(DEV)
+    dval[pad:pad + nnz] = torch.from_numpy(val).to(DEV)
+    from rode_amd import _lib
+    lib = _lib.load()
+    out = torch.full((nnz + 2 * pad,), -777.0, device=DEV)
+    dl, dr = torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV)
+    _lib.check(lib.rode_hip_sddmm_f32(m1, m2, n, k, blk.data_ptr(), res.data_ptr(), st.data_ptr(), d_rp.data_ptr(),
+                                      dcol.data_ptr() + 4 * pad, dval.data_ptr() + 4 * pad, dl.data_ptr(), dr.data_ptr(),
+                                      out.data_ptr() + 4 * pad, None, None), "sddmm")
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert (got[:pad] == -777.0).all() and (got[pad + nnz:] == -777.0).all(), "write outside out[0, nnz)"
+    got = got[pad:pad + nnz]
+    assert ((got != -777.0) == expect).all(), "written entries differ from the host model"
+    ref, scale = oracle.sddmm_f64(rp, col, val, lhs, rhs, with_abs=True)
+    assert np.max(np.abs(got[expect] - ref[expect]) / np.maximum(scale[expect], 1e-30)) <= 2e-6
+
+
+def test_headline_configuration_full_size_against_oracle():
+    """The configuration the benchmark reports -- power law, full size, K = 128, the
+    library's default decomposition (>= 16384 block segments, so merged leaders are what
+    runs) -- against the fp64 oracle on a fixed sample of rows: the longest row, rows of
+    32..1024 slots, rows of more than 1024 slots, short rows."""
+    import oracle
+    from gpu_common import DEV, TOL_F32, make_csr
+    from helpers import sddmm_row_l1_errors
+    from rode_amd import rode_sddmm, workloads
+    m, n, rp, col, val = workloads.config("c4_powerlaw")
+    k = 128
+    csr = make_csr(rp, col, val, m, n, k)
+    assert csr.m1 >= 16384
+    g = torch.Generator(device=DEV).manual_seed(77)
+    lhs = torch.randn(m, k, device=DEV, generator=g)
+    rhs = torch.randn(n, k, device=DEV, generator=g)
+    out = rode_sddmm(csr, lhs, rhs)
+    rows = sample_rows(rp, np.random.default_rng(4))
+    sub_rp, idx = sub_csr(rp, rows)
+    ref, scale = oracle.sddmm_f64(sub_rp, col[idx], val[idx], lhs[torch.from_numpy(rows).to(DEV)].cpu().numpy(),
+                                  rhs.cpu().numpy(), with_abs=True)
+    got = out[torch.from_numpy(idx).to(DEV)].cpu().numpy()
+    assert np.max(np.abs(got - ref) / np.maximum(scale, 1e-30)) <= 2e-6
+    err, cond = sddmm_row_l1_errors(got, ref, scale, sub_rp)
+    assert err[cond <= 100].max() <= TOL_F32
+    print(f"c4 K=128 full size: {len(rows)} rows, {len(idx)} nnz, worst row-L1 error {err.max():.2e} "
+          f"({int((cond > 100).sum())} rows with condition > 100, worst {err[cond <= 100].max():.2e} on the others)")
+
+
+def sample_rows(rp, rng):
+    """Longest row, 200 rows of 32..1024 aligned slots, 20 rows above 1024, 500 shorter ones."""
+    lens = np.diff(rp)
+    N = lens + rp[:-1] % 4
+    pick = [np.array([int(np.argmax(lens))])]
+    for mask, count in (((N >= 32) & (N <= 1024), 200), (N > 1024, 20), ((N > 0) & (N < 32), 500)):
+        cand = np.nonzero(mask)[0]
+        pick.append(rng.choice(cand, size=min(count, len(cand)), replace=False))
+    return np.unique(np.concatenate(pick)).astype(np.int64)
+
+
+def sub_csr(rp, rows):
+    """Row pointer of the matrix made of ``rows`` and the indices of their nonzeros."""
+    lens = np.diff(rp)[rows]
+    sub_rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    idx = np.concatenate([np.arange(rp[r], rp[r + 1], dtype=np.int64) for r in rows])
+    return sub_rp, idx

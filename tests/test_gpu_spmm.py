@@ -432,3 +432,66 @@ def test_whole_row_mode_and_split_calls(seg, half):
     typed(0, csr.m2, csr.block_indices.data_ptr(), csr.st_offsets.data_ptr(), C)
     torch.cuda.synchronize()
     assert spmm_row_l1_error(C.cpu().numpy(), ref) <= tol
+
+
+def test_headline_configuration_full_size_against_oracle():
+    """Power law, full size, width 128, through rode_spmm (whole-lists promise with >= 16384
+    block segments: rows of 32..1024 slots are summed by one wave, longer rows by merged
+    leaders plus atomics) against the fp64 oracle on a fixed sample of rows that holds the
+    longest row and rows of every kind."""
+    import oracle
+    from gpu_common import DEV, TOL_F32, make_csr
+    from helpers import spmm_row_l1_error
+    from rode_amd import rode_spmm, workloads
+    from test_gpu_sddmm import sample_rows, sub_csr
+    m, k, rp, col, val = workloads.config("c4_powerlaw")
+    n = 128
+    csr = make_csr(rp, col, val, m, k, n)
+    assert csr.m1 >= 16384
+    g = torch.Generator(device=DEV).manual_seed(78)
+    B = torch.randn(k, n, device=DEV, generator=g)
+    C = rode_spmm(csr, B)
+    rows = sample_rows(rp, np.random.default_rng(5))
+    sub_rp, idx = sub_csr(rp, rows)
+    ref, scale = oracle.spmm_f64(sub_rp, col[idx], val[idx], B.cpu().numpy(), with_abs=True)
+    got = C[torch.from_numpy(rows).to(DEV)].cpu().numpy()
+    err = spmm_row_l1_error(got, ref)
+    assert err <= TOL_F32, f"row-L1 error {err}"
+    assert (np.abs(got - ref) / np.maximum(scale, 1e-30)).max() <= 2e-6
+    print(f"c4 width 128 full size: {len(rows)} rows, {len(idx)} nnz, row-L1 error {err:.2e}")
+
+
+def test_measurement_flags_launch_one_kernel_of_the_pair():
+    """RODE_SPMM_ONLY_BLOCK + RODE_SPMM_ONLY_RESIDUE in two calls give the result of one
+    normal call, also under the whole-lists promise (each kernel still skips what the
+    other one sums)."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(9)
+    m, k, n = 20000, 2500, 64
+    lens = rng.choice([0, 3, 31, 40, 100, 700, 1100, 2400], size=m, p=[.1, .2, .1, .2, .2, .1, .05, .05])
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(k, size=l, replace=False)) for l in lens]).astype(np.int32)
+    val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
+    csr = make_csr(rp, col, val, m, k, n, 32)
+    assert csr.m1 >= 16384
+    B = torch.from_numpy(rng.standard_normal((k, n)).astype(np.float32)).to(DEV)
+
+    def call(flags, C):
+        _lib.check(lib.rode_hip_spmm_ex(0, flags, csr.m1, csr.m2, k, n, csr.values.data_ptr(),
+                                        csr.column_indices.data_ptr(), csr.row_offsets.data_ptr(),
+                                        csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
+                                        csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), None, None), "spmm")
+
+    for base in (0, _lib.SPMM_WHOLE_LISTS):
+        both, split = torch.zeros(m, n, device=DEV), torch.zeros(m, n, device=DEV)
+        call(base, both)
+        call(base | _lib.SPMM_ONLY_BLOCK, split)
+        call(base | _lib.SPMM_ONLY_RESIDUE, split)
+        torch.cuda.synchronize()
+        assert (both - split).abs().max().item() <= 1e-4 * both.abs().max().item()
+    assert lib.rode_hip_spmm_ex(0, 6, csr.m1, csr.m2, k, n, csr.values.data_ptr(), csr.column_indices.data_ptr(),
+                                csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(),
+                                csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(), B.data_ptr(),
+                                both.data_ptr(), None, None) != 0

@@ -114,3 +114,33 @@ def test_brute_force_tiny():
         blk, st, res = oracle.preprocess(rp, seg, kb, vl)
         b2, s2, r2 = _brute_force(rp.tolist(), seg, kb, vl)
         assert blk.tolist() == b2 and st.tolist() == s2 and res.tolist() == r2, (rp, seg, kb, vl)
+
+
+@pytest.mark.parametrize("seg", [32, 64, 96, 512, 48, 80, 100, 36, 16])
+def test_block_kernel_ranges_stay_in_their_row_for_any_segment_length(seg):
+    """The SpMM/SDDMM entry points are specified for seg_length % 32 == 0, where every
+    nonzero is covered exactly once.  Lists made with another segment length (the C ABI
+    cannot tell) must still keep every access of the merging block kernels inside the
+    arrays and inside the leader's own row, with no index written twice; they may leave
+    nonzeros out (the reference's kernels drop slots there too)."""
+    import oracle
+    from helpers import merged_block_ranges, residue_ranges
+    rng = np.random.default_rng(seg)
+    for trial in range(40):
+        m = int(rng.integers(1, 60))
+        lens = rng.choice([0, 1, 3, 31, 32, 33, 47, 48, 49, 95, 96, 97, 130, 500, 1300], size=m)
+        rp = np.concatenate([[int(rng.integers(0, 4))], lens]).cumsum().astype(np.int32)
+        blk, st, res = oracle.preprocess(rp, seg)
+        nnz = int(rp[-1])
+        for merge in (128, 512):
+            hits = np.zeros(nnz, np.int32)
+            for r, first_read, first_written, end in merged_block_ranges(rp, blk, st, merge):
+                assert 0 <= first_read and end <= nnz, "read outside col/val"
+                assert rp[r] <= first_written and end <= rp[r + 1], "write outside the leader's row"
+                hits[first_written:end] += 1
+            for r, first, end in residue_ranges(rp, res):
+                assert rp[r] <= first and end <= rp[r + 1]
+                hits[first:end] += 1
+            assert hits.max(initial=0) <= 1, "an index is written by two work items"
+            if seg % 32 == 0:
+                assert (hits[rp[0]:] == 1).all(), "a nonzero is left out"
