@@ -68,8 +68,9 @@ class SpmmFunction(torch.autograd.Function):
             csr_t, perm = csr.transpose()
             d_dense = _spmm(csr_t, values.float()[perm], g).to(dense.dtype)
         if ctx.needs_input_grad[1]:
-            if g.shape[1] not in (32, 64, 128):
-                raise NotImplementedError("gradient with respect to the sparse values needs a dense width of 32, 64 or 128")
+            if g.shape[1] % 4 != 0 or g.shape[1] > 512:
+                raise NotImplementedError("the gradient with respect to the sparse values is an SDDMM over the dense "
+                                          "width, which must be a multiple of 4 up to 512")
             d_values = _sddmm(csr, torch.ones_like(values, dtype=torch.float32), g, dense.float()).to(values.dtype)
         return None, d_values, d_dense
 

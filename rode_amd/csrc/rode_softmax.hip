@@ -22,8 +22,9 @@ __device__ __forceinline__ float wave_max(float v)
 }
 
 __global__ void __launch_bounds__(kWgThreads)
-csr_softmax_kernel(int M, const int* __restrict__ row_ptr, const float* __restrict__ in, float* __restrict__ out,
-                   float scale)
+csr_softmax_kernel(int M, const int* __restrict__ row_ptr, const float* in, float* out, float scale)
+// in / out (and dp / ds below) may be the same array: no __restrict__ on them; every index
+// is read and then written by the same lane
 {
     const int lane = threadIdx.x % kWave;
     const int row = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + threadIdx.x / kWave;
@@ -41,8 +42,8 @@ csr_softmax_kernel(int M, const int* __restrict__ row_ptr, const float* __restri
 }
 
 __global__ void __launch_bounds__(kWgThreads)
-csr_softmax_backward_kernel(int M, const int* __restrict__ row_ptr, const float* __restrict__ p,
-                            const float* __restrict__ dp, float* __restrict__ ds, float scale)
+csr_softmax_backward_kernel(int M, const int* __restrict__ row_ptr, const float* __restrict__ p, const float* dp,
+                            float* ds, float scale)
 {
     const int lane = threadIdx.x % kWave;
     const int row = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + threadIdx.x / kWave;

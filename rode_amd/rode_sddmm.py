@@ -54,6 +54,7 @@ class RoDeCSR:
         self.column_indices = column_indices.to(dtype=torch.int32, device=self.device).contiguous()
         self.values = values.to(dtype=torch.float32, device=self.device).contiguous()
         self.row_offsets = self.row_offsets_cpu.to(device=self.device)
+        self._shared = {}  # per-pattern cache (the transposed pattern); with_values() copies share it
         self._preprocess()
 
     def _preprocess(self):
@@ -83,7 +84,7 @@ class RoDeCSR:
         """``(csr_t, perm)``: the decomposed pattern of the transposed matrix and the
         permutation with ``csr_t.values == self.values[perm]`` (built on the GPU once,
         then cached).  Needed by the gradients with respect to the column-side operands."""
-        cached = self.__dict__.get("_transpose")
+        cached = self._shared.get("transpose")
         if cached is None:
             lens = (self.row_offsets[1:] - self.row_offsets[:-1]).to(torch.int64)
             rows = torch.repeat_interleave(torch.arange(self.m, device=self.device), lens)
@@ -94,7 +95,7 @@ class RoDeCSR:
             csr_t = RoDeCSR(row_offsets_t.to(torch.int32), rows[perm].to(torch.int32), self.values.float()[perm],
                             self.device, self.n, self.m, self.k, config=self.config)
             cached = (csr_t, perm)
-            self.__dict__["_transpose"] = cached
+            self._shared["transpose"] = cached
         csr_t, perm = cached
         return csr_t.with_values(self.values[perm]), perm
 

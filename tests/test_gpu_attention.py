@@ -61,6 +61,13 @@ def test_transpose():
     assert torch.equal(csr_t.values, csr.values[perm])
     again, _ = csr.transpose()
     assert again.block_indices.data_ptr() == csr_t.block_indices.data_ptr()  # cached
+    # a copy with other values made BEFORE the first transpose shares the cache with its source
+    fresh = make_csr(rp, col, val, m, n, 32)
+    copy = fresh.with_values(fresh.values * 2)
+    t1, _ = copy.transpose()
+    t2, _ = fresh.transpose()
+    assert t1.block_indices.data_ptr() == t2.block_indices.data_ptr()
+    assert torch.equal(t1.values, 2 * t2.values)
 
 
 def test_row_softmax_forward_backward():
@@ -91,7 +98,33 @@ def test_row_softmax_forward_backward():
     assert (s.grad.double() - sd.grad).abs().max().item() < 1e-5
 
 
-@pytest.mark.parametrize("k", [32, 64, 128])
+def test_row_softmax_in_place():
+    """The C ABI allows out == in and ds == dp."""
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(6)
+    m, n = 400, 2000
+    rp, col, val = random_csr(rng, m, n, 70, long_rows=3, long_len=1900, empty_frac=0.1)
+    csr = make_csr(rp, col, val, m, n, 32)
+    s = torch.from_numpy(rng.standard_normal(len(val)).astype(np.float32) * 3).to(DEV)
+    g = torch.from_numpy(rng.standard_normal(len(val)).astype(np.float32)).to(DEV)
+    p = torch.empty_like(s)
+    rp_d = csr.row_offsets.data_ptr()
+    _lib.check(lib.rode_hip_csr_softmax_f32(m, rp_d, s.data_ptr(), p.data_ptr(), 0.5, None), "softmax")
+    inplace = s.clone()
+    _lib.check(lib.rode_hip_csr_softmax_f32(m, rp_d, inplace.data_ptr(), inplace.data_ptr(), 0.5, None), "softmax")
+    ds = torch.empty_like(s)
+    _lib.check(lib.rode_hip_csr_softmax_backward_f32(m, rp_d, p.data_ptr(), g.data_ptr(), ds.data_ptr(), 0.5, None), "bwd")
+    g_inplace = g.clone()
+    _lib.check(lib.rode_hip_csr_softmax_backward_f32(m, rp_d, p.data_ptr(), g_inplace.data_ptr(), g_inplace.data_ptr(),
+                                                     0.5, None), "bwd")
+    torch.cuda.synchronize()
+    assert torch.equal(inplace, p) and torch.equal(g_inplace, ds)
+
+
+@pytest.mark.parametrize("k", [32, 64, 128, 40])
 def test_sddmm_and_spmm_gradients(k):
     from gpu_common import DEV, make_csr
     from helpers import random_csr
