@@ -34,7 +34,8 @@ def kernel_sources_fingerprint():
     sources is not reported."""
     import hashlib
     h = hashlib.sha256()
-    for name in ("rode_device.hpp", "rode_spmm.hip", "rode_sddmm.hip"):
+    for name in ("rode_device.hpp", "rode_items.hpp", "rode_window.hpp", "rode_spmm.hip", "rode_sddmm.hip",
+                 "rode_spmm_window.hip", "rode_sddmm_window.hip"):
         with open(os.path.join(ROOT, "rode_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]
@@ -58,6 +59,8 @@ def parse_args():
                    help="step = SDDMM scores -> row softmax -> clear C -> SpMM with those values (sparse attention)")
     p.add_argument("--memset-c", action="store_true",
                    help="clear all of C before SpMM (the reference's contract) instead of only the rows SpMM adds to")
+    p.add_argument("--no-plan", action="store_true",
+                   help="do not use the locality plan (window kernels for chunks whose dense rows fit an LDS window)")
     p.add_argument("--calibrate", action="store_true",
                    help="also run one plain device copy of 256 MiB (a known size to scale profiler counters by)")
     return p.parse_args()
@@ -106,7 +109,7 @@ def main():
 
     import torch
 
-    from rode_amd import RoDeCSR, _lib, workloads
+    from rode_amd import RoDeCSR, _lib, rode_sddmm_hip, workloads
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -120,7 +123,8 @@ def main():
     nnz = int(row_ptr[-1])
     cfg = None if args.seg == 0 else {"seg_length": args.seg, "k_block": 32, "vec_len": 4}
     csr = RoDeCSR(torch.from_numpy(row_ptr), torch.from_numpy(col), torch.from_numpy(val), dev, m, n,
-                  k if k in RoDeCSR.CONFIGS else 128, config=cfg)
+                  k if k in RoDeCSR.CONFIGS else 128, config=cfg, locality=False if args.no_plan else "auto")
+    plan_dev, plan_counts = rode_sddmm_hip._plan_args(csr.plan)
     gen = torch.Generator(device=dev).manual_seed(3000)
     B = torch.randn(n, k, device=dev, generator=gen).to(tdtype)     # SpMM dense operand, also SDDMM rhs
     L = torch.randn(m, k, device=dev, generator=gen).to(tdtype)     # SDDMM lhs
@@ -129,10 +133,12 @@ def main():
     setup_s = time.time() - t0
 
     stream = torch.cuda.current_stream().cuda_stream
-    def spmm_fn(*a):  # the whole decomposition is passed, and the library is told so
-        return lib.rode_hip_spmm_ex(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS, *a)
+    def spmm_fn(*a, flags=0):  # the whole decomposition is passed, and the library is told so
+        return lib.rode_hip_spmm_planned(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS | flags, *a[:-2],
+                                         plan_dev, plan_counts, *a[-2:])
 
-    sddmm_fn = lib.rode_hip_sddmm_f32 if args.dtype == "f32" else lib.rode_hip_sddmm_f16
+    def sddmm_fn(*a):
+        return lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[args.dtype], *a[:-2], plan_dev, plan_counts, *a[-2:])
 
     main_stream = torch.cuda.current_stream()
     side = torch.cuda.Stream() if args.two_streams else None
@@ -148,11 +154,9 @@ def main():
             main_stream.wait_stream(side)
 
     def spmm_only(flag):  # one kernel of the pair, every other decision as in the full call
-        _lib.check(lib.rode_hip_spmm_ex(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS | flag, csr.m1, csr.m2, n, k,
-                                        csr.values.data_ptr(), csr.column_indices.data_ptr(),
-                                        csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(),
-                                        csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(), B.data_ptr(),
-                                        C.data_ptr(), stream, stream), "spmm")
+        _lib.check(spmm_fn(csr.m1, csr.m2, n, k, csr.values.data_ptr(), csr.column_indices.data_ptr(),
+                           csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
+                           csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, stream, flags=flag), "spmm")
 
     def spmm_reference_contract():
         # what a caller of the reference-signature API does (RoDeSpmm.cu:492-509): memset all of C,
@@ -406,7 +410,9 @@ def main():
                                + ("step = SDDMM -> row softmax -> clear C -> SpMM (chained)" if args.chain
                                   else "step = clear C rows + SpMM + SDDMM"),
                    "rows": m, "cols": n, "nnz": nnz, "K": k, "seg_length": csr.config["seg_length"],
-                   "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale},
+                   "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale,
+                   "locality_plan": None if csr.plan is None else
+                   {"residue_chunks": csr.plan.counts[0], "chunks_with_lds_window": csr.plan.counts[1]}},
         "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C",
                  "reference_contract_ms": round(spmm_contract_ms, 4),
                  "reference_contract": "memset of all of C + the typed entry point without the whole-lists promise "

@@ -143,6 +143,43 @@ int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const v
                      void* stream1, void* stream2);
 
 /*
+ * Locality plan (no counterpart in the reference, whose kernels gather every dense row
+ * from memory: RoDe_SpMM/RoDeSpmm.cu:140-160, RoDe_SDDMM/RoDeSddmm.cu:96-140).
+ * The residue list is cut into chunks of RODE_HIP_PLAN_RESIDUE_CHUNK entries.  For every
+ * chunk the plan records whether the dense rows its nonzeros reference cluster in a window
+ * of at most RODE_HIP_WINDOW_ROWS consecutive rows (banded matrices: FEM, stencils).  The
+ * *_planned entry points below process such a chunk with kernels that stage the window in
+ * LDS once per 128-byte column tile and read it from there; nonzeros outside the window
+ * are still gathered from memory, so a plan never changes a result, only the speed.
+ *   dense_rows   rows of the dense operand the column indices point into (B of SpMM,
+ *                rhs of SDDMM): the number of columns of the sparse matrix
+ *   d_plan       rode_hip_window_plan_bytes(m2) bytes, 16-byte aligned, out.  Layout:
+ *                int[4] header {residue chunks, residue chunks with a window, 0, 0},
+ *                then int[4] per chunk {first window row, window rows (0: none),
+ *                nonzeros inside the window, nonzeros}
+ *   h_counts     NULL, or HOST int[4] that receives the header; the call then waits for
+ *                the kernels (two small launches, each nonzero's column index read once)
+ * A plan belongs to exactly the residue list it was made from (same m2, same arrays).
+ */
+#define RODE_HIP_PLAN_RESIDUE_CHUNK 128
+#define RODE_HIP_WINDOW_ROWS 512
+size_t rode_hip_window_plan_bytes(int m2);
+int rode_hip_window_plan(int m2, int dense_rows, const int* d_row_indices_residue, const int* d_row_offsets,
+                         const int* d_column_indices, void* d_plan, size_t plan_bytes, int* h_counts, void* stream);
+
+/*
+ * rode_hip_spmm_ex with a locality plan.  d_plan: a plan made from these lists, or NULL
+ * (then exactly rode_hip_spmm_ex).  h_plan_counts: NULL, or the HOST int[4] header that
+ * rode_hip_window_plan returned; with it, kernels that would find no chunk to work on are
+ * not launched at all.  fp64 operands, and dense rows of at most 128 bytes, ignore the plan.
+ * Same results as without a plan, up to the order of the fp32 additions inside a row.
+ */
+int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
+                          const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
+                          const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
+                          const void* d_plan, const int* h_plan_counts, void* stream1, void* stream2);
+
+/*
  * Prepares an uninitialised C[M x n] for one of the SpMM calls: zeroes exactly the rows
  * that SpMM adds to (aligned length >= 32) or never touches (rows in no list) and
  * leaves alone the rows it stores.  A cheaper replacement for clearing all of C; the
@@ -188,6 +225,18 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
                        const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                        const int* d_column_indices, const float* d_values, const void* d_lhs_half,
                        const void* d_rhs_half, float* d_out, void* stream1, void* stream2);
+
+/*
+ * SDDMM with a locality plan: dtype RODE_DENSE_F32 or RODE_DENSE_F16 selects the element
+ * type of lhs / rhs; d_plan / h_plan_counts as for rode_hip_spmm_planned (NULL: exactly the
+ * typed functions above).  Same results up to the order of the fp32 additions of a dot
+ * product.  No counterpart in the reference.
+ */
+int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d_row_indices_block,
+                           const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
+                           const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
+                           const void* d_rhs_matrix, float* d_out, const void* d_plan, const int* h_plan_counts,
+                           void* stream1, void* stream2);
 
 /*
  * Row softmax over the values of a CSR pattern, out[idx] = softmax over the row of

@@ -5,10 +5,13 @@
 #include "../../include/RoDeSddmm.h"
 #include "../../include/RoDeSpmm.h"
 #include "rode_internal.hpp"
+#include "rode_items.hpp"
 
 #include <cstdio>
 
 static_assert(RODE_HIP_STATIC_MAX_ROWS == rode::kPreprocessStaticMaxRows, "header and library disagree");
+static_assert(RODE_HIP_PLAN_RESIDUE_CHUNK == rode::kPlanResidueChunk && RODE_HIP_WINDOW_ROWS == rode::kResidueWindowRowsMax,
+              "header and library disagree");
 
 namespace {
 
@@ -95,10 +98,49 @@ int rode_hip_preprocess_host(int seg_length, int k_block, int vec_len, int M, co
     return e;
 }
 
+size_t rode_hip_window_plan_bytes(int m2) { return m2 < 0 ? 0 : rode::window_plan_ints(m2) * sizeof(int); }
+
+int rode_hip_window_plan(int m2, int dense_rows, const int* d_row_indices_residue, const int* d_row_offsets,
+                         const int* d_column_indices, void* d_plan, size_t plan_bytes, int* h_counts, void* stream)
+{
+    if (m2 < 0 || dense_rows < 0 || !d_plan || !aligned16(d_plan)) return hipErrorInvalidValue;
+    if (plan_bytes < rode_hip_window_plan_bytes(m2)) return hipErrorInvalidValue;
+    if (m2 > 0 && (!d_row_indices_residue || !d_row_offsets || !d_column_indices)) return hipErrorInvalidValue;
+    hipError_t e = rode::window_plan_launch(m2, dense_rows, d_row_indices_residue, d_row_offsets, d_column_indices,
+                                            static_cast<int*>(d_plan), as_stream(stream));
+    if (e == hipSuccess && h_counts) {
+        e = hipMemcpyAsync(h_counts, d_plan, 4 * sizeof(int), hipMemcpyDeviceToHost, as_stream(stream));
+        if (e == hipSuccess) e = hipStreamSynchronize(as_stream(stream));
+    }
+    return e;
+}
+
+namespace {
+// The caller's plan as the launchers take it; false if it cannot belong to these lists.
+bool plan_ref(const void* d_plan, const int* h_plan_counts, int m2, rode::PlanRef& plan)
+{
+    if (!d_plan) return true;
+    if (!aligned16(d_plan)) return false;
+    if (h_plan_counts && h_plan_counts[0] != rode::plan_residue_chunks(m2)) return false;
+    plan.dev = static_cast<const int*>(d_plan);
+    plan.host_counts = h_plan_counts;
+    return true;
+}
+} // namespace
+
 int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                      const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                      const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
                      void* stream1, void* stream2)
+{
+    return rode_hip_spmm_planned(dtype, flags, m1, m2, k, n, d_values, d_column_indices, d_row_offsets, d_row_indices1,
+                                 d_row_indices2, d_row_seg_st_offsets, d_B, d_C, nullptr, nullptr, stream1, stream2);
+}
+
+int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
+                          const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
+                          const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
+                          const void* d_plan, const int* h_plan_counts, void* stream1, void* stream2)
 {
     (void)k;
     constexpr int kKnown = RODE_SPMM_WHOLE_LISTS | RODE_SPMM_ONLY_BLOCK | RODE_SPMM_ONLY_RESIDUE;
@@ -109,19 +151,21 @@ int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const v
     if (m1 == 0 && m2 == 0) return hipSuccess;
     if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
     hipStream_t s1 = as_stream(stream1), s2 = as_stream(stream2);
+    rode::PlanRef plan;
+    if (!plan_ref(d_plan, h_plan_counts, m2, plan)) return hipErrorInvalidValue;
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
                                         d_column_indices, static_cast<const float*>(d_values),
-                                        static_cast<const float*>(d_B), static_cast<float*>(d_C), flags, s1, s2);
+                                        static_cast<const float*>(d_B), static_cast<float*>(d_C), flags, plan, s1, s2);
     case RODE_DENSE_F16:
         return rode::spmm_launch<__half>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets,
                                          d_row_offsets, d_column_indices, static_cast<const float*>(d_values),
-                                         static_cast<const __half*>(d_B), static_cast<float*>(d_C), flags, s1, s2);
+                                         static_cast<const __half*>(d_B), static_cast<float*>(d_C), flags, plan, s1, s2);
     case RODE_DENSE_F64:
         return rode::spmm_launch<double>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets,
                                          d_row_offsets, d_column_indices, static_cast<const double*>(d_values),
-                                         static_cast<const double*>(d_B), static_cast<double*>(d_C), flags, s1, s2);
+                                         static_cast<const double*>(d_B), static_cast<double*>(d_C), flags, plan, s1, s2);
     default: return hipErrorInvalidValue;
     }
 }
@@ -160,18 +204,42 @@ int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const
                             d_row_indices2, d_row_seg_st_offsets, d_B_half, d_C, stream1, stream2);
 }
 
-int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,
-                       const int* d_st_offsets, const int* d_row_offsets, const int* d_column_indices,
-                       const float* d_values, const float* d_lhs_matrix, const float* d_rhs_matrix, float* d_out,
-                       void* stream1, void* stream2)
+int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d_row_indices_block,
+                           const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
+                           const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
+                           const void* d_rhs_matrix, float* d_out, const void* d_plan, const int* h_plan_counts,
+                           void* stream1, void* stream2)
 {
     (void)n;
     if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
     if (m1 == 0 && m2 == 0) return hipSuccess;
     if (!aligned16(d_lhs_matrix) || !aligned16(d_rhs_matrix)) return hipErrorInvalidValue;
-    return rode::sddmm_launch<float>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
-                                     d_row_offsets, d_column_indices, d_values, d_lhs_matrix, d_rhs_matrix, d_out,
-                                     as_stream(stream1), as_stream(stream2));
+    rode::PlanRef plan;
+    if (!plan_ref(d_plan, h_plan_counts, m2, plan)) return hipErrorInvalidValue;
+    switch (dtype) {
+    case RODE_DENSE_F32:
+        return rode::sddmm_launch<float>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
+                                         d_row_offsets, d_column_indices, d_values,
+                                         static_cast<const float*>(d_lhs_matrix), static_cast<const float*>(d_rhs_matrix),
+                                         d_out, plan, as_stream(stream1), as_stream(stream2));
+    case RODE_DENSE_F16:
+        return rode::sddmm_launch<__half>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
+                                          d_row_offsets, d_column_indices, d_values,
+                                          static_cast<const __half*>(d_lhs_matrix),
+                                          static_cast<const __half*>(d_rhs_matrix), d_out, plan, as_stream(stream1),
+                                          as_stream(stream2));
+    default: return hipErrorInvalidValue;
+    }
+}
+
+int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,
+                       const int* d_st_offsets, const int* d_row_offsets, const int* d_column_indices,
+                       const float* d_values, const float* d_lhs_matrix, const float* d_rhs_matrix, float* d_out,
+                       void* stream1, void* stream2)
+{
+    return rode_hip_sddmm_planned(RODE_DENSE_F32, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
+                                  d_row_offsets, d_column_indices, d_values, d_lhs_matrix, d_rhs_matrix, d_out, nullptr,
+                                  nullptr, stream1, stream2);
 }
 
 int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,
@@ -179,14 +247,9 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
                        const float* d_values, const void* d_lhs_half, const void* d_rhs_half, float* d_out,
                        void* stream1, void* stream2)
 {
-    (void)n;
-    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
-    if (m1 == 0 && m2 == 0) return hipSuccess;
-    if (!aligned16(d_lhs_half) || !aligned16(d_rhs_half)) return hipErrorInvalidValue;
-    return rode::sddmm_launch<__half>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
-                                      d_row_offsets, d_column_indices, d_values,
-                                      static_cast<const __half*>(d_lhs_half), static_cast<const __half*>(d_rhs_half),
-                                      d_out, as_stream(stream1), as_stream(stream2));
+    return rode_hip_sddmm_planned(RODE_DENSE_F16, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
+                                  d_row_offsets, d_column_indices, d_values, d_lhs_half, d_rhs_half, d_out, nullptr,
+                                  nullptr, stream1, stream2);
 }
 
 int rode_hip_csr_softmax_f32(int M, const int* d_row_offsets, const float* d_in, float* d_out, float scale,

@@ -93,6 +93,12 @@ struct DenseVec<float> {
         const float4 v = *reinterpret_cast<const float4*>(p);
         out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
     }
+    // the same 16 bytes, already in registers (e.g. read back from an LDS copy of the row)
+    __device__ __forceinline__ static void unpack(const uint4& raw, float (&out)[4])
+    {
+        out[0] = __uint_as_float(raw.x); out[1] = __uint_as_float(raw.y);
+        out[2] = __uint_as_float(raw.z); out[3] = __uint_as_float(raw.w);
+    }
 };
 
 template <>
@@ -112,7 +118,10 @@ struct DenseVec<__half> {
     static constexpr int kElems = 8;
     __device__ __forceinline__ static void load(const __half* p, float (&out)[8])
     {
-        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        unpack(*reinterpret_cast<const uint4*>(p), out);
+    }
+    __device__ __forceinline__ static void unpack(const uint4& raw, float (&out)[8])
+    {
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {

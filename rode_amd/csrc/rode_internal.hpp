@@ -25,17 +25,40 @@ template <> struct SpmmAcc<double> { using type = double; };
 // flags: the RODE_SPMM_* bits of the C ABI
 constexpr int kSpmmWholeLists = 1, kSpmmOnlyBlock = 2, kSpmmOnlyResidue = 4;
 
+// A locality plan (rode_plan.hip): device array, and optionally a host copy of its four
+// header ints (chunk counts), with which launches that have nothing to do are left out.
+struct PlanRef {
+    const int* dev = nullptr;
+    const int* host_counts = nullptr;
+};
+
+size_t window_plan_ints(int m2);
+hipError_t window_plan_launch(int m2, int dense_rows, const int* residue_rows, const int* row_ptr, const int* col,
+                              int* plan, hipStream_t stream);
+
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                        const int* row_ptr, const int* col, const typename SpmmAcc<T>::type* val, const T* B,
-                       typename SpmmAcc<T>::type* C, int flags, hipStream_t s1, hipStream_t s2);
+                       typename SpmmAcc<T>::type* C, int flags, PlanRef plan, hipStream_t s1, hipStream_t s2);
+
+// the window kernel of SpMM over the planned chunks of the residue list (T = float or __half)
+template <typename T>
+hipError_t spmm_window_launch(int m2, int n, int owned_slots, const int* residue_rows, const int* row_ptr,
+                              const int* col, const float* val, const T* B, float* C, const int* plan,
+                              hipStream_t stream);
 
 hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, void* C, hipStream_t stream);
 
 template <typename T>
 hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int* residue_rows, const int* st_off,
                         const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs,
-                        float* out, hipStream_t s1, hipStream_t s2);
+                        float* out, PlanRef plan, hipStream_t s1, hipStream_t s2);
+
+// the window kernel of SDDMM over the planned chunks of the residue list
+template <typename T>
+hipError_t sddmm_window_launch(int m2, int k, const int* residue_rows, const int* row_ptr, const int* col,
+                               const float* val, const T* lhs, const T* rhs, float* out, const int* plan,
+                               hipStream_t stream);
 
 hipError_t csr_softmax_launch(int M, const int* row_ptr, const float* in, float* out, float scale,
                               hipStream_t stream);

@@ -1,0 +1,145 @@
+// Work items of the RoDe kernels: which nonzero slots a block-segment wave and a
+// residue lane group process.  One statement of the index arithmetic, shared by the
+// standard kernels and the window kernels, so that both always agree on who owns
+// what (reference arithmetic: RoDe_SpMM/RoDeSpmm.cu:71-82, 210-234;
+// RoDe_SDDMM/RoDeSddmm.cu:33-58, 237-243).
+#pragma once
+#include "rode_device.hpp"
+
+namespace rode {
+
+// Aligned slot range [base, base + cnt) of one block work item; the first `mask` slots
+// belong to the previous row (unaligned start) and must not contribute.
+struct BlockItem {
+    int row, base, mask, cnt;
+};
+
+// Consecutive segments of one row whose starts fall into the same window of MERGE slots
+// are handled by the wave of the first of them (the "leader"); with segments of MERGE
+// slots or more every segment is its own leader.  Returns false for a follower.  All
+// 64 lanes of the wave must call this together.  st_off[m1] must exist: the sentinel, or
+// the next segment when the lists are a slice.
+template <int MERGE>
+__device__ __forceinline__ bool merged_leader(int seg, int m1, int lane, int row, int row_start, int row_end,
+                                              const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                                              BlockItem& it)
+{
+    const int start = st_off[seg];
+    const int row_base = row_start - (row_start & (kVecLen - 1));
+    const int window = (start - row_base) / MERGE;
+    if (seg > 0 && block_rows[seg - 1] == row && (st_off[seg - 1] - row_base) / MERGE == window) return false;
+    // the next leader: the first later segment of another row or another window
+    const int probe = seg + 1 + lane;
+    const bool follower = probe < m1 && block_rows[probe] == row && (st_off[probe] - row_base) / MERGE == window;
+    const unsigned long long not_follower = ~__ballot(follower);
+    const int next = seg + 1 + (not_follower ? __builtin_ctzll(not_follower) : kWave);
+    // end of the row's block part, or the start of the next leader if that comes first
+    // (another row's start, or the sentinel, lies past block_end)
+    const int block_end = row_base + (row_end - row_base) / kBlockItems * kBlockItems;
+    const int end = min(block_end, st_off[next]);
+    it.row = row;
+    it.mask = start & (kVecLen - 1);
+    it.base = start - it.mask;
+    it.cnt = end - it.base;
+    return true;
+}
+
+constexpr int kSddmmMergeSlots = 128;
+constexpr int kSpmmMergeSlots = 512;
+
+// SDDMM: merging needs no promise from the caller (an output computed twice at a slice
+// boundary is harmless).
+__device__ __forceinline__ bool sddmm_block_item(int seg, int m1, int lane, const int* __restrict__ block_rows,
+                                                 const int* __restrict__ st_off, const int* __restrict__ row_ptr,
+                                                 BlockItem& it)
+{
+    const int row = block_rows[seg];
+    return merged_leader<kSddmmMergeSlots>(seg, m1, lane, row, row_ptr[row], row_ptr[row + 1], block_rows, st_off, it);
+}
+
+// SpMM.  owned_slots > 0 means that the caller promised complete lists: a row of at
+// most owned_slots aligned slots is then summed whole - all its segments and its tail -
+// by the wave of its first segment (one update of C), longer rows are merged into
+// leaders.  owned_slots == 0: every segment on its own, rounded to whole 32-slot units
+// as in RoDeSpmm.cu:210-234.
+__device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots, int lane,
+                                                const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                                                const int* __restrict__ row_ptr, BlockItem& it)
+{
+    const int row = block_rows[seg];
+    const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
+    if (row_end - row_start + (row_start & (kVecLen - 1)) <= owned_slots) {
+        if (seg > 0 && block_rows[seg - 1] == row) return false;
+        it.row = row;
+        it.mask = row_start & (kVecLen - 1);
+        it.base = row_start - it.mask;
+        it.cnt = row_end - it.base;
+        return true;
+    }
+    if (owned_slots > 0)
+        return merged_leader<kSpmmMergeSlots>(seg, m1, lane, row, row_start, row_end, block_rows, st_off, it);
+    const int start = st_off[seg];
+    const int end = min(row_end, st_off[seg + 1]);
+    it.row = row;
+    it.mask = start & (kVecLen - 1);
+    it.base = start - it.mask;
+    it.cnt = (end - start + it.mask) / kBlockItems * kBlockItems;
+    return true;
+}
+
+// Slots [first, first + cnt) of one residue row: with N = len + (start & 3), rows with
+// N >= 32 keep only their last N % 32 slots, starting at (start & ~3) + floor(N / 32) * 32,
+// and are accumulated into (the row also has block segments); shorter rows are taken
+// whole and stored.
+struct ResidueItem {
+    int first, cnt, aligned; // aligned = N
+    bool accumulate;
+};
+
+__device__ __forceinline__ ResidueItem residue_item(int row, const int* __restrict__ row_ptr)
+{
+    const int s = row_ptr[row], e = row_ptr[row + 1];
+    const int pad = s & (kVecLen - 1);
+    ResidueItem it;
+    it.aligned = e - s + pad;
+    it.accumulate = it.aligned >= kBlockItems;
+    it.first = it.accumulate ? (s - pad) + it.aligned / kBlockItems * kBlockItems : s;
+    it.cnt = it.accumulate ? it.aligned % kBlockItems : e - s;
+    return it;
+}
+
+// ---- locality plan --------------------------------------------------------------
+// A plan cuts the residue list into chunks of consecutive entries and says, for every
+// chunk, whether the dense rows its nonzeros reference cluster in a window of at most
+// kResidueWindowRowsMax consecutive rows (banded matrices).  A chunk with a window is
+// processed by the window kernels (the window of the dense operand is staged in LDS once
+// per column tile and every slot that falls into it reads LDS instead of gathering from
+// L2); the standard residue kernels skip it.  Slots outside the window are still gathered
+// from memory, so a plan never changes which nonzeros contribute - only where their dense
+// rows are read from.  Layout of the int array:
+//   [0] residue chunks  [1] residue chunks with a window  [2], [3] zero
+//   then one WindowDesc per residue chunk.
+constexpr int kPlanHeaderInts = 4;
+constexpr int kPlanDescInts = 4;
+constexpr int kPlanResidueChunk = 128;     // residue-list entries per chunk
+constexpr int kResidueWindowRowsMax = 512; // dense rows of one window
+
+// Window of one chunk: dense rows [w0, w0 + wn); wn == 0: no window.  hits / slots: how
+// many of the chunk's nonzero slots fall into the window / exist (statistics of the plan).
+struct WindowDesc {
+    int w0, wn, hits, slots;
+};
+
+__host__ __device__ inline int plan_residue_chunks(int m2) { return (m2 + kPlanResidueChunk - 1) / kPlanResidueChunk; }
+__host__ __device__ inline size_t plan_ints(int m2)
+{
+    return kPlanHeaderInts + (size_t)kPlanDescInts * plan_residue_chunks(m2);
+}
+
+__device__ __forceinline__ WindowDesc plan_residue_desc(const int* __restrict__ plan, int chunk)
+{
+    const int4 v = *reinterpret_cast<const int4*>(plan + kPlanHeaderInts + kPlanDescInts * chunk);
+    return WindowDesc{v.x, v.y, v.z, v.w};
+}
+
+} // namespace rode

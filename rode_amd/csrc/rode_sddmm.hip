@@ -18,7 +18,7 @@
 //   * residue kernel: each group of LPR lanes takes one residue row (< 32 slots),
 //     so a wave works on 64 / LPR rows at once (2 at K=128 fp32, 8 at K=32):
 //     short rows are latency-bound and need many rows in flight per wave.
-#include "rode_device.hpp"
+#include "rode_items.hpp"
 #include "rode_internal.hpp"
 
 namespace rode {
@@ -109,8 +109,6 @@ __device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int ro
     }
 }
 
-constexpr int kMergeSlots = 128;
-
 // One wave per block segment.  Segment s covers the aligned slots
 // [base, base + cnt) with base = st_off[s] & ~3 and cnt = floor((len + mask) / 32) * 32
 // (RoDeSddmm.cu:35-54); the first `mask` slots belong to the previous row and are
@@ -128,28 +126,14 @@ sddmm_block_kernel(int m1, int k, const int* __restrict__ block_rows, const int*
     if (seg >= m1) return;
 
     // Consecutive segments of one row whose starts fall into the same window of
-    // kMergeSlots slots are handled by the wave of the first of them, so a decomposition
+    // kSddmmMergeSlots slots are handled by the wave of the first of them, so a decomposition
     // with short segments (32 in the reference's K=128 parameter set) still fills whole
-    // 64-slot steps and loads the lhs row once.  Segments of kMergeSlots or more are
-    // unaffected.  (Outputs are pure functions of the inputs, so this is safe even when a
-    // caller passes a slice of the lists: the worst case is an output computed twice.)
-    const int row = block_rows[seg];
-    const int start = st_off[seg];
-    const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
-    const int row_base = row_start - (row_start & (kVecLen - 1));
-    const int window = (start - row_base) / kMergeSlots;
-    if (seg > 0 && block_rows[seg - 1] == row && (st_off[seg - 1] - row_base) / kMergeSlots == window) return;
-    const int probe = seg + 1 + lane; // the next leader: first later segment of another row or window
-    const bool follower = probe < m1 && block_rows[probe] == row && (st_off[probe] - row_base) / kMergeSlots == window;
-    const unsigned long long not_follower = ~__ballot(follower);
-    const int next = seg + 1 + (not_follower ? __builtin_ctzll(not_follower) : kWave);
-    // end of the row's block part, or the start of the next leader if that comes first
-    // (st_off[m1] exists: the sentinel, or the next segment when the lists are a slice)
-    const int block_end = row_base + (row_end - row_base) / kBlockItems * kBlockItems;
-    const int end = min(block_end, st_off[next]);
-    const int mask = start & (kVecLen - 1);
-    const int base = start - mask;
-    const int cnt = end - base;
+    // 64-slot steps and loads the lhs row once.  Longer segments are unaffected.  (Outputs
+    // are pure functions of the inputs, so this is safe even when a caller passes a slice of
+    // the lists: the worst case is an output computed twice.)
+    BlockItem it;
+    if (!sddmm_block_item(seg, m1, lane, block_rows, st_off, row_ptr, it)) return;
+    const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
 
     float a[NS][S::kVec];
     load_lhs_slice<T, KT, NS, EDGE>(lhs, row, k, lane, a);
@@ -181,7 +165,7 @@ template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
 sddmm_residue_kernel(int m2, int k, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
                      const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
-                     const T* __restrict__ rhs, float* __restrict__ out)
+                     const T* __restrict__ rhs, float* __restrict__ out, const int* __restrict__ plan)
 {
     using S = SddmmShape<T, KT>;
     constexpr int VEC = S::kVec, LPR = S::kLpr;
@@ -193,16 +177,11 @@ sddmm_residue_kernel(int m2, int k, const int* __restrict__ residue_rows, const 
     const int group = lane / LPR, ls = lane % LPR;
     const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * RPW + group;
     if (item >= m2) return;
+    if (plan && plan_residue_desc(plan, item / kPlanResidueChunk).wn > 0) return; // the window kernel has this chunk
 
     const int row = residue_rows[item];
-    const int s = row_ptr[row], e = row_ptr[row + 1];
-    const int pad = s & (kVecLen - 1);
-    const int N = e - s + pad;
-    int first = s, cnt = e - s;
-    if (N >= kBlockItems) {
-        first = (s - pad) + N / kBlockItems * kBlockItems;
-        cnt = N % kBlockItems;
-    }
+    const ResidueItem it = residue_item(row, row_ptr);
+    const int first = it.first, cnt = it.cnt;
     if (cnt <= 0) return; // an empty, unaligned row is listed as a residue but owns no slot
 
     int* my_cols = lds + (wave * RPW + group) * kBlockItems;
@@ -264,46 +243,60 @@ inline int grid_for_waves(long long nwaves)
 template <typename T, int KT, int NS, bool EDGE>
 hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* residue_rows, const int* st_off,
                   const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
-                  hipStream_t s1, hipStream_t s2)
+                  PlanRef plan, hipStream_t s1, hipStream_t s2)
 {
     constexpr int RPW = kWave / SddmmShape<T, KT>::kLpr;
     const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0) return hipErrorInvalidConfiguration;
+    // With a host copy of the plan's header, a kernel that would find every chunk taken by
+    // the other one is not launched at all.
+    bool standard_residue = true, window_residue = plan.dev != nullptr;
+    if (plan.dev && plan.host_counts) {
+        standard_residue = plan.host_counts[1] < plan.host_counts[0];
+        window_residue = plan.host_counts[1] > 0;
+    }
     if (m1 > 0) {
         sddmm_block_kernel<T, KT, NS, EDGE><<<g1, kWgThreads, 0, s1>>>(
             m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
     }
-    if (m2 > 0) {
+    if (m2 > 0 && standard_residue) {
         sddmm_residue_kernel<T, KT, NS, EDGE><<<g2, kWgThreads, 0, s2>>>(
-            m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out);
+            m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev);
     }
-    return hipGetLastError();
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess && m2 > 0 && window_residue)
+        e = sddmm_window_launch<T>(m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev, s2);
+    return e;
 }
 
 template <typename T, int KT, int NS>
 hipError_t launch_edge(bool edge, int m1, int m2, int k, const int* block_rows, const int* residue_rows,
                        const int* st_off, const int* row_ptr, const int* col, const float* val, const T* lhs,
-                       const T* rhs, float* out, hipStream_t s1, hipStream_t s2)
+                       const T* rhs, float* out, PlanRef plan, hipStream_t s1, hipStream_t s2)
 {
     return edge ? launch<T, KT, NS, true>(m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out,
-                                          s1, s2)
+                                          plan, s1, s2)
                 : launch<T, KT, NS, false>(m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs,
-                                           out, s1, s2);
+                                           out, plan, s1, s2);
 }
 
 } // namespace
 
 // k: any positive multiple of the 128-bit vector width (4 for fp32, 8 for fp16) up to 512.
-// 32, 64 and 128 (the reference has 32 and 128) run without any bounds test.
+// 32, 64 and 128 (the reference has 32 and 128) run without any bounds test.  Chunks of the
+// residue list for which `plan` holds a window go to the window kernel when a dense row
+// is wider than one 128-byte tile (with a single tile the window is not reused often
+// enough to repay its staging).
 template <typename T>
 hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int* residue_rows, const int* st_off,
                         const int* row_ptr, const int* col, const float* val, const T* lhs, const T* rhs,
-                        float* out, hipStream_t s1, hipStream_t s2)
+                        float* out, PlanRef plan, hipStream_t s1, hipStream_t s2)
 {
     if (k <= 0 || k % DenseVec<T>::kElems != 0 || k > 512) return hipErrorInvalidValue;
+    if ((size_t)k * sizeof(T) <= 128) plan = PlanRef{};
 #define RODE_SDDMM_CASE(KT, NS)                                                                                   \
     return launch_edge<T, KT, NS>(k != (KT) * (NS), m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, \
-                                  lhs, rhs, out, s1, s2)
+                                  lhs, rhs, out, plan, s1, s2)
     if (k <= 32) RODE_SDDMM_CASE(32, 1);
     if (k <= 64) RODE_SDDMM_CASE(64, 1);
     if (k <= 128) RODE_SDDMM_CASE(128, 1);
@@ -314,8 +307,8 @@ hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int*
 }
 
 template hipError_t sddmm_launch<float>(int, int, int, const int*, const int*, const int*, const int*, const int*,
-                                        const float*, const float*, const float*, float*, hipStream_t, hipStream_t);
+                                        const float*, const float*, const float*, float*, PlanRef, hipStream_t, hipStream_t);
 template hipError_t sddmm_launch<__half>(int, int, int, const int*, const int*, const int*, const int*, const int*,
-                                         const float*, const __half*, const __half*, float*, hipStream_t, hipStream_t);
+                                         const float*, const __half*, const __half*, float*, PlanRef, hipStream_t, hipStream_t);
 
 } // namespace rode

@@ -25,7 +25,7 @@
 // segment) are neutralised with value 0 *and* the column of the first real slot,
 // so a non-finite B row can never leak into a row that does not reference it
 // (the reference multiplies B[0, :] by zero there, RoDeSpmm.cu:271-274).
-#include "rode_device.hpp"
+#include "rode_items.hpp"
 #include "rode_internal.hpp"
 
 #include <type_traits>
@@ -35,15 +35,14 @@ namespace rode {
 namespace {
 
 // Rows of at most `owned_slots` aligned slots (and at least 32, i.e. rows that have block
-// segments) are summed by a single wave of the block kernel.  The launcher passes 1024
-// when the caller promises that the two lists are the complete decomposition of the
-// matrix (a row's first segment and its residue entry are then both in this call) and
-// there are enough block segments to keep every CU busy anyway; else 0 (every work item
-// on its own wave: small matrices need the parallelism more than they mind the extra
-// atomics).
+// segments) are summed by a single wave of the block kernel (spmm_block_item).  The
+// launcher passes kOwnedRowSlots when the caller promises that the two lists are the
+// complete decomposition of the matrix (a row's first segment and its residue entry are
+// then both in this call) and there are enough block segments to keep every CU busy
+// anyway; else 0 (every work item on its own wave: small matrices need the parallelism
+// more than they mind the extra atomics).
 constexpr int kOwnedRowSlots = 1024;
 constexpr int kOwnedMinSegments = 16384;
-constexpr int kMergeSlots = 512; // under the same promise, short segments of a longer row are merged up to this many slots
 
 template <typename T, int TN>
 struct SpmmShape {
@@ -127,46 +126,9 @@ spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int seg = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (seg >= m1) return;
-
-    const int row = block_rows[seg];
-    const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
-    int mask, base, cnt;
-    if (row_end - row_start + (row_start & (kVecLen - 1)) <= owned_slots) {
-        // A moderately long row is summed by ONE wave, the one of its first segment:
-        // all its segments and its tail, one update of C instead of one per work item.
-        // The residue kernel skips such rows by the same test.
-        if (seg > 0 && block_rows[seg - 1] == row) return;
-        mask = row_start & (kVecLen - 1);
-        base = row_start - mask;
-        cnt = row_end - base;
-    } else if (owned_slots > 0) {
-        // Long row, complete lists: consecutive segments of the row whose starts fall into the
-        // same window of kMergeSlots slots are summed by the wave of the first of them (the
-        // "leader"), so a decomposition with short segments (the reference's 32) does not
-        // multiply the atomic updates of C.  With segments of kMergeSlots or more every
-        // segment is its own leader and nothing changes.
-        const int start = st_off[seg];
-        const int row_base = row_start - (row_start & (kVecLen - 1));
-        const int window = (start - row_base) / kMergeSlots;
-        if (seg > 0 && block_rows[seg - 1] == row && (st_off[seg - 1] - row_base) / kMergeSlots == window) return;
-        // the next leader is the first later segment of another row or another window
-        const int probe = seg + 1 + lane;
-        const bool follower = probe < m1 && block_rows[probe] == row && (st_off[probe] - row_base) / kMergeSlots == window;
-        const unsigned long long not_follower = ~__ballot(follower); // 64 lanes cover kMergeSlots / 32 = 16 segments
-        const int followers = not_follower ? __builtin_ctzll(not_follower) : kWave;
-        const int next = seg + 1 + followers;
-        const int block_end = row_base + (row_end - row_base) / kBlockItems * kBlockItems; // end of the row's block part
-        const int end = min(block_end, st_off[next]); // another row's start (or the sentinel) lies past block_end
-        mask = start & (kVecLen - 1);
-        base = start - mask;
-        cnt = end - base;
-    } else {
-        const int start = st_off[seg];
-        const int end = min(row_end, st_off[seg + 1]);
-        mask = start & (kVecLen - 1);
-        base = start - mask;
-        cnt = (end - start + mask) / kBlockItems * kBlockItems;
-    }
+    BlockItem it;
+    if (!spmm_block_item(seg, m1, owned_slots, lane, block_rows, st_off, row_ptr, it)) return;
+    const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
 
     const int ls = lane % LPR, group = lane / LPR;
     const int tile = blockIdx.y * TN;
@@ -217,9 +179,10 @@ spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_
 // group walks its row's slot quads one after the other, no cross-lane reduction.
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
-                    const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
-                    const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C)
+spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ residue_rows,
+                    const int* __restrict__ row_ptr, const int* __restrict__ col,
+                    const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
+                    typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
     using S = SpmmShape<T, TN>;
     using A = typename S::Acc;
@@ -233,17 +196,13 @@ spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ resi
     const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * RPW + group;
     if (item >= m2) return;
 
+    if (plan && plan_residue_desc(plan, item / kPlanResidueChunk).wn > 0) return; // the window kernel has this chunk
+
     const int row = residue_rows[item];
-    const int s = row_ptr[row], e = row_ptr[row + 1];
-    const int pad = s & (kVecLen - 1);
-    const int N = e - s + pad;
-    int first = s, cnt = e - s;
-    const bool accumulate = N >= kBlockItems; // the row also has block segments
-    if (accumulate) {
-        if (N <= owned_slots) return; // summed entirely, tail included, by the block kernel
-        first = (s - pad) + N / kBlockItems * kBlockItems;
-        cnt = N % kBlockItems;
-    }
+    const ResidueItem it = residue_item(row, row_ptr);
+    const bool accumulate = it.accumulate; // the row also has block segments
+    if (accumulate && it.aligned <= owned_slots) return; // summed entirely, tail included, by the block kernel
+    const int first = it.first, cnt = it.cnt;
 
     const int tile = blockIdx.y * TN;
     const bool col_ok = !EDGE || tile + ls * VEC < n;
@@ -321,35 +280,50 @@ inline int grid_for_waves(long long nwaves)
 template <typename T, int TN, bool EDGE>
 hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                   const int* row_ptr, const int* col, const typename DenseVec<T>::Acc* val, const T* B,
-                  typename DenseVec<T>::Acc* C, int flags, hipStream_t s1, hipStream_t s2)
+                  typename DenseVec<T>::Acc* C, int flags, PlanRef plan, hipStream_t s1, hipStream_t s2)
 {
     const int tiles = (n + TN - 1) / TN;
     const int owned_slots = (flags & kSpmmWholeLists) && m1 >= kOwnedMinSegments ? kOwnedRowSlots : 0;
     constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
     const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0 || tiles > 65535) return hipErrorInvalidConfiguration;
+    // With a host copy of the plan's header, a kernel that would find every chunk taken by
+    // the other one is not launched at all.
+    bool standard_residue = true, window_residue = plan.dev != nullptr;
+    if (plan.dev && plan.host_counts) {
+        standard_residue = plan.host_counts[1] < plan.host_counts[0];
+        window_residue = plan.host_counts[1] > 0;
+    }
     if (m1 > 0 && !(flags & kSpmmOnlyResidue)) {
         dim3 grid(g1, tiles);
         spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, owned_slots, block_rows, st_off, row_ptr, col,
                                                                     val, B, C);
     }
+    hipError_t e = hipGetLastError();
     if (m2 > 0 && !(flags & kSpmmOnlyBlock)) {
-        dim3 grid(g2, tiles);
-        spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, residue_rows, row_ptr, col, val,
-                                                                      B, C);
+        if (standard_residue) {
+            dim3 grid(g2, tiles);
+            spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, residue_rows, row_ptr, col,
+                                                                          val, B, C, plan.dev);
+            e = hipGetLastError();
+        }
+        if constexpr (!std::is_same<T, double>::value) {
+            if (e == hipSuccess && window_residue)
+                e = spmm_window_launch<T>(m2, n, owned_slots, residue_rows, row_ptr, col, val, B, C, plan.dev, s2);
+        }
     }
-    return hipGetLastError();
+    return e;
 }
 
 template <typename T, int TN>
 hipError_t launch_edge(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                        const int* row_ptr, const int* col, const typename DenseVec<T>::Acc* val, const T* B,
-                       typename DenseVec<T>::Acc* C, int flags, hipStream_t s1, hipStream_t s2)
+                       typename DenseVec<T>::Acc* C, int flags, PlanRef plan, hipStream_t s1, hipStream_t s2)
 {
     return n % TN ? launch<T, TN, true>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C,
-                                        flags, s1, s2)
+                                        flags, plan, s1, s2)
                   : launch<T, TN, false>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C,
-                                         flags, s1, s2);
+                                         flags, plan, s1, s2);
 }
 
 } // namespace
@@ -357,14 +331,18 @@ hipError_t launch_edge(int m1, int m2, int n, const int* block_rows, const int* 
 // n: any positive multiple of the 128-bit vector width (4 fp32, 8 fp16, 2 fp64).  The
 // dense row is cut into tiles of 32, 64 or 128 columns (at most 32 lanes per tile row);
 // the tile width with the least padding wins, the widest on a tie.  Multiples of 32 (all
-// the reference supports) run without any bounds test.
+// the reference supports) run without any bounds test.  Chunks of the residue list for
+// which `plan` holds a window go to the window kernel (fp32 and fp16 operands wider than
+// one 128-byte tile; fp64 and narrower operands ignore the plan: with a single tile the
+// window is not reused often enough to repay its staging).
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                        const int* row_ptr, const int* col, const typename SpmmAcc<T>::type* val, const T* B,
-                       typename SpmmAcc<T>::type* C, int flags, hipStream_t s1, hipStream_t s2)
+                       typename SpmmAcc<T>::type* C, int flags, PlanRef plan, hipStream_t s1, hipStream_t s2)
 {
     static_assert(std::is_same<typename SpmmAcc<T>::type, typename DenseVec<T>::Acc>::value, "accumulation type");
     if (n <= 0 || n % DenseVec<T>::kElems != 0) return hipErrorInvalidValue;
+    if (std::is_same<T, double>::value || (size_t)n * sizeof(T) <= 128) plan = PlanRef{};
     constexpr int kMaxTile = 32 * DenseVec<T>::kElems >= 128 ? 128 : 32 * DenseVec<T>::kElems;
     auto padded = [n](int tn) { return (n + tn - 1) / tn * tn; };
     int best = 32;
@@ -373,12 +351,12 @@ hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* 
     if constexpr (kMaxTile >= 128) {
         if (best == 128)
             return launch_edge<T, 128>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, flags,
-                                       s1, s2);
+                                       plan, s1, s2);
     }
     if (best == 64)
-        return launch_edge<T, 64>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, flags, s1,
-                                  s2);
-    return launch_edge<T, 32>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, flags, s1, s2);
+        return launch_edge<T, 64>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, flags, plan,
+                                  s1, s2);
+    return launch_edge<T, 32>(m1, m2, n, block_rows, residue_rows, st_off, row_ptr, col, val, B, C, flags, plan, s1, s2);
 }
 
 hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, void* C, hipStream_t stream)
@@ -393,10 +371,10 @@ hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, v
 }
 
 template hipError_t spmm_launch<float>(int, int, int, const int*, const int*, const int*, const int*, const int*,
-                                       const float*, const float*, float*, int, hipStream_t, hipStream_t);
+                                       const float*, const float*, float*, int, PlanRef, hipStream_t, hipStream_t);
 template hipError_t spmm_launch<__half>(int, int, int, const int*, const int*, const int*, const int*, const int*,
-                                        const float*, const __half*, float*, int, hipStream_t, hipStream_t);
+                                        const float*, const __half*, float*, int, PlanRef, hipStream_t, hipStream_t);
 template hipError_t spmm_launch<double>(int, int, int, const int*, const int*, const int*, const int*, const int*,
-                                        const double*, const double*, double*, int, hipStream_t, hipStream_t);
+                                        const double*, const double*, double*, int, PlanRef, hipStream_t, hipStream_t);
 
 } // namespace rode

@@ -34,8 +34,9 @@ class RoDeCSR:
 
     DEFAULT_CONFIG = {"seg_length": 512, "k_block": 32, "vec_len": 4}  # for a k that is not in CONFIGS
     MAX_K = 512
+    PLAN_MIN_CHUNKS = 512  # windowed chunks of 128 residue rows below which "auto" drops the plan
 
-    def __init__(self, row_offsets, column_indices, values, device, m, n, k=128, config=None):
+    def __init__(self, row_offsets, column_indices, values, device, m, n, k=128, config=None, locality="auto"):
         if not (isinstance(k, int) and 0 < k <= self.MAX_K and k % 4 == 0):
             raise ValueError(f"k must be a positive multiple of 4 up to {self.MAX_K} (the reference: 32 or 128), got {k}")
         self.m = m
@@ -54,6 +55,9 @@ class RoDeCSR:
         self.column_indices = column_indices.to(dtype=torch.int32, device=self.device).contiguous()
         self.values = values.to(dtype=torch.float32, device=self.device).contiguous()
         self.row_offsets = self.row_offsets_cpu.to(device=self.device)
+        if locality not in (True, False, "auto"):
+            raise ValueError(f'locality must be True, False or "auto", got {locality!r}')
+        self.locality = locality
         self._shared = {}  # per-pattern cache (the transposed pattern); with_values() copies share it
         self._preprocess()
 
@@ -67,6 +71,17 @@ class RoDeCSR:
         self.residue_indices = res
         self.m1 = m1
         self.m2 = m2
+        # Locality plan: chunks of the residue list whose dense rows cluster in a window that
+        # fits LDS (banded matrices) go to the window kernels.  Kept only when it pays:
+        # "auto" wants windows on at least half of the chunks and enough of them to fill the
+        # GPU twice (a few windowed chunks only add launches); True keeps any plan with a
+        # window; False makes none.
+        self.plan = None
+        if self.locality and m2 > 0:
+            plan = rode_sddmm_hip.window_plan(res, m2, self.row_offsets, self.column_indices, self.n)
+            enough = plan.windowed >= max(self.PLAN_MIN_CHUNKS, (plan.counts[0] + 1) // 2)
+            if plan.windowed > 0 and (self.locality is True or enough):
+                self.plan = plan
 
     def with_values(self, values):
         """The same pattern and decomposition with other values (no preprocessing is
@@ -93,7 +108,7 @@ class RoDeCSR:
             row_offsets_t = torch.zeros(self.n + 1, dtype=torch.int64, device=self.device)
             row_offsets_t[1:] = torch.cumsum(torch.bincount(cols, minlength=self.n), 0)
             csr_t = RoDeCSR(row_offsets_t.to(torch.int32), rows[perm].to(torch.int32), self.values.float()[perm],
-                            self.device, self.n, self.m, self.k, config=self.config)
+                            self.device, self.n, self.m, self.k, config=self.config, locality=self.locality)
             cached = (csr_t, perm)
             self._shared["transpose"] = cached
         csr_t, perm = cached
@@ -157,7 +172,7 @@ def rode_sddmm(sparse_matrix, lhs, rhs, values=None):
     return rode_sddmm_hip.sddmm_forward(
         sparse_matrix.block_indices, sparse_matrix.residue_indices, sparse_matrix.st_offsets,
         sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,
-        sparse_matrix.values, m, n, lhs.contiguous(), rhs.contiguous(), k)
+        sparse_matrix.values, m, n, lhs.contiguous(), rhs.contiguous(), k, plan=sparse_matrix.plan)
 
 
 def torch_sddmm_reference(sparse_csr, lhs_matrix, rhs_matrix):

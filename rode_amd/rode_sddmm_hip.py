@@ -9,6 +9,8 @@ Additions with no counterpart in the reference module: ``preprocess_device``
 (decomposition of a row pointer that already lives on the GPU, results stay on
 the GPU) and ``spmm_forward``.
 """
+import ctypes
+
 import torch
 
 from . import _lib
@@ -70,6 +72,53 @@ def preprocess_device(row_offsets, nnz, seg_length, k_block, vec_len):
     return blk[: max(n_blk, 1)].clone(), st[: n_blk + 1].clone(), res[: max(n_res, 1)].clone(), n_blk, n_res
 
 
+class WindowPlan:
+    """Locality plan of one decomposition (``rode_hip_window_plan``): the device array and
+    a host copy of its header ``[residue chunks, residue chunks with a window, 0, 0]``."""
+
+    def __init__(self, data, counts):
+        self.data = data
+        self.counts = counts                                   # list of 4 ints
+        self._header = (ctypes.c_int * 4)(*counts)             # what the C ABI reads
+
+    @property
+    def windowed(self):
+        return self.counts[1]
+
+    def descriptors(self):
+        """int32 array of shape (residue chunks, 4): first window row, window rows (0: none),
+        nonzeros inside the window, nonzeros of the chunk."""
+        return self.data.cpu().numpy()[4:].reshape(-1, 4)
+
+
+def window_plan(residue_indices, m2, row_offsets, column_indices, dense_rows):
+    """Locality plan for the residue list of one decomposition: which chunks of 128 residue
+    rows have their dense rows inside a window small enough for LDS.  ``dense_rows``: number
+    of columns of the sparse matrix.  Waits for the two small kernels (it returns the chunk
+    counts)."""
+    for t, name in ((residue_indices, "residue_indices"), (row_offsets, "row_offsets"),
+                    (column_indices, "column_indices")):
+        _check_input(t, name)
+        _check(t.dtype == torch.int32, f"{name} must be int32")
+    lib = _lib.load()
+    dev = row_offsets.device
+    nbytes = lib.rode_hip_window_plan_bytes(m2)
+    with torch.cuda.device(dev):
+        data = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
+        counts = (ctypes.c_int * 4)()
+        code = lib.rode_hip_window_plan(m2, dense_rows, residue_indices.data_ptr(), row_offsets.data_ptr(),
+                                        column_indices.data_ptr(), data.data_ptr(), nbytes, ctypes.addressof(counts),
+                                        _stream_handle(dev))
+    _lib.check(code, "rode_hip_window_plan")
+    return WindowPlan(data, list(counts))
+
+
+def _plan_args(plan):
+    if plan is None:
+        return None, None
+    return plan.data.data_ptr(), ctypes.addressof(plan._header)
+
+
 def preprocess(row_offsets, nnz, seg_length, k_block, vec_len):
     """``rode_sddmm_cuda.preprocess`` (``rode_sddmm_cuda.cu:54-131``): takes the CPU
     int32 row pointer and returns CPU tensors, as the reference does; the
@@ -91,14 +140,15 @@ def _dense_kind(lhs_matrix, rhs_matrix, lhs_name, rhs_name):
 
 
 def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, n,
-                  lhs_matrix, rhs_matrix, k_version):
+                  lhs_matrix, rhs_matrix, k_version, plan=None):
     """``rode_sddmm_cuda.sddmm_forward`` (``rode_sddmm_cuda.cu:136-249``).
 
     Differences from the reference, none of which changes a result: any k_version
     that is a multiple of 4 up to 512 (multiple of 8 for fp16) and fp16
     ``lhs_matrix``/``rhs_matrix`` (fp32 accumulate) are accepted too; the
     kernels are queued on PyTorch's current stream instead of two streams that
-    are created, synchronised and destroyed per call (``:203-246``).
+    are created, synchronised and destroyed per call (``:203-246``).  ``plan``: a
+    ``WindowPlan`` made from this very residue list, or None.
     """
     for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
                     (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
@@ -124,25 +174,27 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
     if m1 == 0 and m2 == 0:
         return out
     lib = _lib.load()
-    fn = lib.rode_hip_sddmm_f32 if kind == "f32" else lib.rode_hip_sddmm_f16
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
-        code = fn(m1, m2, n, k, block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
-                  row_offsets.data_ptr(), column_indices.data_ptr(), values.data_ptr(), lhs_matrix.data_ptr(),
-                  rhs_matrix.data_ptr(), out.data_ptr(), s, s)
-    _lib.check(code, "rode_hip_sddmm")
+        plan_dev, plan_counts = _plan_args(plan)
+        code = lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[kind], m1, m2, n, k, block_indices.data_ptr(),
+                                          residue_indices.data_ptr(), st_offsets.data_ptr(), row_offsets.data_ptr(),
+                                          column_indices.data_ptr(), values.data_ptr(), lhs_matrix.data_ptr(),
+                                          rhs_matrix.data_ptr(), out.data_ptr(), plan_dev, plan_counts, s, s)
+    _lib.check(code, "rode_hip_sddmm_planned")
     return out
 
 
 def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, k,
-                 dense_matrix, out=None, whole_lists=True):
+                 dense_matrix, out=None, whole_lists=True, plan=None):
     """C = A_csr @ dense_matrix through ``rode_hip_spmm_f32`` / ``_f16``
     (host API ``RoDe_SpMM/RoDeSpmm.h:4-8``).  ``dense_matrix`` is (k, n) with n a
     multiple of 4 (8 for fp16, 2 for fp64), fp32 / fp16 (fp32 ``values``) or fp64 (fp64 ``values``); the
     result is a new zero-initialised (m, n) tensor of the dtype of ``values``, or
     ``out`` accumulated in place the way the reference kernels do (long rows add,
     short rows overwrite).  ``whole_lists`` promises that the index tensors are the
-    complete decomposition (always true for a ``RoDeCSR``); pass False for a slice."""
+    complete decomposition (always true for a ``RoDeCSR``); pass False for a slice.
+    ``plan``: a ``WindowPlan`` made from these very lists, or None."""
     for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
                     (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
                     (values, "values"), (dense_matrix, "dense_matrix")):
@@ -178,9 +230,10 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     dtype = {torch.float32: 0, torch.float16: 1, torch.float64: 2}[dense_matrix.dtype]  # RODE_DENSE_*
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
-        code = lib.rode_hip_spmm_ex(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
-                                    values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
-                                    block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
-                                    dense_matrix.data_ptr(), out.data_ptr(), s, s)
-    _lib.check(code, "rode_hip_spmm_ex")
+        plan_dev, plan_counts = _plan_args(plan)
+        code = lib.rode_hip_spmm_planned(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
+                                         values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
+                                         block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
+                                         dense_matrix.data_ptr(), out.data_ptr(), plan_dev, plan_counts, s, s)
+    _lib.check(code, "rode_hip_spmm_planned")
     return out
