@@ -48,7 +48,8 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=3)
     p.add_argument("--workload", default="c4_powerlaw")
     p.add_argument("--k", type=int, default=128, help="dense width (SpMM n, SDDMM k)")
-    p.add_argument("--seg", type=int, default=0, help="segment length (0: the library's choice for this k)")
+    p.add_argument("--seg", type=int, default=0,
+                   help="segment length (0: picked from the row lengths by RoDeCSR.auto_config; -1: the fixed table)")
     p.add_argument("--dtype", default="f32", choices=["f32", "f16"], help="dense operand type (accumulation is fp32)")
     p.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (debugging only)")
     p.add_argument("--cpu-seconds", type=float, default=8.0, help="CPU time budget per operation of the baseline")
@@ -121,7 +122,7 @@ def main():
     t0 = time.time()
     m, n, row_ptr, col, val = workloads.config(args.workload, args.scale)
     nnz = int(row_ptr[-1])
-    cfg = None if args.seg == 0 else {"seg_length": args.seg, "k_block": 32, "vec_len": 4}
+    cfg = "auto" if args.seg == 0 else None if args.seg < 0 else {"seg_length": args.seg, "k_block": 32, "vec_len": 4}
     csr = RoDeCSR(torch.from_numpy(row_ptr), torch.from_numpy(col), torch.from_numpy(val), dev, m, n,
                   k if k in RoDeCSR.CONFIGS else 128, config=cfg, locality=False if args.no_plan else "auto")
     plan_dev, plan_counts = rode_sddmm_hip._plan_args(csr.plan)

@@ -17,10 +17,10 @@ struct BlockItem {
 // Consecutive segments of one row whose starts fall into the same window of MERGE slots
 // are handled by the wave of the first of them (the "leader"); with segments of MERGE
 // slots or more every segment is its own leader.  Returns false for a follower.  All
-// 64 lanes of the wave must call this together.  st_off[m1] must exist: the sentinel, or
-// the next segment when the lists are a slice.
-template <int MERGE>
-__device__ __forceinline__ bool merged_leader(int seg, int m1, int lane, int row, int row_start, int row_end,
+// 64 lanes of the wave must call this together (they probe the next 64 segments, so a
+// window may hold at most 64 followers: MERGE <= 64 x 32).  st_off[m1] must exist: the
+// sentinel, or the next segment when the lists are a slice.
+__device__ __forceinline__ bool merged_leader(int MERGE, int seg, int m1, int lane, int row, int row_start, int row_end,
                                               const int* __restrict__ block_rows, const int* __restrict__ st_off,
                                               BlockItem& it)
 {
@@ -54,7 +54,7 @@ __device__ __forceinline__ bool sddmm_block_item(int seg, int m1, int lane, cons
                                                  BlockItem& it)
 {
     const int row = block_rows[seg];
-    return merged_leader<kSddmmMergeSlots>(seg, m1, lane, row, row_ptr[row], row_ptr[row + 1], block_rows, st_off, it);
+    return merged_leader(kSddmmMergeSlots, seg, m1, lane, row, row_ptr[row], row_ptr[row + 1], block_rows, st_off, it);
 }
 
 // SpMM.  owned_slots > 0 means that the caller promised complete lists: a row of at
@@ -77,7 +77,7 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
         return true;
     }
     if (owned_slots > 0)
-        return merged_leader<kSpmmMergeSlots>(seg, m1, lane, row, row_start, row_end, block_rows, st_off, it);
+        return merged_leader(kSpmmMergeSlots, seg, m1, lane, row, row_start, row_end, block_rows, st_off, it);
     const int start = st_off[seg];
     const int end = min(row_end, st_off[seg + 1]);
     it.row = row;

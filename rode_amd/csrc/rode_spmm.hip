@@ -124,11 +124,25 @@ spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int seg = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
-    if (seg >= m1) return;
-    BlockItem it;
-    if (!spmm_block_item(seg, m1, owned_slots, lane, block_rows, st_off, row_ptr, it)) return;
-    const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
+    const int seg0 = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg;
+    const int seg = seg0 + wave;
+    // Do neighbouring segments of this workgroup belong to one row (a long row)?  Every
+    // wave finds the same answer.  If so, the waves add their sums up in LDS and the row
+    // of C gets one update per workgroup instead of one per segment.
+    bool shared_row = false;
+    {
+        int prev = -1;
+#pragma unroll
+        for (int i = 0; i < kWavesPerWg; ++i) {
+            const int r = seg0 + i < m1 ? block_rows[seg0 + i] : -2 - i;
+            shared_row = shared_row || r == prev;
+            prev = r;
+        }
+    }
+    BlockItem it{-1, 0, 0, 0};
+    const bool active = seg < m1 && spmm_block_item(seg, m1, owned_slots, lane, block_rows, st_off, row_ptr, it);
+    if (!active && !shared_row) return; // nobody waits for this wave
+    const int row = it.row, mask = it.mask, base = it.base, cnt = active ? it.cnt : 0;
 
     const int ls = lane % LPR, group = lane / LPR;
     const int tile = blockIdx.y * TN;
@@ -167,12 +181,29 @@ spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_
 
     // combine the lane groups, then spread the atomics over them
     constexpr int EPG = VEC / G > 0 ? VEC / G : 1; // elements each group adds
+    A total[VEC];
+#pragma unroll
+    for (int x = 0; x < VEC; ++x) total[x] = butterfly_sum<LPR, kWave>(acc[x]);
+    if (shared_row) {
+        __shared__ __attribute__((aligned(16))) A wg_sum[kWavesPerWg][TN];
+        __shared__ int wg_row[kWavesPerWg];
+        if (group == 0) {
+#pragma unroll
+            for (int x = 0; x < VEC; ++x) wg_sum[wave][ls * VEC + x] = total[x];
+        }
+        if (lane == 0) wg_row[wave] = active ? row : -1;
+        __syncthreads();
+        // the first wave of a run of equal rows takes the sums of the others
+        if (!active || (wave > 0 && wg_row[wave - 1] == row)) return;
+        for (int w = wave + 1; w < kWavesPerWg && wg_row[w] == row; ++w) {
+#pragma unroll
+            for (int x = 0; x < VEC; ++x) total[x] += wg_sum[w][ls * VEC + x];
+        }
+    }
     A* c_lane = C + (size_t)row * n + tile + ls * VEC;
 #pragma unroll
-    for (int x = 0; x < VEC; ++x) {
-        const A total = butterfly_sum<LPR, kWave>(acc[x]);
-        if (group == x / EPG && col_ok) atomicAdd(c_lane + x, total);
-    }
+    for (int x = 0; x < VEC; ++x)
+        if (group == x / EPG && col_ok) atomicAdd(c_lane + x, total[x]);
 }
 
 // One group of LPR lanes per residue row (tail selection: RoDeSpmm.cu:71-82); the

@@ -25,7 +25,8 @@ class RoDeCSR:
     # in 64-slot steps whatever its length, so one segment length serves every k;
     # 512 measured best on MI355X (short segments multiply the atomics of SpMM,
     # longer ones unbalance the waves).  Any multiple of 32 is valid, including the
-    # reference's values, through the ``config`` argument.
+    # reference's values, through the ``config`` argument; ``config="auto"`` picks the
+    # length from the matrix (``auto_config``).
     CONFIGS = {
         32: {"seg_length": 512, "k_block": 32, "vec_len": 4},
         64: {"seg_length": 512, "k_block": 32, "vec_len": 4},
@@ -44,6 +45,11 @@ class RoDeCSR:
         self.k = k
         self.nnz = values.numel()
         self.device = torch.device(device)
+        self.row_offsets_cpu = row_offsets.to(dtype=torch.int32, device="cpu").contiguous()
+        if isinstance(config, str):
+            if config != "auto":
+                raise ValueError(f'config must be a dict, None or "auto", got {config!r}')
+            config = self.auto_config(self.row_offsets_cpu)
         self.config = dict(config) if config is not None else dict(self.CONFIGS.get(k, self.DEFAULT_CONFIG))
         cfg = self.config
         if cfg.get("k_block") != 32 or cfg.get("vec_len") != 4 or cfg.get("seg_length", 0) <= 0 \
@@ -51,7 +57,6 @@ class RoDeCSR:
             # the kernels process 32-slot chunks from 4-aligned offsets, as the reference's do
             raise ValueError(f"config must have k_block=32, vec_len=4 and seg_length a positive multiple of 32, got {cfg}")
 
-        self.row_offsets_cpu = row_offsets.to(dtype=torch.int32, device="cpu").contiguous()
         self.column_indices = column_indices.to(dtype=torch.int32, device=self.device).contiguous()
         self.values = values.to(dtype=torch.float32, device=self.device).contiguous()
         self.row_offsets = self.row_offsets_cpu.to(device=self.device)
@@ -60,6 +65,34 @@ class RoDeCSR:
         self.locality = locality
         self._shared = {}  # per-pattern cache (the transposed pattern); with_values() copies share it
         self._preprocess()
+
+    @classmethod
+    def auto_config(cls, row_offsets):
+        """Segment length picked from the row lengths (the reference hard-codes one per k,
+        rode_sddmm.py:35-38).  Measured on MI355X over the five benchmark patterns:
+
+        * a small matrix (fewer than 16384 segments of 512 slots: not enough work items to
+          fill the GPU, and one wavefront per whole row is not used below that count) wants
+          short segments, 128: more wavefronts, and the kernels merge what is too short;
+        * otherwise a row should be a single segment where that is possible, so that one
+          wavefront sums it whole: the power of two that holds 90 % of the rows that have
+          block segments, between 512 and 2048 (attention masks: 1024; power-law graphs:
+          512 - their hub rows are cut into many segments either way, and the block kernel
+          adds the sums of neighbouring segments up before it updates the row of C).
+        """
+        ro = row_offsets.to(dtype=torch.int64, device="cpu")
+        start, lens = ro[:-1], ro[1:] - ro[:-1]
+        aligned = lens + start % 4
+        blocked = aligned[aligned >= 32]
+        seg = 512
+        if blocked.numel() > 0:
+            if int(((blocked + 511) // 512).sum()) < 16384:
+                seg = 128
+            else:
+                p90 = int(torch.quantile(blocked.to(torch.float64), 0.9, interpolation="higher"))
+                while seg < p90 and seg < 2048:
+                    seg *= 2
+        return {"seg_length": seg, "k_block": 32, "vec_len": 4}
 
     def _preprocess(self):
         """Row decomposition on the GPU; the index arrays never visit the host."""

@@ -97,3 +97,21 @@ def test_compare_results_rule():
     assert not bad["passed"] and bad["error_count"] == 1
     size = compare_results(torch.tensor([1.0, 5.0, 2.0, 3.0]), ref, type("F", (), {"values": torch.ones(4)})())
     assert not size["passed"] and size["error_count"] == -1
+
+
+def test_auto_config_picks_the_segment_length_from_the_row_lengths():
+    """The choice follows the measured sweep: 128 for small matrices, else one segment per
+    row where possible (512..2048), 512 when no row has block segments (reference table:
+    rode_sddmm.py:35-38)."""
+    from rode_amd import workloads
+    want = {"c1_uniform": (1.0, 128), "c2_lognormal": (1.0, 128), "c3_banded": (0.05, 512),
+            "c4_powerlaw": (0.25, 512), "c5_attention": (1.0, 1024)}
+    for name, (scale, seg) in want.items():
+        _, _, rp, _, _ = workloads.config(name, scale)
+        cfg = RoDeCSR.auto_config(torch.from_numpy(rp))
+        assert cfg == {"seg_length": seg, "k_block": 32, "vec_len": 4}, (name, cfg)
+    # rows of about 1500 slots, many of them: one segment per row
+    rp = np.zeros(40001, dtype=np.int64)
+    rp[1:] = np.cumsum(np.full(40000, 1500))
+    assert RoDeCSR.auto_config(torch.from_numpy(rp))["seg_length"] == 2048
+    assert RoDeCSR.auto_config(torch.zeros(5, dtype=torch.int32))["seg_length"] == 512
