@@ -151,14 +151,24 @@ int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const v
  * *_planned entry points below process such a chunk with kernels that stage the window in
  * LDS once per 128-byte column tile and read it from there; nonzeros outside the window
  * are still gathered from memory, so a plan never changes a result, only the speed.
+ * A plan is made in two steps; the second, larger part is only worth making when the first
+ * finds windows (h_counts[1] > 0):
+ *
+ * 1. rode_hip_window_plan: the descriptors.
  *   dense_rows   rows of the dense operand the column indices point into (B of SpMM,
  *                rhs of SDDMM): the number of columns of the sparse matrix
  *   d_plan       rode_hip_window_plan_bytes(m2) bytes, 16-byte aligned, out.  Layout:
  *                int[4] header {residue chunks, residue chunks with a window, 0, 0},
  *                then int[4] per chunk {first window row, window rows (0: none),
- *                nonzeros inside the window, nonzeros}
+ *                nonzeros, nonzeros outside the window}
  *   h_counts     NULL, or HOST int[4] that receives the header; the call then waits for
- *                the kernels (two small launches, each nonzero's column index read once)
+ *                the kernels (three small launches, each nonzero's column index read once)
+ * 2. rode_hip_window_rows: for every residue row of a chunk with a window, where in the
+ *    window each of its nonzeros is (what the window kernels would otherwise work out per
+ *    call), in the order they will be read.
+ *   d_rows       rode_hip_window_rows_bytes(m2) bytes (10 KiB per chunk of 128 residue
+ *                rows), 16-byte aligned, out
+ *
  * A plan belongs to exactly the residue list it was made from (same m2, same arrays).
  */
 #define RODE_HIP_PLAN_RESIDUE_CHUNK 128
@@ -166,18 +176,23 @@ int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const v
 size_t rode_hip_window_plan_bytes(int m2);
 int rode_hip_window_plan(int m2, int dense_rows, const int* d_row_indices_residue, const int* d_row_offsets,
                          const int* d_column_indices, void* d_plan, size_t plan_bytes, int* h_counts, void* stream);
+size_t rode_hip_window_rows_bytes(int m2);
+int rode_hip_window_rows(int m2, const int* d_row_indices_residue, const int* d_row_offsets,
+                         const int* d_column_indices, const void* d_plan, void* d_rows, size_t rows_bytes, void* stream);
 
 /*
- * rode_hip_spmm_ex with a locality plan.  d_plan: a plan made from these lists, or NULL
- * (then exactly rode_hip_spmm_ex).  h_plan_counts: NULL, or the HOST int[4] header that
- * rode_hip_window_plan returned; with it, kernels that would find no chunk to work on are
- * not launched at all.  fp64 operands, and dense rows of at most 128 bytes, ignore the plan.
- * Same results as without a plan, up to the order of the fp32 additions inside a row.
+ * rode_hip_spmm_ex with a locality plan.  d_plan / d_plan_rows: both parts of a plan made
+ * from these lists, or NULL (then exactly rode_hip_spmm_ex).  h_plan_counts: NULL, or the
+ * HOST int[4] header that rode_hip_window_plan returned; with it, kernels that would find
+ * no chunk to work on are not launched at all.  fp64 operands, and dense rows of at most
+ * 128 bytes, ignore the plan.  Same results as without a plan, up to the order of the fp32
+ * additions inside a row.
  */
 int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                           const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                           const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
-                          const void* d_plan, const int* h_plan_counts, void* stream1, void* stream2);
+                          const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, void* stream1,
+                          void* stream2);
 
 /*
  * Prepares an uninitialised C[M x n] for one of the SpMM calls: zeroes exactly the rows
@@ -228,15 +243,15 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
 
 /*
  * SDDMM with a locality plan: dtype RODE_DENSE_F32 or RODE_DENSE_F16 selects the element
- * type of lhs / rhs; d_plan / h_plan_counts as for rode_hip_spmm_planned (NULL: exactly the
- * typed functions above).  Same results up to the order of the fp32 additions of a dot
+ * type of lhs / rhs; d_plan / d_plan_rows / h_plan_counts as for rode_hip_spmm_planned (NULL:
+ * exactly the typed functions above).  Same results up to the order of the fp32 additions of a dot
  * product.  No counterpart in the reference.
  */
 int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d_row_indices_block,
                            const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                            const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
-                           const void* d_rhs_matrix, float* d_out, const void* d_plan, const int* h_plan_counts,
-                           void* stream1, void* stream2);
+                           const void* d_rhs_matrix, float* d_out, const void* d_plan, const void* d_plan_rows,
+                           const int* h_plan_counts, void* stream1, void* stream2);
 
 /*
  * Row softmax over the values of a CSR pattern, out[idx] = softmax over the row of

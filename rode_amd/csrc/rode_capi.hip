@@ -115,14 +115,28 @@ int rode_hip_window_plan(int m2, int dense_rows, const int* d_row_indices_residu
     return e;
 }
 
+size_t rode_hip_window_rows_bytes(int m2) { return m2 < 0 ? 0 : rode::window_plan_rows_bytes(m2); }
+
+int rode_hip_window_rows(int m2, const int* d_row_indices_residue, const int* d_row_offsets,
+                         const int* d_column_indices, const void* d_plan, void* d_rows, size_t rows_bytes, void* stream)
+{
+    if (m2 < 0 || !d_plan || !aligned16(d_plan)) return hipErrorInvalidValue;
+    if (m2 == 0) return hipSuccess;
+    if (!d_rows || !aligned16(d_rows) || rows_bytes < rode_hip_window_rows_bytes(m2)) return hipErrorInvalidValue;
+    if (!d_row_indices_residue || !d_row_offsets || !d_column_indices) return hipErrorInvalidValue;
+    return rode::window_plan_rows_launch(m2, d_row_indices_residue, d_row_offsets, d_column_indices,
+                                         static_cast<const int*>(d_plan), d_rows, as_stream(stream));
+}
+
 namespace {
 // The caller's plan as the launchers take it; false if it cannot belong to these lists.
-bool plan_ref(const void* d_plan, const int* h_plan_counts, int m2, rode::PlanRef& plan)
+bool plan_ref(const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, int m2, rode::PlanRef& plan)
 {
-    if (!d_plan) return true;
-    if (!aligned16(d_plan)) return false;
+    if (!d_plan || !d_plan_rows) return true; // no plan, or one without rows: the standard kernels do everything
+    if (!aligned16(d_plan) || !aligned16(d_plan_rows)) return false;
     if (h_plan_counts && h_plan_counts[0] != rode::plan_residue_chunks(m2)) return false;
     plan.dev = static_cast<const int*>(d_plan);
+    plan.rows = d_plan_rows;
     plan.host_counts = h_plan_counts;
     return true;
 }
@@ -134,13 +148,15 @@ int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const v
                      void* stream1, void* stream2)
 {
     return rode_hip_spmm_planned(dtype, flags, m1, m2, k, n, d_values, d_column_indices, d_row_offsets, d_row_indices1,
-                                 d_row_indices2, d_row_seg_st_offsets, d_B, d_C, nullptr, nullptr, stream1, stream2);
+                                 d_row_indices2, d_row_seg_st_offsets, d_B, d_C, nullptr, nullptr, nullptr, stream1,
+                                 stream2);
 }
 
 int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                           const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                           const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
-                          const void* d_plan, const int* h_plan_counts, void* stream1, void* stream2)
+                          const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, void* stream1,
+                          void* stream2)
 {
     (void)k;
     constexpr int kKnown = RODE_SPMM_WHOLE_LISTS | RODE_SPMM_ONLY_BLOCK | RODE_SPMM_ONLY_RESIDUE;
@@ -152,7 +168,7 @@ int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, co
     if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
     hipStream_t s1 = as_stream(stream1), s2 = as_stream(stream2);
     rode::PlanRef plan;
-    if (!plan_ref(d_plan, h_plan_counts, m2, plan)) return hipErrorInvalidValue;
+    if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, m2, plan)) return hipErrorInvalidValue;
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
@@ -207,15 +223,15 @@ int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const
 int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d_row_indices_block,
                            const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                            const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
-                           const void* d_rhs_matrix, float* d_out, const void* d_plan, const int* h_plan_counts,
-                           void* stream1, void* stream2)
+                           const void* d_rhs_matrix, float* d_out, const void* d_plan, const void* d_plan_rows,
+                           const int* h_plan_counts, void* stream1, void* stream2)
 {
     (void)n;
     if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
     if (m1 == 0 && m2 == 0) return hipSuccess;
     if (!aligned16(d_lhs_matrix) || !aligned16(d_rhs_matrix)) return hipErrorInvalidValue;
     rode::PlanRef plan;
-    if (!plan_ref(d_plan, h_plan_counts, m2, plan)) return hipErrorInvalidValue;
+    if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, m2, plan)) return hipErrorInvalidValue;
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::sddmm_launch<float>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
@@ -239,7 +255,7 @@ int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_bl
 {
     return rode_hip_sddmm_planned(RODE_DENSE_F32, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
                                   d_row_offsets, d_column_indices, d_values, d_lhs_matrix, d_rhs_matrix, d_out, nullptr,
-                                  nullptr, stream1, stream2);
+                                  nullptr, nullptr, stream1, stream2);
 }
 
 int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,
@@ -249,7 +265,7 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
 {
     return rode_hip_sddmm_planned(RODE_DENSE_F16, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
                                   d_row_offsets, d_column_indices, d_values, d_lhs_half, d_rhs_half, d_out, nullptr,
-                                  nullptr, stream1, stream2);
+                                  nullptr, nullptr, stream1, stream2);
 }
 
 int rode_hip_csr_softmax_f32(int M, const int* d_row_offsets, const float* d_in, float* d_out, float scale,

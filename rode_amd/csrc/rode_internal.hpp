@@ -28,13 +28,17 @@ constexpr int kSpmmWholeLists = 1, kSpmmOnlyBlock = 2, kSpmmOnlyResidue = 4;
 // A locality plan (rode_plan.hip): device array, and optionally a host copy of its four
 // header ints (chunk counts), with which launches that have nothing to do are left out.
 struct PlanRef {
-    const int* dev = nullptr;
+    const int* dev = nullptr;         // descriptors
+    const void* rows = nullptr;       // planned rows of the chunks with a window
     const int* host_counts = nullptr;
 };
 
 size_t window_plan_ints(int m2);
+size_t window_plan_rows_bytes(int m2);
 hipError_t window_plan_launch(int m2, int dense_rows, const int* residue_rows, const int* row_ptr, const int* col,
                               int* plan, hipStream_t stream);
+hipError_t window_plan_rows_launch(int m2, const int* residue_rows, const int* row_ptr, const int* col, const int* plan,
+                                   void* rows, hipStream_t stream);
 
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
@@ -43,9 +47,8 @@ hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* 
 
 // the window kernel of SpMM over the planned chunks of the residue list (T = float or __half)
 template <typename T>
-hipError_t spmm_window_launch(int m2, int n, int owned_slots, const int* residue_rows, const int* row_ptr,
-                              const int* col, const float* val, const T* B, float* C, const int* plan,
-                              hipStream_t stream);
+hipError_t spmm_window_launch(int m2, int n, int owned_slots, const int* col, const float* val, const T* B, float* C,
+                              const int* plan, const void* plan_rows, hipStream_t stream);
 
 hipError_t spmm_clear_rows_launch(int M, size_t row_bytes, const int* row_ptr, void* C, hipStream_t stream);
 
@@ -56,9 +59,8 @@ hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int*
 
 // the window kernel of SDDMM over the planned chunks of the residue list
 template <typename T>
-hipError_t sddmm_window_launch(int m2, int k, const int* residue_rows, const int* row_ptr, const int* col,
-                               const float* val, const T* lhs, const T* rhs, float* out, const int* plan,
-                               hipStream_t stream);
+hipError_t sddmm_window_launch(int m2, int k, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
+                               const int* plan, const void* plan_rows, hipStream_t stream);
 
 hipError_t csr_softmax_launch(int M, const int* row_ptr, const float* in, float* out, float scale,
                               hipStream_t stream);

@@ -116,19 +116,44 @@ __device__ __forceinline__ ResidueItem residue_item(int row, const int* __restri
 // per column tile and every slot that falls into it reads LDS instead of gathering from
 // L2); the standard residue kernels skip it.  Slots outside the window are still gathered
 // from memory, so a plan never changes which nonzeros contribute - only where their dense
-// rows are read from.  Layout of the int array:
-//   [0] residue chunks  [1] residue chunks with a window  [2], [3] zero
-//   then one WindowDesc per residue chunk.
+// rows are read from.  The plan has two device arrays:
+//   descriptors, int[]:  [0] residue chunks  [1] residue chunks with a window  [2], [3] zero,
+//                        then one WindowDesc per residue chunk;
+//   rows, one PlannedChunk per chunk (filled for the chunks with a window): what the
+//                        window kernels would otherwise work out per call for every
+//                        residue row - its slots as positions in the window.
 constexpr int kPlanHeaderInts = 4;
 constexpr int kPlanDescInts = 4;
 constexpr int kPlanResidueChunk = 128;     // residue-list entries per chunk
-constexpr int kResidueWindowRowsMax = 512; // dense rows of one window
+constexpr int kResidueWindowRowsMax = 512; // dense rows of one window (9 bits of a slot's 16-bit entry)
 
-// Window of one chunk: dense rows [w0, w0 + wn); wn == 0: no window.  hits / slots: how
-// many of the chunk's nonzero slots fall into the window / exist (statistics of the plan).
+// Window of one chunk: dense rows [w0, w0 + wn); wn == 0: no window.  slots / misses: how
+// many nonzero slots the chunk has / how many of them fall outside the window.
 struct WindowDesc {
-    int w0, wn, hits, slots;
+    int w0, wn, slots, misses;
 };
+
+// One residue row of a chunk with a window.  Its cnt slots are listed in an order chosen
+// for the LDS banks (see below), entry i = (window row of the slot's column) | (slot << 9),
+// slot counted from the row's first residue slot `first`; a slot whose column is outside
+// the window (bit i of missmask) carries the window row of one that is inside; entries
+// cnt..31 repeat such a window row and have no slot (their value is 0).
+// Order: a ds_read_b128 of a wave serves lane groups (0, 3), (1, 2), (4, 7), (5, 6) in
+// the same cycles, and two 128-byte window rows of equal parity collide in the banks.
+// Rows that lane groups 0, 1, 4, 5 will take list their even window rows first, the rows
+// of groups 2, 3, 6, 7 their odd ones: two groups that meet mostly read different parities.
+struct PlannedRowMeta {
+    int row;       // the residue row (-1: no such entry)
+    int first;     // its first residue slot (index into column_indices / values)
+    int packed;    // cnt | accumulate << 8 | min(aligned length, 0xffff) << 16
+    unsigned missmask;
+};
+struct PlannedChunk {
+    int w0, wn, reserved[2]; // the chunk's window again: the kernels need nothing else to start
+    PlannedRowMeta meta[kPlanResidueChunk];
+    unsigned short entry[kPlanResidueChunk][kBlockItems];
+};
+static_assert(sizeof(PlannedChunk) == 16 + kPlanResidueChunk * (16 + 2 * kBlockItems), "packed layout");
 
 __host__ __device__ inline int plan_residue_chunks(int m2) { return (m2 + kPlanResidueChunk - 1) / kPlanResidueChunk; }
 __host__ __device__ inline size_t plan_ints(int m2)

@@ -123,7 +123,7 @@ plan_chunks_kernel(int m2, int dense_rows, const int* __restrict__ residue_rows,
     __syncthreads();
     const int q25 = quart[0], q75 = quart[1];
     if ((long long)q75 - q25 + 1 > ROWS_MAX || dense_rows <= 0) {
-        if (tid == 0) *reinterpret_cast<int4*>(desc) = make_int4(0, 0, 0, total);
+        if (tid == 0) *reinterpret_cast<int4*>(desc) = make_int4(0, 0, total, total);
         return;
     }
     int w0 = q25 + (q75 - q25) / 2 - ROWS_MAX / 2;
@@ -159,22 +159,115 @@ plan_chunks_kernel(int m2, int dense_rows, const int* __restrict__ residue_rows,
         // 4. decision
         const int wn = hi_hit - lo_hit + 1;
         const bool take = hits > 0 && 2ll * hits >= total && hits >= 2ll * wn;
-        *reinterpret_cast<int4*>(desc) = take ? make_int4(lo_hit, wn, hits, total) : make_int4(0, 0, hits, total);
+        *reinterpret_cast<int4*>(desc) = take ? make_int4(lo_hit, wn, total, total - hits) : make_int4(0, 0, total, total - hits);
         if (take) atomicAdd(plan + 1, 1);
+    }
+}
+
+// Fills the PlannedChunk of every chunk that has a window: 8 threads per residue row.
+__global__ void __launch_bounds__(kPlanResidueChunk * 8)
+plan_rows_kernel(int m2, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
+                 const int* __restrict__ col, const int* __restrict__ plan, PlannedChunk* __restrict__ rows)
+{
+    constexpr int L = 8, OWN = kBlockItems / L;
+    __shared__ unsigned char keys[kPlanResidueChunk][kBlockItems];
+    const int chunk = blockIdx.x;
+    const WindowDesc d = plan_residue_desc(plan, chunk);
+    PlannedChunk& out = rows[chunk];
+    if (threadIdx.x == 0) {
+        out.w0 = d.w0;
+        out.wn = d.wn;
+        out.reserved[0] = out.reserved[1] = 0;
+    }
+    if (d.wn <= 0) return;
+    const int local = threadIdx.x / L, ls = threadIdx.x % L;
+    const int entry = chunk * kPlanResidueChunk + local;
+    int row = -1, first = 0, cnt = 0, aligned = 0;
+    bool accumulate = false;
+    if (entry < m2) {
+        row = residue_rows[entry];
+        const ResidueItem it = residue_item(row, row_ptr);
+        first = it.first;
+        cnt = it.cnt;
+        aligned = it.aligned;
+        accumulate = it.accumulate;
+    }
+    // which lane group of the window kernels takes this row: groups 2, 3, 6, 7 list odd window rows first
+    const int odd_first = (local >> 1) & 1;
+    unsigned u[OWN];
+    unsigned best = 0xffffu;
+#pragma unroll
+    for (int i = 0; i < OWN; ++i) {
+        const int s = ls + i * L;
+        u[i] = 0xffffu;
+        unsigned char key = 3; // not a slot of the row
+        if (s < cnt) {
+            const unsigned dw = (unsigned)(col[first + s] - d.w0);
+            if (dw < (unsigned)d.wn) {
+                u[i] = dw;
+                key = ((dw & 1u) != (unsigned)odd_first) ? 1 : 0;
+            } else {
+                key = 2; // outside the window: after the ones inside
+            }
+        }
+        keys[local][s] = key;
+        best = min(best, u[i]);
+    }
+#pragma unroll
+    for (int m = 1; m < L; m <<= 1) best = min(best, (unsigned)__shfl_xor((int)best, m, kWave));
+    if (best == 0xffffu) best = 0; // no slot inside the window: every read is replaced anyway
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); // the 8 threads of a row are lanes of one wave
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    unsigned missbits = 0;
+#pragma unroll
+    for (int i = 0; i < OWN; ++i) {
+        const int s = ls + i * L;
+        const int key = keys[local][s];
+        int rank = 0; // position: slots with a smaller key, or the same key and a smaller index, come first
+        for (int o = 0; o < kBlockItems; ++o) {
+            const int other = keys[local][o];
+            rank += (other < key || (other == key && o < s)) ? 1 : 0;
+        }
+        const unsigned where = key == 0 || key == 1 ? u[i] : best;
+        out.entry[local][rank] = (unsigned short)(where | (key <= 2 ? (unsigned)s << 9 : 0u));
+        if (key == 2) missbits |= 1u << rank;
+    }
+#pragma unroll
+    for (int m = 1; m < L; m <<= 1) missbits |= (unsigned)__shfl_xor((int)missbits, m, kWave);
+    if (ls == 0) {
+        PlannedRowMeta meta;
+        meta.row = row;
+        meta.first = first;
+        meta.packed = cnt | (accumulate ? 1 << 8 : 0) | (min(aligned, 0xffff) << 16);
+        meta.missmask = missbits;
+        out.meta[local] = meta;
     }
 }
 
 } // namespace
 
 size_t window_plan_ints(int m2) { return plan_ints(m2); }
+size_t window_plan_rows_bytes(int m2) { return (size_t)plan_residue_chunks(m2) * sizeof(PlannedChunk); }
 
 hipError_t window_plan_launch(int m2, int dense_rows, const int* residue_rows, const int* row_ptr, const int* col,
                               int* plan, hipStream_t stream)
 {
     plan_header_kernel<<<1, kWave, 0, stream>>>(m2, plan);
     const int chunks = plan_residue_chunks(m2);
-    if (chunks > 0)
+    if (chunks > 0) {
         plan_chunks_kernel<<<chunks, kWgThreads, 0, stream>>>(m2, dense_rows, residue_rows, row_ptr, col, plan);
+    }
+    return hipGetLastError();
+}
+
+hipError_t window_plan_rows_launch(int m2, const int* residue_rows, const int* row_ptr, const int* col, const int* plan,
+                                   void* rows, hipStream_t stream)
+{
+    const int chunks = plan_residue_chunks(m2);
+    if (chunks > 0)
+        plan_rows_kernel<<<chunks, kPlanResidueChunk * 8, 0, stream>>>(m2, residue_rows, row_ptr, col, plan,
+                                                                       static_cast<PlannedChunk*>(rows));
     return hipGetLastError();
 }
 

@@ -265,7 +265,7 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
     }
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && m2 > 0 && window_residue)
-        e = sddmm_window_launch<T>(m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev, s2);
+        e = sddmm_window_launch<T>(m2, k, col, val, lhs, rhs, out, plan.dev, plan.rows, s2);
     return e;
 }
 

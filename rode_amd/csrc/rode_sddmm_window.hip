@@ -27,35 +27,35 @@ __device__ __forceinline__ float transpose_reduce8(const float (&p)[8], int ls)
 
 template <typename T, bool EDGE>
 __global__ void __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
-sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
-                            const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
-                            const T* __restrict__ rhs, float* __restrict__ out, const int* __restrict__ plan)
+sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ col, const float* __restrict__ val,
+                            const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out,
+                            const PlannedChunk* __restrict__ rows)
 {
     constexpr int VEC = DenseVec<T>::kElems;
     constexpr int TW = kResLanes * VEC; // elements of a dense row in one tile
     constexpr int QUADS = kBlockItems / 4;
     __shared__ uint4 win[kResWinVecs];
-    __shared__ __attribute__((aligned(16))) float lds_val[kResRows * kBlockItems];
-    __shared__ __attribute__((aligned(16))) unsigned short stage_loc[kResRows * kBlockItems];
+    __shared__ __attribute__((aligned(16))) float lds_val[kResRows * kResValStride];
 
     const int part = xcd_logical_block(blockIdx.x, gridDim.x);
     const int chunk = part / kResParts;
     if (chunk >= plan_residue_chunks(m2)) return;
     const int group = threadIdx.x / kResLanes, ls = threadIdx.x % kResLanes;
-    const int entry = part * kResRows + group;
-    const int listed = entry < m2 ? residue_rows[entry] : -1; // (does not wait for the plan)
-    const WindowDesc d = plan_residue_desc(plan, chunk);
+    const PlannedChunk& pc = rows[chunk];
+    struct { int w0, wn; } d = {pc.w0, pc.wn};
     if (d.wn <= 0) return; // the standard kernel has this chunk
+    const int local = (part % kResParts) * kResRows + group; // this lane group's row of the chunk
     const size_t row_bytes = (size_t)k * sizeof(T);
     const int tiles = (k + TW - 1) / TW;
 
-    // first tile of the lhs row on its way while the sparse data is prepared
+    ResidueRow rr;
+    float* my_v = lds_val + group * kResValStride;
+    load_planned_row(pc, local, 0, val, my_v, rr);
+    const int listed = rr.row;
+    // first tile of the lhs row
     uint4 a_raw = make_uint4(0, 0, 0, 0);
     const T* lhs_row = lhs + (size_t)(listed >= 0 ? listed : 0) * k;
     if ((!EDGE || ls * VEC < k) && listed >= 0) a_raw = *reinterpret_cast<const uint4*>(lhs_row + ls * VEC);
-    ResidueRow rr;
-    float* my_v = lds_val + group * kBlockItems;
-    prepare_residue_row(listed, 0, d, row_ptr, col, val, stage_loc + group * kBlockItems, my_v, rr);
     const int wave_quads = wave_max_quads(rr.quads);
     const bool wave_all_hit = __ballot(rr.missmask != 0) == 0ull;
 
@@ -80,11 +80,11 @@ sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ residue_rows,
         }
         __syncthreads();
         // (the miss path's inputs are made opaque per tile: otherwise the compiler computes
-        // every slot's test and memory address once, outside the tile loop, and holds them
-        // in registers of their own - more than there are)
-        int abase_t = rr.abase, head_t = rr.head, end_t = rr.end;
+        // every position's test and memory address once, outside the tile loop, and holds
+        // them in registers of their own - more than there are)
+        int first_t = rr.first;
         unsigned miss_t = rr.missmask;
-        if (!wave_all_hit) asm volatile("" : "+v"(abase_t), "+v"(head_t), "+v"(end_t), "+v"(miss_t));
+        if (!wave_all_hit) asm volatile("" : "+v"(first_t), "+v"(miss_t));
 #pragma unroll
         for (int q = 0; q < QUADS; ++q) {
             if (q < wave_quads) { // the same for every lane of the wave
@@ -95,11 +95,9 @@ sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ residue_rows,
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         if ((miss_t >> (4 * q + j)) & 1u) {
-                            // outside the window: the column again (a slot outside the row repeats
-                            // one of the row's own columns), then the rhs row from memory
-                            const int s = min(max(4 * q + j, head_t), end_t - 1);
-                            raw[j] = col_ok ? *reinterpret_cast<const uint4*>(rhs_lane + (size_t)col[abase_t + s] * k)
-                                            : make_uint4(0, 0, 0, 0);
+                            // outside the window: the slot's column, then the rhs row from memory
+                            const int c = col[first_t + planned_slot(pc, local, 4 * q + j)];
+                            raw[j] = col_ok ? *reinterpret_cast<const uint4*>(rhs_lane + (size_t)c * k) : make_uint4(0, 0, 0, 0);
                         }
                     }
                 }
@@ -114,15 +112,15 @@ sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ residue_rows,
         }
     }
 
-    // lane l of the group ends up with the dot products of the slots l, 8 + l, 16 + l, 24 + l
+    // lane l of the group ends up with the dot products of the positions l, 8 + l, 16 + l, 24 + l
 #pragma unroll
     for (int i = 0; i < kBlockItems / kResLanes; ++i) {
         float part8[kResLanes];
 #pragma unroll
         for (int j = 0; j < kResLanes; ++j) part8[j] = p[i * kResLanes + j];
         const float dot = transpose_reduce8(part8, ls);
-        const int s = i * kResLanes + ls;
-        if (s >= rr.head && s < rr.end) out[rr.abase + s] = my_v[s] * dot;
+        const int pos = i * kResLanes + ls;
+        if (pos < rr.cnt) out[rr.first + planned_slot(pc, local, pos)] = my_v[pos] * dot;
     }
 }
 
@@ -130,24 +128,22 @@ sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ residue_rows,
 
 // The window kernel over the planned chunks of the residue list.  T = float or __half.
 template <typename T>
-hipError_t sddmm_window_launch(int m2, int k, const int* residue_rows, const int* row_ptr, const int* col,
-                               const float* val, const T* lhs, const T* rhs, float* out, const int* plan,
-                               hipStream_t stream)
+hipError_t sddmm_window_launch(int m2, int k, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
+                               const int* plan, const void* plan_rows, hipStream_t stream)
 {
     if (m2 <= 0) return hipSuccess;
     const int g = grid_for_residue_parts(m2);
+    const PlannedChunk* rows = static_cast<const PlannedChunk*>(plan_rows);
     if (((size_t)k * sizeof(T)) % (kResLanes * 16) != 0)
-        sddmm_residue_window_kernel<T, true><<<g, kResThreads, 0, stream>>>(m2, k, residue_rows, row_ptr, col, val, lhs, rhs,
-                                                                            out, plan);
+        sddmm_residue_window_kernel<T, true><<<g, kResThreads, 0, stream>>>(m2, k, col, val, lhs, rhs, out, rows);
     else
-        sddmm_residue_window_kernel<T, false><<<g, kResThreads, 0, stream>>>(m2, k, residue_rows, row_ptr, col, val, lhs,
-                                                                             rhs, out, plan);
+        sddmm_residue_window_kernel<T, false><<<g, kResThreads, 0, stream>>>(m2, k, col, val, lhs, rhs, out, rows);
     return hipGetLastError();
 }
 
-template hipError_t sddmm_window_launch<float>(int, int, const int*, const int*, const int*, const float*, const float*,
-                                               const float*, float*, const int*, hipStream_t);
-template hipError_t sddmm_window_launch<__half>(int, int, const int*, const int*, const int*, const float*, const __half*,
-                                                const __half*, float*, const int*, hipStream_t);
+template hipError_t sddmm_window_launch<float>(int, int, const int*, const float*, const float*, const float*, float*,
+                                               const int*, const void*, hipStream_t);
+template hipError_t sddmm_window_launch<__half>(int, int, const int*, const float*, const __half*, const __half*, float*,
+                                                const int*, const void*, hipStream_t);
 
 } // namespace rode

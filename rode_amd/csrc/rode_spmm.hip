@@ -340,7 +340,7 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
         }
         if constexpr (!std::is_same<T, double>::value) {
             if (e == hipSuccess && window_residue)
-                e = spmm_window_launch<T>(m2, n, owned_slots, residue_rows, row_ptr, col, val, B, C, plan.dev, s2);
+                e = spmm_window_launch<T>(m2, n, owned_slots, col, val, B, C, plan.dev, plan.rows, s2);
         }
     }
     return e;

@@ -13,13 +13,16 @@
 // LDS (77 KB) and registers (128) are sized so that two workgroups share a CU: while one
 // waits for memory the other computes.  The lanes of a group keep the LDS address of every
 // slot's dense row in registers for all tiles, so a slot costs one ds_read_b128 plus its
-// multiply-adds.
+// multiply-adds.  Which window row a slot reads is not worked out here: the plan holds it
+// for every residue row of a chunk with a window (PlannedChunk), in an order that keeps
+// lane groups that meet in the LDS banks on rows of different parity.
 #pragma once
 #include "rode_items.hpp"
 
 #ifdef RODE_PHASE_TIMING
 // Debug builds only: cycles spent per phase, summed over workgroups.
-__device__ unsigned long long rode_phase_clk[8];
+static __device__ unsigned long long rode_phase_clk[8];
+#ifdef RODE_PHASE_READER
 extern "C" void rode_phase_read(unsigned long long* out, int reset)
 {
     (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(rode_phase_clk), sizeof(unsigned long long) * 8);
@@ -28,19 +31,20 @@ extern "C" void rode_phase_read(unsigned long long* out, int reset)
         (void)hipMemcpyToSymbol(HIP_SYMBOL(rode_phase_clk), z, sizeof(z));
     }
 }
+#endif
 #define RODE_PHASE(i)                                                                    \
     do {                                                                                 \
-        const unsigned long long now_ = __builtin_readcyclecounter();                    \
+        const unsigned now_ = (unsigned)__builtin_readcyclecounter();                    \
         phase_acc_[i] += now_ - phase_t_;                                                \
         phase_t_ = now_;                                                                 \
     } while (0)
 #define RODE_PHASE_BEGIN                                                                 \
-    unsigned long long phase_acc_[8] = {0, 0, 0, 0, 0, 0, 0, 0};                         \
-    unsigned long long phase_t_ = __builtin_readcyclecounter()
+    unsigned phase_acc_[5] = {0, 0, 0, 0, 0};                                            \
+    unsigned phase_t_ = (unsigned)__builtin_readcyclecounter()
 #define RODE_PHASE_END                                                                   \
     do {                                                                                 \
         if (threadIdx.x == 0)                                                            \
-            for (int i_ = 0; i_ < 8; ++i_) atomicAdd(&rode_phase_clk[i_], phase_acc_[i_]); \
+            for (int i_ = 0; i_ < 5; ++i_) atomicAdd(&rode_phase_clk[i_], (unsigned long long)phase_acc_[i_]); \
     } while (0)
 #else
 #define RODE_PHASE(i)
@@ -56,9 +60,12 @@ constexpr int kResRows = kResThreads / kResLanes;         // residue rows per wo
 constexpr int kResParts = kPlanResidueChunk / kResRows;   // workgroups per chunk of the plan
 constexpr int kResWinVecs = kResidueWindowRowsMax * kResLanes;                 // 16-byte pieces of a window
 constexpr int kResPrefetch = (kResWinVecs + kResThreads - 1) / kResThreads;    // pieces one thread moves per tile
-constexpr unsigned kMiss = 0xffffu; // 16-bit window row of a slot whose dense row is outside the window
+// A group's 32 values in LDS are 36 floats apart: the eight groups of a wave read their
+// float4 of the same quad from eight different sets of banks (32 apart, four groups would
+// share each set).
+constexpr int kResValStride = kBlockItems + 4;
 static_assert(kPlanResidueChunk % kResRows == 0, "a workgroup takes a whole fraction of a chunk");
-static_assert(kResidueWindowRowsMax < (int)kMiss, "window rows must fit 16 bits");
+static_assert(kResidueWindowRowsMax == 512 && kBlockItems == 32, "a plan entry holds 9 bits of window row and 5 of slot");
 
 inline int grid_for_residue_parts(int m2)
 {
@@ -109,86 +116,64 @@ __device__ __forceinline__ void res_fill(uint4* win, const char* src_lane, size_
     }
 }
 
-__device__ __forceinline__ unsigned window_locator(int c, int w0, int wn)
-{
-    const unsigned d = (unsigned)(c - w0);
-    return d < (unsigned)wn ? d : kMiss;
-}
-
-// One residue row as its lane group keeps it: its slots as whole quads from the 4-aligned
-// slot `abase` at or before its first one; the row's own slots are [head, end) of the 32.
-// addr[s]: LDS byte address of this lane's 16 bytes of slot s's dense row; for a slot
-// whose dense row is outside the window (bit s of missmask) it is the address of one of
-// the row's slots that is inside, and the data has to come from memory instead.
+// One residue row as its lane group keeps it: cnt slots at positions 0 .. cnt - 1 (the order
+// of the plan), the rest of the 32 positions carry value 0.
+// addr[i]: LDS byte address of this lane's 16 bytes of the dense row of position i; for a
+// position whose dense row is outside the window (bit i of missmask) it is the address of
+// one of the row's positions that is inside, and the data has to come from memory instead.
 struct ResidueRow {
-    int row; // -1: nothing to do
-    int abase, head, end, quads;
+    int row;   // -1: nothing to do
+    int first; // first residue slot of the row in column_indices / values
+    int cnt, quads;
     unsigned missmask;
-    bool accumulate;      // the row also has block segments (SpMM adds instead of storing)
+    bool accumulate; // the row also has block segments (SpMM adds instead of storing)
     int addr[kBlockItems];
 };
 
-// Prepares the residue row `listed` (-1: none) of this lane group: the 8 lanes classify 4
-// slots each against the window, exchange the result through `stage_loc` (32 shorts of
-// this group) and leave the row's values in `my_val` (32 floats of this group; 0 outside
-// the row).  A slot outside the row gets value 0 and the column of the row's first slot.
-// skip_owned_slots: rows with block segments and at most that many aligned slots are left
-// to the block kernel (SpMM under the whole-lists promise); 0 for SDDMM.
-__device__ __forceinline__ void prepare_residue_row(int listed, int skip_owned_slots, const WindowDesc& d,
-                                                    const int* __restrict__ row_ptr, const int* __restrict__ col,
-                                                    const float* __restrict__ val, unsigned short* stage_loc,
-                                                    float* my_val, ResidueRow& rr)
+// The slot (counted from rr.first) that the plan put at position i of row `local` of a chunk.
+__device__ __forceinline__ int planned_slot(const PlannedChunk& pc, int local, int i)
+{
+    return (pc.entry[local][i] >> 9) & (kBlockItems - 1);
+}
+
+// Loads row `local` of a planned chunk for this lane group: the LDS addresses of its 32
+// positions into registers, its values (in position order, 0 past the row) into `my_val`
+// (32 floats of this group; the 8 lanes write 4 each).  skip_owned_slots: rows with block
+// segments and at most that many aligned slots are left to the block kernel (SpMM under
+// the whole-lists promise); 0 for SDDMM.
+__device__ __forceinline__ void load_planned_row(const PlannedChunk& pc, int local, int skip_owned_slots,
+                                                 const float* __restrict__ val, float* my_val, ResidueRow& rr)
 {
     const int ls = threadIdx.x % kResLanes;
-    rr.row = -1;
-    rr.abase = rr.head = rr.end = 0;
-    rr.accumulate = false;
-    int fill = d.w0;
-    if (listed >= 0) {
-        const ResidueItem it = residue_item(listed, row_ptr);
-        if (!(it.accumulate && it.aligned <= skip_owned_slots)) {
-            rr.row = listed;
-            rr.accumulate = it.accumulate;
-            if (it.cnt > 0) {
-                rr.abase = it.first & ~(kVecLen - 1);
-                rr.head = it.first - rr.abase;
-                rr.end = rr.head + it.cnt;
-                fill = col[it.first];
-            }
-        }
+    const int4 meta = *reinterpret_cast<const int4*>(&pc.meta[local]);
+    const uint4* entries = reinterpret_cast<const uint4*>(pc.entry[local]);
+    uint4 e4[kBlockItems / 8];
+#pragma unroll
+    for (int i = 0; i < kBlockItems / 8; ++i) e4[i] = entries[i];
+    rr.row = meta.x;
+    rr.first = meta.y;
+    rr.cnt = meta.z & 0xff;
+    rr.accumulate = (meta.z >> 8) & 1;
+    rr.missmask = (unsigned)meta.w;
+    if (rr.row < 0 || (rr.accumulate && ((meta.z >> 16) & 0xffff) <= skip_owned_slots)) {
+        rr.row = -1;
+        rr.cnt = 0;
+        rr.missmask = 0;
     }
-    rr.quads = (rr.end + 3) / 4;
+    rr.quads = (rr.cnt + 3) / 4;
     constexpr int OWN = kBlockItems / kResLanes;
-    unsigned u[OWN];
-    unsigned best = kMiss, missbits = 0;
 #pragma unroll
     for (int i = 0; i < OWN; ++i) {
-        const int s = ls + i * kResLanes;
-        const bool in = s >= rr.head && s < rr.end;
-        u[i] = window_locator(in ? col[rr.abase + s] : fill, d.w0, d.wn);
-        my_val[s] = in ? val[rr.abase + s] : 0.f;
-        best = min(best, u[i]);
-        if (u[i] == kMiss) missbits |= 1u << s;
+        const int pos = ls + i * kResLanes;
+        my_val[pos] = pos < rr.cnt ? val[rr.first + planned_slot(pc, local, pos)] : 0.f;
     }
-#pragma unroll
-    for (int m = 1; m < kResLanes; m <<= 1) {
-        best = min(best, (unsigned)__shfl_xor((int)best, m, kWave));
-        missbits |= (unsigned)__shfl_xor((int)missbits, m, kWave);
-    }
-    if (best == kMiss) best = 0; // no slot inside the window: every read is replaced anyway
-    rr.missmask = missbits;
-#pragma unroll
-    for (int i = 0; i < OWN; ++i) stage_loc[ls + i * kResLanes] = (unsigned short)(u[i] == kMiss ? best : u[i]);
-    wave_lds_sync(); // the 8 lanes of a group are lanes of one wave
-    const uint4* src = reinterpret_cast<const uint4*>(stage_loc);
 #pragma unroll
     for (int i = 0; i < kBlockItems / 8; ++i) {
-        const uint4 w4 = src[i];
-        const unsigned w[4] = {w4.x, w4.y, w4.z, w4.w};
+        const unsigned w[4] = {e4[i].x, e4[i].y, e4[i].z, e4[i].w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            rr.addr[8 * i + 2 * j] = (int)(((w[j] & 0xffffu) * kResLanes + ls) * 16);
-            rr.addr[8 * i + 2 * j + 1] = (int)(((w[j] >> 16) * kResLanes + ls) * 16);
+            rr.addr[8 * i + 2 * j] = (int)((((w[j] & 0xffffu) & (kResidueWindowRowsMax - 1)) * kResLanes + ls) * 16);
+            rr.addr[8 * i + 2 * j + 1] = (int)((((w[j] >> 16) & (kResidueWindowRowsMax - 1)) * kResLanes + ls) * 16);
         }
     }
 }

@@ -114,7 +114,7 @@ class RoDeCSR:
             plan = rode_sddmm_hip.window_plan(res, m2, self.row_offsets, self.column_indices, self.n)
             enough = plan.windowed >= max(self.PLAN_MIN_CHUNKS, (plan.counts[0] + 1) // 2)
             if plan.windowed > 0 and (self.locality is True or enough):
-                self.plan = plan
+                self.plan = rode_sddmm_hip.window_plan_rows(plan, res, m2, self.row_offsets, self.column_indices)
 
     def with_values(self, values):
         """The same pattern and decomposition with other values (no preprocessing is

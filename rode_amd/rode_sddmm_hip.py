@@ -76,8 +76,9 @@ class WindowPlan:
     """Locality plan of one decomposition (``rode_hip_window_plan``): the device array and
     a host copy of its header ``[residue chunks, residue chunks with a window, 0, 0]``."""
 
-    def __init__(self, data, counts):
-        self.data = data
+    def __init__(self, data, counts, rows=None):
+        self.data = data                                       # descriptors (device int32)
+        self.rows = rows                                       # planned rows of the chunks with a window (device bytes)
         self.counts = counts                                   # list of 4 ints
         self._header = (ctypes.c_int * 4)(*counts)             # what the C ABI reads
 
@@ -87,7 +88,7 @@ class WindowPlan:
 
     def descriptors(self):
         """int32 array of shape (residue chunks, 4): first window row, window rows (0: none),
-        nonzeros inside the window, nonzeros of the chunk."""
+        nonzeros, nonzeros outside the window."""
         return self.data.cpu().numpy()[4:].reshape(-1, 4)
 
 
@@ -109,14 +110,30 @@ def window_plan(residue_indices, m2, row_offsets, column_indices, dense_rows):
         code = lib.rode_hip_window_plan(m2, dense_rows, residue_indices.data_ptr(), row_offsets.data_ptr(),
                                         column_indices.data_ptr(), data.data_ptr(), nbytes, ctypes.addressof(counts),
                                         _stream_handle(dev))
-    _lib.check(code, "rode_hip_window_plan")
+        _lib.check(code, "rode_hip_window_plan")
     return WindowPlan(data, list(counts))
 
 
+def window_plan_rows(plan, residue_indices, m2, row_offsets, column_indices):
+    """Second part of a plan (``rode_hip_window_rows``): for every residue row of a chunk
+    with a window, where in the window its nonzeros are.  10 KiB per 128 residue rows; made
+    only for a plan that is going to be used."""
+    lib = _lib.load()
+    dev = row_offsets.device
+    with torch.cuda.device(dev):
+        rbytes = lib.rode_hip_window_rows_bytes(m2)
+        plan.rows = torch.empty(rbytes // 16, 4, dtype=torch.int32, device=dev)
+        code = lib.rode_hip_window_rows(m2, residue_indices.data_ptr(), row_offsets.data_ptr(),
+                                        column_indices.data_ptr(), plan.data.data_ptr(), plan.rows.data_ptr(), rbytes,
+                                        _stream_handle(dev))
+    _lib.check(code, "rode_hip_window_rows")
+    return plan
+
+
 def _plan_args(plan):
-    if plan is None:
-        return None, None
-    return plan.data.data_ptr(), ctypes.addressof(plan._header)
+    if plan is None or plan.rows is None:
+        return None, None, None
+    return plan.data.data_ptr(), plan.rows.data_ptr(), ctypes.addressof(plan._header)
 
 
 def preprocess(row_offsets, nnz, seg_length, k_block, vec_len):
@@ -176,11 +193,10 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
     lib = _lib.load()
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
-        plan_dev, plan_counts = _plan_args(plan)
         code = lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[kind], m1, m2, n, k, block_indices.data_ptr(),
                                           residue_indices.data_ptr(), st_offsets.data_ptr(), row_offsets.data_ptr(),
                                           column_indices.data_ptr(), values.data_ptr(), lhs_matrix.data_ptr(),
-                                          rhs_matrix.data_ptr(), out.data_ptr(), plan_dev, plan_counts, s, s)
+                                          rhs_matrix.data_ptr(), out.data_ptr(), *_plan_args(plan), s, s)
     _lib.check(code, "rode_hip_sddmm_planned")
     return out
 
@@ -230,10 +246,9 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     dtype = {torch.float32: 0, torch.float16: 1, torch.float64: 2}[dense_matrix.dtype]  # RODE_DENSE_*
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
-        plan_dev, plan_counts = _plan_args(plan)
         code = lib.rode_hip_spmm_planned(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
                                          values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
                                          block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
-                                         dense_matrix.data_ptr(), out.data_ptr(), plan_dev, plan_counts, s, s)
+                                         dense_matrix.data_ptr(), out.data_ptr(), *_plan_args(plan), s, s)
     _lib.check(code, "rode_hip_spmm_planned")
     return out
