@@ -113,16 +113,17 @@ __device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int ro
 // [base, base + cnt) with base = st_off[s] & ~3 and cnt = floor((len + mask) / 32) * 32
 // (RoDeSddmm.cu:35-54); the first `mask` slots belong to the previous row and are
 // computed but never stored (RoDeSddmm.cu:56-58, 197).
+// (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
 template <typename T, int KT, int NS, bool EDGE>
-__global__ void __launch_bounds__(kWgThreads)
-sddmm_block_kernel(int m1, int k, const int* __restrict__ block_rows, const int* __restrict__ st_off,
-                   const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
-                   const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
+__device__ __forceinline__ void
+sddmm_block_body(int bid, int nblocks, int m1, int k, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                 const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
+                 const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
 {
     using S = SddmmShape<T, KT>;
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int seg = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
+    const int seg = xcd_logical_block(bid, nblocks) * kWavesPerWg + wave;
     if (seg >= m1) return;
 
     // Consecutive segments of one row whose starts fall into the same window of
@@ -162,10 +163,11 @@ sddmm_block_kernel(int m1, int k, const int* __restrict__ block_rows, const int*
 // starting at (s & ~3) + floor(N / 32) * 32; shorter rows are taken whole.
 // Lane ls of the group owns the slots ls, ls + LPR, ... (value, result, store).
 template <typename T, int KT, int NS, bool EDGE>
-__global__ void __launch_bounds__(kWgThreads)
-sddmm_residue_kernel(int m2, int k, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
-                     const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
-                     const T* __restrict__ rhs, float* __restrict__ out, const int* __restrict__ plan)
+__device__ __forceinline__ void
+sddmm_residue_body(int bid, int nblocks, int m2, int k, const int* __restrict__ residue_rows,
+                   const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
+                   const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out,
+                   const int* __restrict__ plan)
 {
     using S = SddmmShape<T, KT>;
     constexpr int VEC = S::kVec, LPR = S::kLpr;
@@ -175,7 +177,7 @@ sddmm_residue_kernel(int m2, int k, const int* __restrict__ residue_rows, const 
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * RPW * kBlockItems];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int group = lane / LPR, ls = lane % LPR;
-    const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * RPW + group;
+    const int item = (xcd_logical_block(bid, nblocks) * kWavesPerWg + wave) * RPW + group;
     if (item >= m2) return;
     if (plan && plan_residue_desc(plan, item / kPlanResidueChunk).wn > 0) return; // the window kernel has this chunk
 
@@ -231,6 +233,44 @@ sddmm_residue_kernel(int m2, int k, const int* __restrict__ residue_rows, const 
     }
 }
 
+template <typename T, int KT, int NS, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+sddmm_block_kernel(int m1, int k, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                   const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
+                   const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
+{
+    sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+}
+
+template <typename T, int KT, int NS, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+sddmm_residue_kernel(int m2, int k, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
+                     const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
+                     const T* __restrict__ rhs, float* __restrict__ out, const int* __restrict__ plan)
+{
+    sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out, plan);
+}
+
+// Both lists in one launch: the first g1 workgroups work on block segments, the others on
+// residue rows.  For matrices so small that a launch costs as much as its kernel.
+template <typename T, int KT, int NS, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+sddmm_pair_kernel(int g1, int m1, int m2, int k, const int* __restrict__ block_rows, const int* __restrict__ residue_rows,
+                  const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
+                  const float* __restrict__ val, const T* __restrict__ lhs, const T* __restrict__ rhs,
+                  float* __restrict__ out, const int* __restrict__ plan)
+{
+    if ((int)blockIdx.x < g1)
+        sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, g1, m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+    else
+        sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, k, residue_rows, row_ptr, col, val, lhs,
+                                            rhs, out, plan);
+}
+
+// Up to this many workgroups, and when both kernels go to the same stream, the two lists
+// are processed by one launch.
+constexpr int kPairMaxWorkgroups = 16384;
+
 inline int grid_for_waves(long long nwaves)
 {
     long long wgs = (nwaves + kWavesPerWg - 1) / kWavesPerWg;
@@ -255,13 +295,18 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
         standard_residue = plan.host_counts[1] < plan.host_counts[0];
         window_residue = plan.host_counts[1] > 0;
     }
-    if (m1 > 0) {
-        sddmm_block_kernel<T, KT, NS, EDGE><<<g1, kWgThreads, 0, s1>>>(
-            m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
-    }
-    if (m2 > 0 && standard_residue) {
-        sddmm_residue_kernel<T, KT, NS, EDGE><<<g2, kWgThreads, 0, s2>>>(
-            m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev);
+    if (m1 > 0 && m2 > 0 && standard_residue && s1 == s2 && g1 + g2 <= kPairMaxWorkgroups) {
+        sddmm_pair_kernel<T, KT, NS, EDGE><<<g1 + g2, kWgThreads, 0, s1>>>(
+            g1, m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);
+    } else {
+        if (m1 > 0) {
+            sddmm_block_kernel<T, KT, NS, EDGE><<<g1, kWgThreads, 0, s1>>>(
+                m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+        }
+        if (m2 > 0 && standard_residue) {
+            sddmm_residue_kernel<T, KT, NS, EDGE><<<g2, kWgThreads, 0, s2>>>(
+                m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev);
+        }
     }
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && m2 > 0 && window_residue)

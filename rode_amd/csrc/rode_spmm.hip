@@ -43,6 +43,10 @@ namespace {
 // more than they mind the extra atomics).
 constexpr int kOwnedRowSlots = 1024;
 constexpr int kOwnedMinSegments = 16384;
+// Up to this many workgroups, and when both kernels go to the same stream, the two lists
+// are processed by one launch (spmm_pair_kernel).  Above it the residue kernel runs on its
+// own: it needs a quarter of the block kernel's registers and keeps twice the waves per CU.
+constexpr int kPairMaxWorkgroups = 16384;
 
 template <typename T, int TN>
 struct SpmmShape {
@@ -111,12 +115,13 @@ __device__ __forceinline__ void store_row(double* dst, const double (&acc)[VEC])
 
 // One wave per block segment (see sddmm_block_kernel for the slot arithmetic,
 // identical at RoDeSpmm.cu:210-234).
+// (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
 template <typename T, int TN, bool EDGE>
-__global__ void __launch_bounds__(kWgThreads)
-spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_rows, const int* __restrict__ st_off,
-                  const int* __restrict__ row_ptr, const int* __restrict__ col,
-                  const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
-                  typename DenseVec<T>::Acc* __restrict__ C)
+__device__ __forceinline__ void
+spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, const int* __restrict__ block_rows,
+                const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
+                const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
+                typename DenseVec<T>::Acc* __restrict__ C)
 {
     using S = SpmmShape<T, TN>;
     using A = typename S::Acc;
@@ -124,7 +129,7 @@ spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int seg0 = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg;
+    const int seg0 = xcd_logical_block(bid, nblocks) * kWavesPerWg;
     const int seg = seg0 + wave;
     // Do neighbouring segments of this workgroup belong to one row (a long row)?  Every
     // wave finds the same answer.  If so, the waves add their sums up in LDS and the row
@@ -209,11 +214,11 @@ spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_
 // One group of LPR lanes per residue row (tail selection: RoDeSpmm.cu:71-82); the
 // group walks its row's slot quads one after the other, no cross-lane reduction.
 template <typename T, int TN, bool EDGE>
-__global__ void __launch_bounds__(kWgThreads)
-spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ residue_rows,
-                    const int* __restrict__ row_ptr, const int* __restrict__ col,
-                    const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
-                    typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
+__device__ __forceinline__ void
+spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, const int* __restrict__ residue_rows,
+                  const int* __restrict__ row_ptr, const int* __restrict__ col,
+                  const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
+                  typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
     using S = SpmmShape<T, TN>;
     using A = typename S::Acc;
@@ -224,7 +229,7 @@ spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ resi
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * RPW * kBlockItems];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int group = lane / LPR, ls = lane % LPR;
-    const int item = (xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave) * RPW + group;
+    const int item = (xcd_logical_block(bid, nblocks) * kWavesPerWg + wave) * RPW + group;
     if (item >= m2) return;
 
     if (plan && plan_residue_desc(plan, item / kPlanResidueChunk).wn > 0) return; // the window kernel has this chunk
@@ -267,6 +272,43 @@ spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ resi
     } else {
         store_row<VEC>(c_lane, acc);
     }
+}
+
+template <typename T, int TN, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                  const int* __restrict__ row_ptr, const int* __restrict__ col,
+                  const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
+                  typename DenseVec<T>::Acc* __restrict__ C)
+{
+    spmm_block_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m1, n, owned_slots, block_rows, st_off, row_ptr, col, val, B, C);
+}
+
+template <typename T, int TN, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ residue_rows,
+                    const int* __restrict__ row_ptr, const int* __restrict__ col,
+                    const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
+                    typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
+{
+    spmm_residue_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m2, n, owned_slots, residue_rows, row_ptr, col, val, B, C, plan);
+}
+
+// Both lists in one launch: the first g1 workgroups of a grid row work on block segments,
+// the others on residue rows.  For matrices so small that a launch costs as much as its
+// kernel (a kernel of a few microseconds); the two parts then also fill the GPU together.
+template <typename T, int TN, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, const int* __restrict__ block_rows,
+                 const int* __restrict__ residue_rows, const int* __restrict__ st_off, const int* __restrict__ row_ptr,
+                 const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
+                 const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
+{
+    if ((int)blockIdx.x < g1)
+        spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, block_rows, st_off, row_ptr, col, val, B, C);
+    else
+        spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, owned_slots, residue_rows, row_ptr, col, val,
+                                       B, C, plan);
 }
 
 constexpr int kClearRowsPerGroup = 8;
@@ -325,23 +367,30 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
         standard_residue = plan.host_counts[1] < plan.host_counts[0];
         window_residue = plan.host_counts[1] > 0;
     }
-    if (m1 > 0 && !(flags & kSpmmOnlyResidue)) {
-        dim3 grid(g1, tiles);
-        spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, owned_slots, block_rows, st_off, row_ptr, col,
-                                                                    val, B, C);
-    }
-    hipError_t e = hipGetLastError();
-    if (m2 > 0 && !(flags & kSpmmOnlyBlock)) {
-        if (standard_residue) {
+    const bool block = m1 > 0 && !(flags & kSpmmOnlyResidue), residue = m2 > 0 && !(flags & kSpmmOnlyBlock);
+    hipError_t e = hipSuccess;
+    if (block && residue && standard_residue && s1 == s2 && (long long)(g1 + g2) * tiles <= kPairMaxWorkgroups) {
+        dim3 grid(g1 + g2, tiles);
+        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, owned_slots, block_rows, residue_rows,
+                                                                   st_off, row_ptr, col, val, B, C, plan.dev);
+        e = hipGetLastError();
+    } else {
+        if (block) {
+            dim3 grid(g1, tiles);
+            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, owned_slots, block_rows, st_off, row_ptr,
+                                                                        col, val, B, C);
+            e = hipGetLastError();
+        }
+        if (residue && standard_residue) {
             dim3 grid(g2, tiles);
             spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, residue_rows, row_ptr, col,
                                                                           val, B, C, plan.dev);
-            e = hipGetLastError();
+            if (e == hipSuccess) e = hipGetLastError();
         }
-        if constexpr (!std::is_same<T, double>::value) {
-            if (e == hipSuccess && window_residue)
-                e = spmm_window_launch<T>(m2, n, owned_slots, col, val, B, C, plan.dev, plan.rows, s2);
-        }
+    }
+    if constexpr (!std::is_same<T, double>::value) {
+        if (e == hipSuccess && residue && window_residue)
+            e = spmm_window_launch<T>(m2, n, owned_slots, col, val, B, C, plan.dev, plan.rows, s2);
     }
     return e;
 }
