@@ -392,9 +392,12 @@ def main():
             failures.append(f"SpMM row-L1 error {spmm_err:.3g} > {tol}")
         if sddmm_err > tol:
             failures.append(f"SDDMM row-L1 error {sddmm_err:.3g} > {tol} on rows with condition <= 100")
-        if gpu_err_bad > max(2.0 * cpu_err_bad, tol):
-            failures.append(f"SDDMM error {gpu_err_bad:.3g} on ill-conditioned rows exceeds twice the reference CPU loop's "
-                            f"{cpu_err_bad:.3g}")
+        # (on those rows both errors are one draw each of rounding noise of size condition x eps,
+        # in different summation orders, and the maximum is over a handful of rows: the ratio is
+        # a sanity bound; the binding check for them is the per-element one below)
+        if gpu_err_bad > max(10.0 * cpu_err_bad, tol):
+            failures.append(f"SDDMM error {gpu_err_bad:.3g} on ill-conditioned rows exceeds ten times the reference CPU "
+                            f"loop's {cpu_err_bad:.3g}")
         if sddmm_strict > (2e-6 if args.dtype == "f32" else 2e-3):
             failures.append(f"SDDMM per-element error {sddmm_strict:.3g} of the summed terms' magnitude")
         if args.dtype == "f32" and ref_rule_errors:
