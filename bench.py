@@ -34,7 +34,7 @@ def kernel_sources_fingerprint():
     sources is not reported."""
     import hashlib
     h = hashlib.sha256()
-    for name in ("rode_device.hpp", "rode_items.hpp", "rode_window.hpp", "rode_spmm.hip", "rode_sddmm.hip",
+    for name in ("rode_device.hpp", "rode_items.hpp", "rode_units.hpp", "rode_window.hpp", "rode_spmm.hip", "rode_sddmm.hip",
                  "rode_spmm_window.hip", "rode_sddmm_window.hip"):
         with open(os.path.join(ROOT, "rode_amd", "csrc", name), "rb") as f:
             h.update(f.read())
@@ -56,6 +56,9 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--two-streams", action="store_true",
                    help="residue kernels on a second stream (forked from / joined to the first with events)")
+    p.add_argument("--fused", choices=["no", "yes", "probs"], default="no",
+                   help="with --chain: the step is the one-kernel attention forward (rode_hip_attention_forward), "
+                        "\"probs\" also writes the probabilities a gradient needs")
     p.add_argument("--chain", action="store_true",
                    help="step = SDDMM scores -> row softmax -> clear C -> SpMM with those values (sparse attention)")
     p.add_argument("--memset-c", action="store_true",
@@ -197,6 +200,12 @@ def main():
                            csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, stream), "spmm")
 
     def step():
+        if args.chain and args.fused != "no":
+            _lib.check(lib.rode_hip_attention_forward(
+                _lib.DENSE_CODE[args.dtype], m, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
+                csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), B.data_ptr(), float(k) ** -0.5, C.data_ptr(),
+                probs.data_ptr() if args.fused == "probs" else None, stream), "attention")
+            return
         if args.chain:
             sddmm(csr.m1, csr.m2)
             _lib.check(lib.rode_hip_csr_softmax_f32(m, csr.row_offsets.data_ptr(), out.data_ptr(), probs.data_ptr(),
@@ -411,7 +420,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32" if elem == 4 else "f16->f32",
         "data": "synthetic",
         "config": {"workload": f"{args.workload} ({workloads.CONFIGS[args.workload][5]}), K={k}, "
-                               + ("step = SDDMM -> row softmax -> clear C -> SpMM (chained)" if args.chain
+                               + (("step = fused attention forward (one kernel" + (", probabilities written)" if args.fused == "probs" else ")")
+                                   if args.fused != "no" else "step = SDDMM -> row softmax -> clear C -> SpMM (chained)")
+                                  if args.chain
                                   else "step = clear C rows + SpMM + SDDMM"),
                    "rows": m, "cols": n, "nnz": nnz, "K": k, "seg_length": csr.config["seg_length"],
                    "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale,

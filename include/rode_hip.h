@@ -267,6 +267,25 @@ int rode_hip_csr_softmax_f32(int M, const int* d_row_offsets, const float* d_in,
 int rode_hip_csr_softmax_backward_f32(int M, const int* d_row_offsets, const float* d_p, const float* d_dp,
                                       float* d_ds, float scale, void* stream);
 
+/*
+ * Sparse attention in one kernel: out[r, :] = sum over the row's nonzeros of
+ * p[idx] * v[col(idx), :] with p = softmax over the row of
+ * scale * values[idx] * <q[r, :], k[col(idx), :]> -- the results of SDDMM, the row softmax
+ * above and SpMM chained, without their intermediate arrays.  No counterpart in the
+ * reference (its op is the forward SDDMM alone, RoDe_SDDMM/rode_sddmm.py:194-248).
+ *   dtype        RODE_DENSE_F32 or RODE_DENSE_F16: element type of q, k and v
+ *   M            rows of the pattern (= rows of q and of out)
+ *   d            width of q, k and v: 32, 64 or 128
+ *   d_row_offsets, d_column_indices, d_values   the CSR pattern; the row decomposition is
+ *                not used: one wave takes a whole row, whatever its length
+ *   d_q [M x d], d_k, d_v [columns x d]   row-major, 16-byte aligned
+ *   d_out        float [M x d]; rows without nonzeros are written as zeros
+ *   d_probs      NULL, or float [nnz] that receives p (what a gradient needs)
+ */
+int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
+                               const float* d_values, const void* d_q, const void* d_k, const void* d_v,
+                               float scale, float* d_out, float* d_probs, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -115,15 +115,100 @@ def csr_row_softmax(sparse_matrix, scores, scale=1.0):
     return CsrSoftmaxFunction.apply(sparse_matrix, scores, scale)
 
 
-def sparse_attention(mask, q, k, v, scale=None):
+# Rows longer than this many nonzeros keep the one wavefront that the fused kernel gives a
+# row busy for too long; such patterns go through the three separate kernels, whose row
+# decomposition balances them.
+FUSED_MAX_ROW = 16384
+
+
+def _attention_call(csr, values, q, k, v, scale, want_probs):
+    lib = _lib.load()
+    m, d = q.shape
+    out = torch.empty((m, d), dtype=torch.float32, device=q.device)
+    probs = torch.empty_like(values) if want_probs else None
+    with torch.cuda.device(q.device):
+        code = lib.rode_hip_attention_forward(
+            _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"], m, d, csr.row_offsets.data_ptr(),
+            csr.column_indices.data_ptr(), values.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale),
+            out.data_ptr(), probs.data_ptr() if want_probs else None, torch.cuda.current_stream(q.device).cuda_stream)
+    _lib.check(code, "rode_hip_attention_forward")
+    return out, probs
+
+
+class FusedAttentionFunction(torch.autograd.Function):
+    """Forward: one kernel (``rode_hip_attention_forward``).  Backward: the kernels of the
+    chain on the saved probabilities - dP = (dOut v^T)|pattern (SDDMM), the softmax
+    gradient, dq and dk as SpMM on the pattern and its transpose, dv = P^T dOut."""
+
+    @staticmethod
+    def forward(ctx, csr, q, k, v, scale):
+        need = any(ctx.needs_input_grad[1:4])
+        values = csr.values
+        out, probs = _attention_call(csr, values, q.detach().contiguous(), k.detach().contiguous(),
+                                     v.detach().contiguous(), scale, need)
+        ctx.csr, ctx.scale = csr, float(scale)
+        if need:
+            ctx.save_for_backward(probs, q, k, v)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        csr, scale = ctx.csr, ctx.scale
+        probs, q, k, v = ctx.saved_tensors
+        g = g.contiguous().float()
+        dq = dk = dv = None
+        csr_t = perm = None
+        if ctx.needs_input_grad[2] or ctx.needs_input_grad[3]:
+            csr_t, perm = csr.transpose()
+        if ctx.needs_input_grad[3]:
+            dv = _spmm(csr_t, probs[perm], g).to(v.dtype)
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            dp = _sddmm(csr, torch.ones_like(probs), g, v.float())
+            ds = _softmax_call("rode_hip_csr_softmax_backward_f32", csr.row_offsets, probs, dp, scale)
+            ds.mul_(csr.values)  # scores are values (.) (q k^T)
+            if ctx.needs_input_grad[1]:
+                dq = _spmm(csr, ds, k.float()).to(q.dtype)
+            if ctx.needs_input_grad[2]:
+                dk = _spmm(csr_t, ds[perm], q.float()).to(k.dtype)
+        return None, dq, dk, dv, None
+
+
+def sparse_attention(mask, q, k, v, scale=None, fused="auto"):
     """softmax(scale * mask (.) (q k^T)) v on the sparsity pattern of ``mask`` (a
     ``RoDeCSR``; its values multiply the scores, use 1 for a pure mask).  q is (m, d),
     k is (n, d) with d in {32, 64, 128}; v is (n, dv) with dv a multiple of 32.  One
-    row decomposition serves all three kernels; differentiable in q, k and v."""
+    row decomposition serves all three kernels; differentiable in q, k and v.
+
+    ``fused``: "auto" runs the forward pass as one kernel when it applies (dv == d, q, k
+    and v of one dtype, float32 mask values, no row longer than ``FUSED_MAX_ROW``) and as
+    SDDMM -> softmax -> SpMM otherwise; True insists on the one kernel (``ValueError`` when
+    it does not apply), False on the three."""
     from .rode_sddmm import rode_sddmm
     from .rode_spmm import rode_spmm
     if scale is None:
         scale = q.shape[1] ** -0.5
+    if fused not in (True, False, "auto"):
+        raise ValueError(f'fused must be True, False or "auto", got {fused!r}')
+    if fused:
+        why = None
+        if q.dim() != 2 or k.dim() != 2 or v.dim() != 2:
+            why = "q, k and v must be 2-D"
+        elif q.shape[1] not in (32, 64, 128) or k.shape[1] != q.shape[1] or v.shape[1] != q.shape[1]:
+            why = "q, k and v must have the same width, 32, 64 or 128"
+        elif not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.float32, torch.float16)):
+            why = "q, k and v must share one dtype, float32 or float16"
+        elif mask.values.dtype != torch.float32:
+            why = "the mask values must be float32"
+        elif q.shape[0] != mask.m or k.shape[0] != mask.n or v.shape[0] != mask.n:
+            why = f"q must have {mask.m} rows, k and v {mask.n}"
+        elif not (q.is_cuda and q.device == mask.device and k.device == q.device and v.device == q.device):
+            why = f"q, k and v must be on {mask.device}"
+        elif fused == "auto" and mask.max_row_length > FUSED_MAX_ROW:
+            why = "rows too long"
+        if why is None:
+            return FusedAttentionFunction.apply(mask, q, k, v, scale)
+        if fused is True:
+            raise ValueError(f"the fused attention kernel does not apply: {why}")
     scores = rode_sddmm(mask, q, k)
     probs = csr_row_softmax(mask, scores, scale)
     return rode_spmm(mask, v, values=probs)

@@ -282,6 +282,25 @@ int rode_hip_csr_softmax_backward_f32(int M, const int* d_row_offsets, const flo
     return rode::csr_softmax_backward_launch(M, d_row_offsets, d_p, d_dp, d_ds, scale, as_stream(stream));
 }
 
+int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
+                               const float* d_values, const void* d_q, const void* d_k, const void* d_v,
+                               float scale, float* d_out, float* d_probs, void* stream)
+{
+    if (M < 0 || !d_row_offsets) return hipErrorInvalidValue;
+    if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
+    if (M > 0 && (!d_column_indices || !d_values || !d_q || !d_k || !d_v || !d_out)) return hipErrorInvalidValue;
+    if (!aligned16(d_q) || !aligned16(d_k) || !aligned16(d_v) || !aligned16(d_out)) return hipErrorInvalidValue;
+    if (dtype == RODE_DENSE_F32)
+        return rode::attention_launch<float>(M, d, d_row_offsets, d_column_indices, d_values, static_cast<const float*>(d_q),
+                                             static_cast<const float*>(d_k), static_cast<const float*>(d_v), scale, d_out,
+                                             d_probs, as_stream(stream));
+    if (dtype == RODE_DENSE_F16)
+        return rode::attention_launch<__half>(M, d, d_row_offsets, d_column_indices, d_values,
+                                              static_cast<const __half*>(d_q), static_cast<const __half*>(d_k),
+                                              static_cast<const __half*>(d_v), scale, d_out, d_probs, as_stream(stream));
+    return hipErrorInvalidValue;
+}
+
 } // extern "C"
 
 // ---- reference-signature C++ entry points ----------------------------------

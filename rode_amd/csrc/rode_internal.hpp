@@ -62,6 +62,9 @@ template <typename T>
 hipError_t sddmm_window_launch(int m2, int k, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
                                const int* plan, const void* plan_rows, hipStream_t stream);
 
+template <typename T>
+hipError_t attention_launch(int M, int d, const int* row_ptr, const int* col, const float* val, const T* q, const T* k,
+                            const T* v, float scale, float* out, float* probs, hipStream_t stream);
 hipError_t csr_softmax_launch(int M, const int* row_ptr, const float* in, float* out, float scale,
                               hipStream_t stream);
 hipError_t csr_softmax_backward_launch(int M, const int* row_ptr, const float* p, const float* dp, float* ds,

@@ -19,95 +19,12 @@
 //     so a wave works on 64 / LPR rows at once (2 at K=128 fp32, 8 at K=32):
 //     short rows are latency-bound and need many rows in flight per wave.
 #include "rode_items.hpp"
+#include "rode_units.hpp"
 #include "rode_internal.hpp"
 
 namespace rode {
 
 namespace {
-
-// KT = width of the lane tile (32, 64 or 128 elements): LPR = KT / VEC lanes read KT
-// consecutive elements of a dense row per load instruction.  A row of K elements is
-// covered by NS such slabs (KT * NS >= K); EDGE says that the last slab is partial, in
-// which case the lanes past K read nothing and contribute zero.
-template <typename T, int KT>
-struct SddmmShape {
-    static constexpr int kVec = DenseVec<T>::kElems;
-    static constexpr int kLpr = KT / kVec;     // lanes that cover one slab of a dense row
-    static constexpr int kQuads = kLpr / 4;    // slot quads per lane group per unit
-    static_assert(KT % kVec == 0 && kLpr >= 4 && kLpr <= 32 && (kLpr & (kLpr - 1)) == 0,
-                  "unsupported tile width for this dense type");
-};
-
-// <lhs row, rhs row> restricted to this lane's elements.
-template <typename T, int KT, int NS, bool EDGE>
-__device__ __forceinline__ float lane_dot(const float (&a)[NS][SddmmShape<T, KT>::kVec], const T* __restrict__ row_lane,
-                                          int k, int lane_elem)
-{
-    constexpr int VEC = SddmmShape<T, KT>::kVec;
-    float d = 0.f;
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        if (!EDGE || lane_elem + s * KT < k) {
-            float b[VEC];
-            DenseVec<T>::load(row_lane + s * KT, b);
-#pragma unroll
-            for (int x = 0; x < VEC; ++x) d = fmaf(a[s][x], b[x], d);
-        }
-    }
-    return d;
-}
-
-// Dot products of one 32-slot unit of a block segment.  `my_col` is the column of this
-// lane's slot.  Returns the dot product for this lane's slot.
-template <typename T, int KT, int NS, bool EDGE>
-__device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane, const float (&a)[NS][SddmmShape<T, KT>::kVec],
-                                            int my_col, int k, int* lds_cols, int lane)
-{
-    using S = SddmmShape<T, KT>;
-    constexpr int LPR = S::kLpr;
-
-    lds_cols[lane] = my_col;
-    wave_lds_sync();
-
-    const int ls = lane % LPR;                    // lane inside its group
-    const int group_first = (lane & 31) - ls;     // first slot (within the half) of this group
-    const int* group_cols = lds_cols + (lane & 32) + group_first;
-    float result = 0.f;
-
-#pragma unroll
-    for (int q = 0; q < S::kQuads; ++q) {
-        const int4 c4 = *reinterpret_cast<const int4*>(group_cols + 4 * q);
-        const int c[4] = {c4.x, c4.y, c4.z, c4.w};
-        float p[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            p[j] = lane_dot<T, KT, NS, EDGE>(a, rhs_lane + (size_t)c[j] * k, k, ls * S::kVec);
-        // transpose-reduce: afterwards lane (ls & 3) == j holds slot j of the quad
-        const bool hi2 = ls & 2, hi1 = ls & 1;
-        const float k0 = hi2 ? p[2] : p[0], s0 = hi2 ? p[0] : p[2];
-        const float k1 = hi2 ? p[3] : p[1], s1 = hi2 ? p[1] : p[3];
-        const float q0 = k0 + lane_xor2(s0);
-        const float q1 = k1 + lane_xor2(s1);
-        float r = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
-        r = butterfly_sum<4, LPR>(r);
-        if ((ls >> 2) == q) result = r;
-    }
-    return result;
-}
-
-template <typename T, int KT, int NS, bool EDGE>
-__device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int row, int k, int lane,
-                                               float (&a)[NS][SddmmShape<T, KT>::kVec])
-{
-    using S = SddmmShape<T, KT>;
-    const int e0 = (lane % S::kLpr) * S::kVec;
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-#pragma unroll
-        for (int x = 0; x < S::kVec; ++x) a[s][x] = 0.f;
-        if (!EDGE || e0 + s * KT < k) DenseVec<T>::load(lhs + (size_t)row * k + e0 + s * KT, a[s]);
-    }
-}
 
 // One wave per block segment.  Segment s covers the aligned slots
 // [base, base + cnt) with base = st_off[s] & ~3 and cnt = floor((len + mask) / 32) * 32

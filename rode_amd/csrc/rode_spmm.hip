@@ -26,6 +26,7 @@
 // so a non-finite B row can never leak into a row that does not reference it
 // (the reference multiplies B[0, :] by zero there, RoDeSpmm.cu:271-274).
 #include "rode_items.hpp"
+#include "rode_units.hpp"
 #include "rode_internal.hpp"
 
 #include <type_traits>
@@ -47,56 +48,6 @@ constexpr int kOwnedMinSegments = 16384;
 // are processed by one launch (spmm_pair_kernel).  Above it the residue kernel runs on its
 // own: it needs a quarter of the block kernel's registers and keeps twice the waves per CU.
 constexpr int kPairMaxWorkgroups = 16384;
-
-template <typename T, int TN>
-struct SpmmShape {
-    using Acc = typename DenseVec<T>::Acc;          // type of values, accumulators and C
-    static constexpr int kVec = DenseVec<T>::kElems;
-    static constexpr int kLpr = TN / kVec;          // lanes that cover one B-row tile
-    static constexpr int kGroupsWave = kWave / kLpr; // lane groups per wave
-    static_assert(TN % kVec == 0 && kLpr >= 4 && kLpr <= 32 && (kLpr & (kLpr - 1)) == 0,
-                  "unsupported tile width for this dense type");
-};
-
-__device__ __forceinline__ void load_quad(const float* p, float (&v)[4])
-{
-    const float4 t = *reinterpret_cast<const float4*>(p);
-    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-}
-__device__ __forceinline__ void load_quad(const double* p, double (&v)[4])
-{
-    const double2 t0 = *reinterpret_cast<const double2*>(p), t1 = *reinterpret_cast<const double2*>(p + 2);
-    v[0] = t0.x; v[1] = t0.y; v[2] = t1.x; v[3] = t1.y;
-}
-
-// acc += sum over the slot quads {first_quad, first_quad + stride, ...} < nquads of
-// value * B[col, tile].  QUADS_MAX bounds the trip count at compile time.
-template <typename T, int TN, int QUADS_MAX, bool FULL>
-__device__ __forceinline__ void spmm_gather(const T* __restrict__ b_lane, size_t ldb,
-                                            typename DenseVec<T>::Acc (&acc)[SpmmShape<T, TN>::kVec],
-                                            const int* lds_col, const typename DenseVec<T>::Acc* lds_val,
-                                            int first_quad, int stride, int nquads)
-{
-    using A = typename DenseVec<T>::Acc;
-    constexpr int VEC = SpmmShape<T, TN>::kVec;
-#pragma unroll
-    for (int i = 0; i < QUADS_MAX; ++i) {
-        const int q = first_quad + i * stride;
-        if (FULL || q < nquads) {
-            const int4 c4 = *reinterpret_cast<const int4*>(lds_col + 4 * q);
-            const int c[4] = {c4.x, c4.y, c4.z, c4.w};
-            A v[4];
-            load_quad(lds_val + 4 * q, v);
-            A b[4][VEC];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) DenseVec<T>::load(b_lane + (size_t)c[j] * ldb, b[j]);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int x = 0; x < VEC; ++x) acc[x] = fma(v[j], b[j][x], acc[x]);
-        }
-    }
-}
 
 template <int VEC>
 __device__ __forceinline__ void store_row(float* dst, const float (&acc)[VEC])

@@ -60,6 +60,8 @@ class RoDeCSR:
         self.column_indices = column_indices.to(dtype=torch.int32, device=self.device).contiguous()
         self.values = values.to(dtype=torch.float32, device=self.device).contiguous()
         self.row_offsets = self.row_offsets_cpu.to(device=self.device)
+        ro = self.row_offsets_cpu
+        self.max_row_length = int((ro[1:] - ro[:-1]).max()) if ro.numel() > 1 else 0
         if locality not in (True, False, "auto"):
             raise ValueError(f'locality must be True, False or "auto", got {locality!r}')
         self.locality = locality

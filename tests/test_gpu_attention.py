@@ -162,8 +162,9 @@ def test_sddmm_and_spmm_gradients(k):
     assert not rode_sddmm(csr, lhs.detach(), rhs.detach()).requires_grad
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("half", [False, True])
-def test_sparse_attention_against_dense(half):
+def test_sparse_attention_against_dense(half, fused):
     from gpu_common import DEV, make_csr
     from rode_amd import sparse_attention, workloads
     m, n, rp, col, val = workloads.config("c5_attention", 1 / 16)
@@ -174,7 +175,7 @@ def test_sparse_attention_against_dense(half):
     q, k, v = mk(m).requires_grad_(), mk(n).requires_grad_(), mk(n).requires_grad_()
     w = torch.from_numpy(rng.standard_normal((m, d)).astype(np.float32)).to(DEV)
     mask = make_csr(rp, col, val, m, n, d)
-    out = sparse_attention(mask, q, k, v)
+    out = sparse_attention(mask, q, k, v, fused=fused)
     (out * w).sum().backward()
     q64, k64, v64 = (t.detach().double().requires_grad_() for t in (q, k, v))
     allowed = _dense(rp, col, val, m, n) != 0
@@ -185,3 +186,83 @@ def test_sparse_attention_against_dense(half):
     for got, want in ((out, ref), (q.grad, q64.grad), (k.grad, k64.grad), (v.grad, v64.grad)):
         scale = want.abs().max().item()
         assert (got.detach().double() - want.detach()).abs().max().item() <= tol * scale
+
+
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("half", [False, True])
+def test_fused_attention_kernel_against_the_three_kernels(d, half):
+    """rode_hip_attention_forward against fp64 on the host and against SDDMM -> softmax ->
+    SpMM of this library: weighted mask values, rows without nonzeros, rows of 1, 63, 64,
+    65 and 700 nonzeros (one step, a full step, a step and one slot, many steps), scores
+    large enough that the running maximum matters."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import csr_row_softmax, rode_sddmm, sparse_attention
+    from rode_amd.autograd import _attention_call
+    rng = np.random.default_rng(100 + d)
+    m, n = 300, 900
+    lens = rng.integers(0, 90, m)
+    lens[:8] = [0, 1, 63, 64, 65, 700, 0, 128]
+    rp = np.zeros(m + 1, dtype=np.int32)
+    rp[1:] = np.cumsum(lens)
+    col = np.concatenate([np.sort(rng.choice(n, l, replace=False)) for l in lens]).astype(np.int32)
+    val = rng.uniform(0.5, 1.5, len(col)).astype(np.float32)
+    dt = torch.float16 if half else torch.float32
+    mk = lambda r, s: torch.from_numpy((s * rng.standard_normal((r, d))).astype(np.float32)).to(DEV, dt)
+    q, k, v = mk(m, 1.5), mk(n, 1.5), mk(n, 1.0)
+    mask = make_csr(rp, col, val, m, n, d)
+    scale = 0.37
+    out, probs = _attention_call(mask, mask.values, q, k, v, scale, True)
+    out_only, none = _attention_call(mask, mask.values, q, k, v, scale, False)
+    assert none is None and torch.equal(out, out_only)
+    # fp64 on the host
+    q64, k64, v64 = (t.double().cpu().numpy() for t in (q, k, v))
+    rows = np.repeat(np.arange(m), lens)
+    sc = scale * val.astype(np.float64) * np.einsum("ij,ij->i", q64[rows], k64[col])
+    ref_out = np.zeros((m, d))
+    ref_p = np.zeros(len(col))
+    for r in range(m):
+        a, b = rp[r], rp[r + 1]
+        if b > a:
+            e = np.exp(sc[a:b] - sc[a:b].max())
+            ref_p[a:b] = e / e.sum()
+            ref_out[r] = ref_p[a:b] @ v64[col[a:b]]
+    # tolerance: scores reach +-30 here, an fp32 dot product of 128 such terms is off by ~1e-5,
+    # and a probability near 1/2 moves by as much; fp16 operands are compared after rounding
+    tol = 2e-3 if half else 5e-5
+    assert np.abs(probs.cpu().numpy() - ref_p).max() <= tol
+    assert np.abs(out.cpu().numpy() - ref_out).max() <= tol * max(1.0, np.abs(ref_out).max())
+    assert not out[0].any() and not out[6].any()  # rows without nonzeros
+    # the three kernels
+    chain_p = csr_row_softmax(mask, rode_sddmm(mask, q, k), scale)
+    assert (chain_p - probs).abs().max().item() <= tol
+    chain = sparse_attention(mask, q, k, v, scale=scale, fused=False)
+    assert (chain - out).abs().max().item() <= tol * max(1.0, chain.abs().max().item())
+
+
+def test_fused_attention_dispatch():
+    from gpu_common import DEV, make_csr
+    from helpers import random_csr
+    from rode_amd import autograd, sparse_attention
+    rng = np.random.default_rng(5)
+    m, n, d = 64, 96, 32
+    rp, col, val = random_csr(rng, m, n, 20)
+    mask = make_csr(rp, col, val, m, n, d)
+    mk = lambda r, w: torch.from_numpy(rng.standard_normal((r, w)).astype(np.float32)).to(DEV)
+    q, k = mk(m, d), mk(n, d)
+    with pytest.raises(ValueError, match="same width"):
+        sparse_attention(mask, q, k, mk(n, 64), fused=True)
+    with pytest.raises(ValueError, match="dtype"):
+        sparse_attention(mask, q, k.half(), mk(n, d), fused=True)
+    with pytest.raises(ValueError, match="fused must be"):
+        sparse_attention(mask, q, k, mk(n, d), fused="yes")
+    # other widths of v, and patterns with very long rows, take the three kernels by themselves
+    assert sparse_attention(mask, q, k, mk(n, 64)).shape == (m, 64)
+    v = mk(n, d)
+    limit = autograd.FUSED_MAX_ROW
+    try:
+        autograd.FUSED_MAX_ROW = 1
+        a = sparse_attention(mask, q, k, v)
+    finally:
+        autograd.FUSED_MAX_ROW = limit
+    b = sparse_attention(mask, q, k, v)
+    assert (a - b).abs().max().item() <= 2e-5 * max(1.0, b.abs().max().item())
