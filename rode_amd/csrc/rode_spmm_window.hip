@@ -40,7 +40,7 @@ spmm_residue_window_kernel(int m2, int n, int owned_slots, const int* __restrict
         const bool ok = !EDGE || ls * VEC < n;
         res_prefetch(pf, reinterpret_cast<const char*>(B + (size_t)d.w0 * n + (ok ? ls * VEC : 0)), row_bytes, d.wn, ok);
     }
-    ResidueRow rr;
+    ResidueRow<false> rr;
     float* my_v = lds_val + group * kResValStride;
     load_planned_row(pc, local, owned_slots, val, my_v, rr);
     const int wave_quads = wave_max_quads(rr.quads);

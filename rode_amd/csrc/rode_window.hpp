@@ -65,6 +65,7 @@ constexpr int kResPrefetch = (kResWinVecs + kResThreads - 1) / kResThreads;    /
 // share each set).
 constexpr int kResValStride = kBlockItems + 4;
 static_assert(kPlanResidueChunk % kResRows == 0, "a workgroup takes a whole fraction of a chunk");
+static_assert(kResWinVecs * 16 <= 65536, "an LDS address of the window fits 16 bits");
 static_assert(kResidueWindowRowsMax == 512 && kBlockItems == 32, "a plan entry holds 9 bits of window row and 5 of slot");
 
 inline int grid_for_residue_parts(int m2)
@@ -121,13 +122,17 @@ __device__ __forceinline__ void res_fill(uint4* win, const char* src_lane, size_
 // addr[i]: LDS byte address of this lane's 16 bytes of the dense row of position i; for a
 // position whose dense row is outside the window (bit i of missmask) it is the address of
 // one of the row's positions that is inside, and the data has to come from memory instead.
+// PACKED: two addresses (each below 64 K) per register, position 2 i in the low half of
+// addr[i] and 2 i + 1 in the high half - for a kernel that needs the 16 registers elsewhere
+// and pays one extra instruction per read for it.
+template <bool PACKED>
 struct ResidueRow {
     int row;   // -1: nothing to do
     int first; // first residue slot of the row in column_indices / values
     int cnt, quads;
     unsigned missmask;
     bool accumulate; // the row also has block segments (SpMM adds instead of storing)
-    int addr[kBlockItems];
+    unsigned addr[PACKED ? kBlockItems / 2 : kBlockItems];
 };
 
 // The slot (counted from rr.first) that the plan put at position i of row `local` of a chunk.
@@ -136,13 +141,51 @@ __device__ __forceinline__ int planned_slot(const PlannedChunk& pc, int local, i
     return (pc.entry[local][i] >> 9) & (kBlockItems - 1);
 }
 
+// Turns a row record of the plan and the row's 32 entries into the lane group's view of
+// the row (everything but the values).  skip_owned_slots: rows with block segments and at
+// most that many aligned slots are left to the block kernel (SpMM under the whole-lists
+// promise); 0 for SDDMM.  usable = false: the chunk has no window (its records are not
+// filled in), the row is skipped.
+template <bool PACKED>
+__device__ __forceinline__ void decode_planned_row(const int4& meta, const uint4 (&e4)[kBlockItems / 8], bool usable,
+                                                   int skip_owned_slots, ResidueRow<PACKED>& rr)
+{
+    const int ls = threadIdx.x % kResLanes;
+    rr.row = meta.x;
+    rr.first = meta.y;
+    rr.cnt = meta.z & 0xff;
+    rr.accumulate = (meta.z >> 8) & 1;
+    rr.missmask = (unsigned)meta.w;
+    if (!usable || rr.row < 0 || (rr.accumulate && ((meta.z >> 16) & 0xffff) <= skip_owned_slots)) {
+        rr.row = -1;
+        rr.first = 0;
+        rr.cnt = 0;
+        rr.missmask = 0;
+    }
+    rr.quads = (rr.cnt + 3) / 4;
+#pragma unroll
+    for (int i = 0; i < kBlockItems / 8; ++i) {
+        const unsigned w[4] = {e4[i].x, e4[i].y, e4[i].z, e4[i].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const unsigned even = (((w[j] & 0xffffu) & (kResidueWindowRowsMax - 1)) * kResLanes + ls) * 16;
+            const unsigned odd = (((w[j] >> 16) & (kResidueWindowRowsMax - 1)) * kResLanes + ls) * 16;
+            if (PACKED) {
+                rr.addr[4 * i + j] = even | (odd << 16);
+            } else {
+                rr.addr[8 * i + 2 * j] = even;
+                rr.addr[8 * i + 2 * j + 1] = odd;
+            }
+        }
+    }
+}
+
 // Loads row `local` of a planned chunk for this lane group: the LDS addresses of its 32
 // positions into registers, its values (in position order, 0 past the row) into `my_val`
-// (32 floats of this group; the 8 lanes write 4 each).  skip_owned_slots: rows with block
-// segments and at most that many aligned slots are left to the block kernel (SpMM under
-// the whole-lists promise); 0 for SDDMM.
+// (32 floats of this group; the 8 lanes write 4 each).
+template <bool PACKED>
 __device__ __forceinline__ void load_planned_row(const PlannedChunk& pc, int local, int skip_owned_slots,
-                                                 const float* __restrict__ val, float* my_val, ResidueRow& rr)
+                                                 const float* __restrict__ val, float* my_val, ResidueRow<PACKED>& rr)
 {
     const int ls = threadIdx.x % kResLanes;
     const int4 meta = *reinterpret_cast<const int4*>(&pc.meta[local]);
@@ -150,31 +193,12 @@ __device__ __forceinline__ void load_planned_row(const PlannedChunk& pc, int loc
     uint4 e4[kBlockItems / 8];
 #pragma unroll
     for (int i = 0; i < kBlockItems / 8; ++i) e4[i] = entries[i];
-    rr.row = meta.x;
-    rr.first = meta.y;
-    rr.cnt = meta.z & 0xff;
-    rr.accumulate = (meta.z >> 8) & 1;
-    rr.missmask = (unsigned)meta.w;
-    if (rr.row < 0 || (rr.accumulate && ((meta.z >> 16) & 0xffff) <= skip_owned_slots)) {
-        rr.row = -1;
-        rr.cnt = 0;
-        rr.missmask = 0;
-    }
-    rr.quads = (rr.cnt + 3) / 4;
+    decode_planned_row(meta, e4, true, skip_owned_slots, rr);
     constexpr int OWN = kBlockItems / kResLanes;
 #pragma unroll
     for (int i = 0; i < OWN; ++i) {
         const int pos = ls + i * kResLanes;
         my_val[pos] = pos < rr.cnt ? val[rr.first + planned_slot(pc, local, pos)] : 0.f;
-    }
-#pragma unroll
-    for (int i = 0; i < kBlockItems / 8; ++i) {
-        const unsigned w[4] = {e4[i].x, e4[i].y, e4[i].z, e4[i].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            rr.addr[8 * i + 2 * j] = (int)((((w[j] & 0xffffu) & (kResidueWindowRowsMax - 1)) * kResLanes + ls) * 16);
-            rr.addr[8 * i + 2 * j + 1] = (int)((((w[j] >> 16) & (kResidueWindowRowsMax - 1)) * kResLanes + ls) * 16);
-        }
     }
 }
 
