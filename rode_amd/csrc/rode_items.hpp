@@ -60,8 +60,12 @@ __device__ __forceinline__ bool sddmm_block_item(int seg, int m1, int lane, cons
 // SpMM.  owned_slots > 0 means that the caller promised complete lists: a row of at
 // most owned_slots aligned slots is then summed whole - all its segments and its tail -
 // by the wave of its first segment (one update of C), longer rows are merged into
-// leaders.  owned_slots == 0: every segment on its own, rounded to whole 32-slot units
-// as in RoDeSpmm.cu:210-234.
+// leaders.  owned_slots < 0: no promise, but segments are merged into leaders all the
+// same - a leader only ever takes segments of the list it was given (a slice of the lists
+// merges within the slice), so every slot still contributes exactly once.
+// owned_slots == 0: every segment on its own, rounded to whole 32-slot units as in
+// RoDeSpmm.cu:210-234 (small launches: they need the waves more than they mind the
+// atomics).
 __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots, int lane,
                                                 const int* __restrict__ block_rows, const int* __restrict__ st_off,
                                                 const int* __restrict__ row_ptr, BlockItem& it)
@@ -76,7 +80,7 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
         it.cnt = row_end - it.base;
         return true;
     }
-    if (owned_slots > 0)
+    if (owned_slots != 0)
         return merged_leader(kSpmmMergeSlots, seg, m1, lane, row, row_start, row_end, block_rows, st_off, it);
     const int start = st_off[seg];
     const int end = min(row_end, st_off[seg + 1]);
@@ -85,6 +89,22 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
     it.base = start - it.mask;
     it.cnt = (end - start + it.mask) / kBlockItems * kBlockItems;
     return true;
+}
+
+// The row of segment `seg` if spmm_block_item() gives it a work item, else -1 (a follower,
+// or past the list).  The same rules, without the extent of the item: what the waves of a
+// workgroup need to know about each other.
+__device__ __forceinline__ int spmm_block_leader_row(int seg, int m1, int owned_slots,
+                                                     const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                                                     const int* __restrict__ row_ptr)
+{
+    if (seg >= m1) return -1;
+    const int row = block_rows[seg];
+    if (seg == 0 || block_rows[seg - 1] != row || owned_slots == 0) return row;
+    const int row_start = row_ptr[row];
+    const int row_base = row_start - (row_start & (kVecLen - 1));
+    if (row_ptr[row + 1] - row_base <= owned_slots) return -1; // summed whole by the wave of its first segment
+    return (st_off[seg] - row_base) / kSpmmMergeSlots == (st_off[seg - 1] - row_base) / kSpmmMergeSlots ? -1 : row;
 }
 
 // Slots [first, first + cnt) of one residue row: with N = len + (start & 3), rows with

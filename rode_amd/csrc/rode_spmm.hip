@@ -82,23 +82,24 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, const int*
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int seg0 = xcd_logical_block(bid, nblocks) * kWavesPerWg;
     const int seg = seg0 + wave;
-    // Do neighbouring segments of this workgroup belong to one row (a long row)?  Every
-    // wave finds the same answer.  If so, the waves add their sums up in LDS and the row
-    // of C gets one update per workgroup instead of one per segment.
-    bool shared_row = false;
-    {
-        int prev = -1;
-#pragma unroll
-        for (int i = 0; i < kWavesPerWg; ++i) {
-            const int r = seg0 + i < m1 ? block_rows[seg0 + i] : -2 - i;
-            shared_row = shared_row || r == prev;
-            prev = r;
-        }
-    }
     BlockItem it{-1, 0, 0, 0};
     const bool active = seg < m1 && spmm_block_item(seg, m1, owned_slots, lane, block_rows, st_off, row_ptr, it);
-    if (!active && !shared_row) return; // nobody waits for this wave
-    const int row = it.row, mask = it.mask, base = it.base, cnt = active ? it.cnt : 0;
+    // A wave without a work item leaves at once (with the reference's 32-slot segments that
+    // is most waves); the barrier below then counts only the waves that are still running
+    // (S_BARRIER waits on the surviving waves of a workgroup).
+    if (!active) return;
+    // Do two work items of this workgroup add to the same row (neighbouring segments of a
+    // long row that are not merged into one leader)?  Every wave finds the same answer.  If
+    // so, the waves add their sums up in LDS and the row of C gets one update per run of
+    // such work items instead of one each.
+    int item_row[kWavesPerWg]; // the row of each wave's work item, -1: that wave has none (and has left)
+    bool shared_row = false;
+#pragma unroll
+    for (int i = 0; i < kWavesPerWg; ++i) {
+        item_row[i] = spmm_block_leader_row(seg0 + i, m1, owned_slots, block_rows, st_off, row_ptr);
+        if (i > 0) shared_row = shared_row || (item_row[i] >= 0 && item_row[i] == item_row[i - 1]);
+    }
+    const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
 
     const int ls = lane % LPR, group = lane / LPR;
     const int tile = blockIdx.y * TN;
@@ -142,19 +143,25 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, const int*
     for (int x = 0; x < VEC; ++x) total[x] = butterfly_sum<LPR, kWave>(acc[x]);
     if (shared_row) {
         __shared__ __attribute__((aligned(16))) A wg_sum[kWavesPerWg][TN];
-        __shared__ int wg_row[kWavesPerWg];
         if (group == 0) {
 #pragma unroll
             for (int x = 0; x < VEC; ++x) wg_sum[wave][ls * VEC + x] = total[x];
         }
-        if (lane == 0) wg_row[wave] = active ? row : -1;
         __syncthreads();
         // the first wave of a run of equal rows takes the sums of the others
-        if (!active || (wave > 0 && wg_row[wave - 1] == row)) return;
-        for (int w = wave + 1; w < kWavesPerWg && wg_row[w] == row; ++w) {
+        bool first_of_run = true, run_goes_on = true;
 #pragma unroll
-            for (int x = 0; x < VEC; ++x) total[x] += wg_sum[w][ls * VEC + x];
+        for (int w = 0; w < kWavesPerWg; ++w) {
+            if (w + 1 == wave && item_row[w] == row) first_of_run = false;
+            if (w > wave) {
+                run_goes_on = run_goes_on && item_row[w] == row;
+                if (run_goes_on && first_of_run) {
+#pragma unroll
+                    for (int x = 0; x < VEC; ++x) total[x] += wg_sum[w][ls * VEC + x];
+                }
+            }
         }
+        if (!first_of_run) return;
     }
     A* c_lane = C + (size_t)row * n + tile + ls * VEC;
 #pragma unroll
@@ -258,7 +265,7 @@ spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, const int* __re
     if ((int)blockIdx.x < g1)
         spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, block_rows, st_off, row_ptr, col, val, B, C);
     else
-        spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, owned_slots, residue_rows, row_ptr, col, val,
+        spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, max(owned_slots, 0), residue_rows, row_ptr, col, val,
                                        B, C, plan);
 }
 
@@ -308,6 +315,9 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
 {
     const int tiles = (n + TN - 1) / TN;
     const int owned_slots = (flags & kSpmmWholeLists) && m1 >= kOwnedMinSegments ? kOwnedRowSlots : 0;
+    // what the block kernel is told: rows it owns, or (negative) only that it may merge short
+    // segments - which needs no promise, and with this many segments costs no parallelism
+    const int block_owned = owned_slots > 0 ? owned_slots : (m1 >= kOwnedMinSegments ? -1 : 0);
     constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
     const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0 || tiles > 65535) return hipErrorInvalidConfiguration;
@@ -322,13 +332,13 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     hipError_t e = hipSuccess;
     if (block && residue && standard_residue && s1 == s2 && (long long)(g1 + g2) * tiles <= kPairMaxWorkgroups) {
         dim3 grid(g1 + g2, tiles);
-        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, owned_slots, block_rows, residue_rows,
+        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, block_rows, residue_rows,
                                                                    st_off, row_ptr, col, val, B, C, plan.dev);
         e = hipGetLastError();
     } else {
         if (block) {
             dim3 grid(g1, tiles);
-            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, owned_slots, block_rows, st_off, row_ptr,
+            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, block_rows, st_off, row_ptr,
                                                                         col, val, B, C);
             e = hipGetLastError();
         }

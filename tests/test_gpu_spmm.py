@@ -390,7 +390,9 @@ def test_whole_row_mode_and_split_calls(seg, half):
     passes), rows of 32..1024 slots are summed by one wave, tail included; rows just
     outside that range, unaligned starts and empty rows sit next to them here.  The
     typed entry points make no such promise: a caller who feeds the two lists in
-    separate calls, or the block list in two halves, must get the same matrix."""
+    separate calls, or the block list in two halves, must get the same matrix (with
+    >= 16384 segments per call the block kernel still merges short segments of a row,
+    within the slice it was given: seg 32 and 96 here)."""
     import oracle
     from gpu_common import DEV, TOL_F16, TOL_F32, make_csr, round_half, run_spmm
     from helpers import spmm_row_l1_error
