@@ -286,6 +286,23 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
                                const float* d_values, const void* d_q, const void* d_k, const void* d_v,
                                float scale, float* d_out, float* d_probs, void* stream);
 
+/*
+ * The transposed pattern of a CSR matrix (M rows, N columns, nnz nonzeros): what the
+ * gradients with respect to the column-side operands (SDDMM's rhs, SpMM's B) run on.  No
+ * counterpart in the reference (forward-only, RoDe_SDDMM/rode_sddmm.py:194-248).
+ *   d_perm               int[nnz] out: the nonzero indices ordered by (column, index), so
+ *                        values_t = values[perm]; nonzeros of one column keep their input
+ *                        order (rows ascending), the result is the same on every run
+ *   d_t_row_offsets      int[N + 1] out
+ *   d_t_column_indices   int[nnz] out: the row of nonzero perm[j]
+ *   d_workspace          rode_hip_csr_transpose_workspace_bytes(nnz) bytes, 16-byte aligned
+ * Column indices must lie in [0, N).  A stable radix sort, 4 bits per pass.
+ */
+size_t rode_hip_csr_transpose_workspace_bytes(int nnz);
+int rode_hip_csr_transpose(int M, int N, int nnz, const int* d_row_offsets, const int* d_column_indices,
+                           int* d_t_row_offsets, int* d_t_column_indices, int* d_perm, void* d_workspace,
+                           size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

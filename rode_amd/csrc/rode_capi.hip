@@ -301,6 +301,20 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
     return hipErrorInvalidValue;
 }
 
+size_t rode_hip_csr_transpose_workspace_bytes(int nnz) { return rode::csr_transpose_workspace_bytes(nnz); }
+
+int rode_hip_csr_transpose(int M, int N, int nnz, const int* d_row_offsets, const int* d_column_indices,
+                           int* d_t_row_offsets, int* d_t_column_indices, int* d_perm, void* d_workspace,
+                           size_t workspace_bytes, void* stream)
+{
+    if (M < 0 || N < 0 || nnz < 0 || !d_t_row_offsets) return hipErrorInvalidValue;
+    if (nnz > 0 && (!d_row_offsets || !d_column_indices || !d_t_column_indices || !d_perm || !d_workspace || N == 0 ||
+                    M == 0 || !aligned16(d_workspace) || workspace_bytes < rode::csr_transpose_workspace_bytes(nnz)))
+        return hipErrorInvalidValue;
+    return rode::csr_transpose_launch(M, N, nnz, d_row_offsets, d_column_indices, d_t_row_offsets, d_t_column_indices,
+                                      d_perm, d_workspace, as_stream(stream));
+}
+
 } // extern "C"
 
 // ---- reference-signature C++ entry points ----------------------------------

@@ -65,6 +65,9 @@ hipError_t sddmm_window_launch(int m2, int k, const int* col, const float* val, 
 template <typename T>
 hipError_t attention_launch(int M, int d, const int* row_ptr, const int* col, const float* val, const T* q, const T* k,
                             const T* v, float scale, float* out, float* probs, hipStream_t stream);
+size_t csr_transpose_workspace_bytes(int nnz);
+hipError_t csr_transpose_launch(int M, int N, int nnz, const int* row_ptr, const int* col, int* t_row_ptr, int* t_col,
+                                int* perm, void* workspace, hipStream_t stream);
 hipError_t csr_softmax_launch(int M, const int* row_ptr, const float* in, float* out, float scale,
                               hipStream_t stream);
 hipError_t csr_softmax_backward_launch(int M, const int* row_ptr, const float* p, const float* dp, float* ds,

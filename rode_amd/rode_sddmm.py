@@ -136,14 +136,11 @@ class RoDeCSR:
         then cached).  Needed by the gradients with respect to the column-side operands."""
         cached = self._shared.get("transpose")
         if cached is None:
-            lens = (self.row_offsets[1:] - self.row_offsets[:-1]).to(torch.int64)
-            rows = torch.repeat_interleave(torch.arange(self.m, device=self.device), lens)
-            cols = self.column_indices.to(torch.int64)
-            _, perm = torch.sort(cols, stable=True)  # rows stay ascending inside a column
-            row_offsets_t = torch.zeros(self.n + 1, dtype=torch.int64, device=self.device)
-            row_offsets_t[1:] = torch.cumsum(torch.bincount(cols, minlength=self.n), 0)
-            csr_t = RoDeCSR(row_offsets_t.to(torch.int32), rows[perm].to(torch.int32), self.values.float()[perm],
-                            self.device, self.n, self.m, self.k, config=self.config, locality=self.locality)
+            row_offsets_t, rows_t, perm = rode_sddmm_hip.csr_transpose(self.row_offsets, self.column_indices,
+                                                                       self.m, self.n)
+            perm = perm.to(torch.int64)
+            csr_t = RoDeCSR(row_offsets_t, rows_t, self.values.float()[perm], self.device, self.n, self.m, self.k,
+                            config=self.config, locality=self.locality)
             cached = (csr_t, perm)
             self._shared["transpose"] = cached
         csr_t, perm = cached

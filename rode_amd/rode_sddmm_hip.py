@@ -130,6 +130,29 @@ def window_plan_rows(plan, residue_indices, m2, row_offsets, column_indices):
     return plan
 
 
+def csr_transpose(row_offsets, column_indices, m, n):
+    """``(row_offsets_t, column_indices_t, perm)`` of the transposed pattern, all int32 on
+    the device of the inputs: nonzero j of the transposed matrix is nonzero ``perm[j]`` of
+    the input (ordered by column, then by index), its column is that nonzero's row."""
+    for t, name in ((row_offsets, "row_offsets"), (column_indices, "column_indices")):
+        _check_input(t, name)
+        _check(t.dtype == torch.int32, f"{name} must be int32")
+    _check(row_offsets.numel() == m + 1, "row_offsets must have m + 1 entries")
+    nnz = column_indices.numel()
+    lib = _lib.load()
+    dev = row_offsets.device
+    row_offsets_t = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    column_indices_t = torch.empty(nnz, dtype=torch.int32, device=dev)
+    perm = torch.empty(nnz, dtype=torch.int32, device=dev)
+    ws_bytes = lib.rode_hip_csr_transpose_workspace_bytes(nnz)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.rode_hip_csr_transpose(m, n, nnz, row_offsets.data_ptr(), column_indices.data_ptr(),
+                                              row_offsets_t.data_ptr(), column_indices_t.data_ptr(), perm.data_ptr(),
+                                              ws.data_ptr(), ws_bytes, _stream_handle(dev)), "rode_hip_csr_transpose")
+    return row_offsets_t, column_indices_t, perm
+
+
 def _plan_args(plan):
     if plan is None or plan.rows is None:
         return None, None, None

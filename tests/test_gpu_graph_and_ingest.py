@@ -84,3 +84,54 @@ def test_matrix_market_file_through_the_path(tmp_path):
         ref, scale = oracle.sddmm_f64(rp_, col_, val_, lhs, B, with_abs=True)
         assert np.max(np.abs(got - ref) / np.maximum(scale, 1e-30), initial=0.0) <= 2e-6
         assert not got[val_ == 0].any()  # padding entries produce zeros
+
+
+def _transpose_reference(rp, col, m, n):
+    """Stable sort by column on the host: (row_offsets_t, rows in that order, perm)."""
+    rows = np.repeat(np.arange(m, dtype=np.int64), np.diff(rp))
+    perm = np.argsort(col, kind="stable")
+    rp_t = np.zeros(n + 1, dtype=np.int64)
+    rp_t[1:] = np.cumsum(np.bincount(col, minlength=n))
+    return rp_t, rows[perm], perm
+
+
+@pytest.mark.parametrize("m,n,mean_len,seed", [
+    (1, 1, 1, 0), (7, 5, 3, 1), (300, 17, 9, 2), (257, 70000, 40, 3), (5000, 4097, 30, 4), (40, 1 << 20, 500, 5),
+])
+def test_csr_transpose_is_the_stable_sort_by_column(m, n, mean_len, seed):
+    """rode_hip_csr_transpose against numpy's stable argsort, exactly: one to six radix
+    passes (n from 1 to 2^20), columns without nonzeros at both ends and in the middle,
+    duplicate (row, column) entries (their input order is kept), empty rows."""
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(seed)
+    lens = rng.poisson(mean_len, m)
+    lens[rng.integers(0, m, max(1, m // 10))] = 0
+    rp = np.zeros(m + 1, dtype=np.int32)
+    rp[1:] = np.cumsum(lens)
+    lo, hi = (n // 8, n - n // 8) if n > 16 else (0, n)   # the first and last columns stay empty
+    col = rng.integers(lo, max(hi, lo + 1), rp[-1]).astype(np.int32)   # with repetitions inside a row
+    dev = torch.device("cuda:0")
+    got = rode_sddmm_hip.csr_transpose(torch.from_numpy(rp).to(dev), torch.from_numpy(col).to(dev), m, n)
+    want = _transpose_reference(rp, col, m, n)
+    for g, w, name in zip(got, want, ("row_offsets_t", "column_indices_t", "perm")):
+        assert g.dtype == torch.int32 and np.array_equal(g.cpu().numpy().astype(np.int64), w), name
+
+
+def test_csr_transpose_edges_and_full_size():
+    from rode_amd import _lib, rode_sddmm_hip, workloads
+    dev = torch.device("cuda:0")
+    # no nonzeros: offsets all zero
+    rp = torch.zeros(6, dtype=torch.int32, device=dev)
+    rp_t, col_t, perm = rode_sddmm_hip.csr_transpose(rp, torch.empty(0, dtype=torch.int32, device=dev), 5, 9)
+    assert rp_t.shape == (10,) and not rp_t.any() and col_t.numel() == 0 and perm.numel() == 0
+    # a workspace that is too small is refused
+    lib = _lib.load()
+    one = torch.zeros(2, dtype=torch.int32, device=dev)
+    assert lib.rode_hip_csr_transpose(1, 1, 1, one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(),
+                                      one.data_ptr(), one.data_ptr(), 8, None) != 0
+    # the power-law benchmark pattern, 2 M x 2 M with 47.9 M nonzeros
+    m, n, rp, col, val = workloads.config("c4_powerlaw")
+    got = rode_sddmm_hip.csr_transpose(torch.from_numpy(rp).to(dev), torch.from_numpy(col).to(dev), m, n)
+    want = _transpose_reference(rp, col, m, n)
+    for g, w, name in zip(got, want, ("row_offsets_t", "column_indices_t", "perm")):
+        assert np.array_equal(g.cpu().numpy().astype(np.int64), w), name
