@@ -296,7 +296,12 @@ def main():
     traffic, traffic_note = None, "no counter run of this workload under profiles/"
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
-        entry = json.load(open(tpath)).get(f"{args.workload}/k{k}/{args.dtype}/seg{csr.config['seg_length']}/{dominant}")
+        table = json.load(open(tpath))
+        prefix = f"{args.workload}/k{k}/{args.dtype}/seg{csr.config['seg_length']}/"
+        # with a locality plan the residue rows are the window kernel's
+        windowed = csr.plan is not None and dominant.endswith("residue") and k * elem > 128
+        entry = table.get(prefix + dominant + "_window") if windowed else None
+        entry = entry or table.get(prefix + dominant)
         if entry is not None and entry.get("sources") == kernel_sources_fingerprint():
             traffic, traffic_note = entry["bytes"], entry.get("kernel")
         elif entry is not None:
