@@ -137,9 +137,13 @@ def main():
     setup_s = time.time() - t0
 
     stream = torch.cuda.current_stream().cuda_stream
+    hub = csr.plan if isinstance(csr.plan, rode_sddmm_hip.HubPlan) else None
+    hub_ws = hub.workspace(k, 4) if hub is not None else None
+
     def spmm_fn(*a, flags=0):  # the whole decomposition is passed, and the library is told so
         return lib.rode_hip_spmm_planned(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS | flags, *a[:-2],
-                                         *plan_args, *a[-2:])
+                                         *plan_args, hub_ws.data_ptr() if hub is not None else None,
+                                         hub_ws.numel() if hub is not None else 0, *a[-2:])
 
     def sddmm_fn(*a):
         return lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[args.dtype], *a[:-2], *plan_args, *a[-2:])

@@ -181,18 +181,53 @@ int rode_hip_window_rows(int m2, const int* d_row_indices_residue, const int* d_
                          const int* d_column_indices, const void* d_plan, void* d_rows, size_t rows_bytes, void* stream);
 
 /*
- * rode_hip_spmm_ex with a locality plan.  d_plan / d_plan_rows: both parts of a plan made
- * from these lists, or NULL (then exactly rode_hip_spmm_ex).  h_plan_counts: NULL, or the
- * HOST int[4] header that rode_hip_window_plan returned; with it, kernels that would find
- * no chunk to work on are not launched at all.  fp64 operands, and dense rows of at most
- * 128 bytes, ignore the plan.  Same results as without a plan, up to the order of the fp32
- * additions inside a row.
+ * Hub plan (no counterpart in the reference either).  For matrices with a few very long
+ * rows (hubs of a power-law graph) whose dense operand is far larger than the caches: the
+ * rows of at least min_len aligned nonzero slots are cut into pieces by column slab
+ * (RODE_HIP_HUB_SLAB_ROWS dense rows) and worked on slab after slab - a few neighbouring
+ * slabs, about 4 MB of the dense operand, at a time - by kernels of their own, so that the
+ * hub rows' nonzeros of those slabs meet in one L2 and a dense row is fetched from memory
+ * once for all of them.  The other kernels leave those rows out.  Results are
+ * the same up to the order of the fp32 additions inside a hub row.
+ *   dense_rows   rows of the dense operand (columns of the sparse matrix)
+ *   min_len      >= RODE_HIP_HUB_MIN_LEN; a piece should hold dozens of nonzeros: 4096 and
+ *                dense_rows / 512 are sensible lower bounds (measured on a 2 M x 2 M
+ *                power-law matrix: 4096 is best, 2048 and 8192 gain less, 1024 loses)
+ *   d_plan       rode_hip_hub_plan_bytes(M, dense_rows, nnz, min_len) bytes, 16-byte aligned, out
+ *   h_counts     HOST int[8], out (the call waits for its two kernels): [0] hub rows,
+ *                [1] slabs, [2] min_len, [3] 1 if the plan is usable - every hub row's column
+ *                indices ascend and lie inside the operand - else 0, [4] room for hub rows;
+ *                the *_planned entry points need it and ignore a plan with [3] == 0 or [0] == 0
+ * A hub plan belongs to the pattern it was made from, and excludes a locality plan: the
+ * *_planned entry points refuse to take both.
+ */
+#define RODE_HIP_HUB_SLAB_ROWS 2048
+#define RODE_HIP_HUB_MIN_LEN 64
+size_t rode_hip_hub_plan_bytes(int M, int dense_rows, int nnz, int min_len);
+size_t rode_hip_hub_workspace_bytes(const int* h_hub_counts, int n, int elem_bytes);
+int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_row_offsets,
+                      const int* d_column_indices, void* d_plan, size_t plan_bytes, int* h_counts, void* stream);
+
+/*
+ * rode_hip_spmm_ex with a plan.  d_plan / d_plan_rows: both parts of a locality plan made
+ * from these lists, or NULL.  h_plan_counts: NULL, or the HOST int[4] header that
+ * rode_hip_window_plan returned; with it, kernels that would find no chunk to work on are
+ * not launched at all.  fp64 operands, and dense rows of at most 128 bytes, ignore the
+ * locality plan.  d_hub_plan / h_hub_counts: a hub plan of this matrix and its header, or
+ * NULL; it needs RODE_SPMM_WHOLE_LISTS (the hub kernels replace work items of both lists)
+ * and no RODE_SPMM_ONLY_* flag.  d_hub_workspace: rode_hip_hub_workspace_bytes(h_hub_counts,
+ * n, 4 or 8) bytes of scratch, 16-byte aligned, that the hub kernels of this call may write
+ * and read (one partial row of C per hub row and slab, summed by a second kernel), or NULL:
+ * the pieces are then added to C atomically, which is slower for wide rows.  With every
+ * plan pointer NULL: exactly rode_hip_spmm_ex.
+ * Same results as without a plan, up to the order of the fp32 additions inside a row.
  */
 int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                           const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                           const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
-                          const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, void* stream1,
-                          void* stream2);
+                          const void* d_plan, const void* d_plan_rows, const int* h_plan_counts,
+                          const void* d_hub_plan, const int* h_hub_counts, void* d_hub_workspace,
+                          size_t hub_workspace_bytes, void* stream1, void* stream2);
 
 /*
  * Prepares an uninitialised C[M x n] for one of the SpMM calls: zeroes exactly the rows
@@ -242,16 +277,19 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
                        const void* d_rhs_half, float* d_out, void* stream1, void* stream2);
 
 /*
- * SDDMM with a locality plan: dtype RODE_DENSE_F32 or RODE_DENSE_F16 selects the element
- * type of lhs / rhs; d_plan / d_plan_rows / h_plan_counts as for rode_hip_spmm_planned (NULL:
- * exactly the typed functions above).  Same results up to the order of the fp32 additions of a dot
- * product.  No counterpart in the reference.
+ * SDDMM with a plan: dtype RODE_DENSE_F32 or RODE_DENSE_F16 selects the element type of
+ * lhs / rhs; d_plan / d_plan_rows / h_plan_counts and d_hub_plan / h_hub_counts as for
+ * rode_hip_spmm_planned (all NULL: exactly the typed functions above).  With a hub plan the
+ * lists must be the complete decomposition (the hub kernels replace work items of both).
+ * Same results up to the order of the fp32 additions of a dot product.  No counterpart in
+ * the reference.
  */
 int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d_row_indices_block,
                            const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                            const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
                            const void* d_rhs_matrix, float* d_out, const void* d_plan, const void* d_plan_rows,
-                           const int* h_plan_counts, void* stream1, void* stream2);
+                           const int* h_plan_counts, const void* d_hub_plan, const int* h_hub_counts, void* stream1,
+                           void* stream2);
 
 /*
  * Row softmax over the values of a CSR pattern, out[idx] = softmax over the row of

@@ -28,11 +28,14 @@ SIGNATURES = {
     "rode_hip_window_plan": (c_int, [c_int] * 2 + [c_void_p] * 4 + [c_size_t, c_void_p, c_void_p]),
     "rode_hip_window_rows_bytes": (c_size_t, [c_int]),
     "rode_hip_window_rows": (c_int, [c_int] + [c_void_p] * 5 + [c_size_t, c_void_p]),
-    "rode_hip_spmm_planned": (c_int, [c_int] * 6 + [c_void_p] * 13),
+    "rode_hip_hub_plan_bytes": (c_size_t, [c_int] * 4),
+    "rode_hip_hub_plan": (c_int, [c_int] * 4 + [c_void_p] * 3 + [c_size_t, c_void_p, c_void_p]),
+    "rode_hip_hub_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
+    "rode_hip_spmm_planned": (c_int, [c_int] * 6 + [c_void_p] * 14 + [c_size_t] + [c_void_p] * 2),
     "rode_hip_spmm_clear_rows": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "rode_hip_sddmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 11),
     "rode_hip_sddmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 11),
-    "rode_hip_sddmm_planned": (c_int, [c_int] * 5 + [c_void_p] * 14),
+    "rode_hip_sddmm_planned": (c_int, [c_int] * 5 + [c_void_p] * 16),
     "rode_hip_csr_softmax_f32": (c_int, [c_int, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p]),
     "rode_hip_csr_softmax_backward_f32": (c_int, [c_int] + [c_void_p] * 4 + [ctypes.c_float, c_void_p]),
     "rode_hip_csr_transpose_workspace_bytes": (c_size_t, [c_int]),

@@ -128,10 +128,49 @@ int rode_hip_window_rows(int m2, const int* d_row_indices_residue, const int* d_
                                          static_cast<const int*>(d_plan), d_rows, as_stream(stream));
 }
 
-namespace {
-// The caller's plan as the launchers take it; false if it cannot belong to these lists.
-bool plan_ref(const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, int m2, rode::PlanRef& plan)
+size_t rode_hip_hub_plan_bytes(int M, int dense_rows, int nnz, int min_len)
 {
+    if (M < 0 || dense_rows < 0 || nnz < 0 || min_len < RODE_HIP_HUB_MIN_LEN) return 0;
+    return rode::hub_plan_ints(M, dense_rows, nnz, min_len) * sizeof(int);
+}
+
+int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_row_offsets,
+                      const int* d_column_indices, void* d_plan, size_t plan_bytes, int* h_counts, void* stream)
+{
+    if (M < 0 || dense_rows < 0 || nnz < 0 || min_len < RODE_HIP_HUB_MIN_LEN || !d_plan || !aligned16(d_plan) || !h_counts)
+        return hipErrorInvalidValue;
+    if (plan_bytes < rode_hip_hub_plan_bytes(M, dense_rows, nnz, min_len)) return hipErrorInvalidValue;
+    if (M > 0 && (!d_row_offsets || (nnz > 0 && !d_column_indices))) return hipErrorInvalidValue;
+    hipError_t e = rode::hub_plan_launch(M, dense_rows, nnz, min_len, d_row_offsets, d_column_indices,
+                                         static_cast<int*>(d_plan), as_stream(stream));
+    if (e == hipSuccess) e = hipMemcpyAsync(h_counts, d_plan, 8 * sizeof(int), hipMemcpyDeviceToHost, as_stream(stream));
+    if (e == hipSuccess) e = hipStreamSynchronize(as_stream(stream));
+    return e;
+}
+
+size_t rode_hip_hub_workspace_bytes(const int* h_hub_counts, int n, int elem_bytes)
+{
+    if (!h_hub_counts || n <= 0 || (elem_bytes != 4 && elem_bytes != 8) || h_hub_counts[0] <= 0 || h_hub_counts[1] <= 0)
+        return 0;
+    const int merge = rode::hub_merge(n * elem_bytes / 4);
+    return (size_t)h_hub_counts[0] * rode::hub_groups(h_hub_counts[1], merge) * n * elem_bytes;
+}
+
+namespace {
+// The caller's plans as the launchers take them; false if they cannot belong to these lists.
+bool plan_ref(const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, const void* d_hub_plan,
+              const int* h_hub_counts, int m2, rode::PlanRef& plan)
+{
+    if (d_hub_plan) {
+        // a hub plan needs its header on the host, and excludes a locality plan (the window
+        // kernels do not know which rows the hub kernels have taken)
+        if (!h_hub_counts || !aligned16(d_hub_plan) || (d_plan && d_plan_rows)) return false;
+        if (h_hub_counts[0] < 0 || h_hub_counts[0] > h_hub_counts[4] || h_hub_counts[1] < 0 ||
+            h_hub_counts[2] < RODE_HIP_HUB_MIN_LEN)
+            return false;
+        plan.hub = static_cast<const int*>(d_hub_plan);
+        plan.hub_counts = h_hub_counts;
+    }
     if (!d_plan || !d_plan_rows) return true; // no plan, or one without rows: the standard kernels do everything
     if (!aligned16(d_plan) || !aligned16(d_plan_rows)) return false;
     if (h_plan_counts && h_plan_counts[0] != rode::plan_residue_chunks(m2)) return false;
@@ -148,14 +187,15 @@ int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const v
                      void* stream1, void* stream2)
 {
     return rode_hip_spmm_planned(dtype, flags, m1, m2, k, n, d_values, d_column_indices, d_row_offsets, d_row_indices1,
-                                 d_row_indices2, d_row_seg_st_offsets, d_B, d_C, nullptr, nullptr, nullptr, stream1,
-                                 stream2);
+                                 d_row_indices2, d_row_seg_st_offsets, d_B, d_C, nullptr, nullptr, nullptr, nullptr, nullptr,
+                                 nullptr, 0, stream1, stream2);
 }
 
 int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                           const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                           const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
-                          const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, void* stream1,
+                          const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, const void* d_hub_plan,
+                          const int* h_hub_counts, void* d_hub_workspace, size_t hub_workspace_bytes, void* stream1,
                           void* stream2)
 {
     (void)k;
@@ -168,7 +208,13 @@ int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, co
     if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
     hipStream_t s1 = as_stream(stream1), s2 = as_stream(stream2);
     rode::PlanRef plan;
-    if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, m2, plan)) return hipErrorInvalidValue;
+    if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, d_hub_plan, h_hub_counts, m2, plan)) return hipErrorInvalidValue;
+    // the hub kernels replace work items of both lists: only with the complete decomposition
+    if (plan.hub && !(flags & RODE_SPMM_WHOLE_LISTS)) return hipErrorInvalidValue;
+    if (plan.hub && d_hub_workspace && aligned16(d_hub_workspace)) {
+        plan.hub_workspace = d_hub_workspace;
+        plan.hub_workspace_bytes = hub_workspace_bytes;
+    }
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
@@ -224,14 +270,15 @@ int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d
                            const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                            const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
                            const void* d_rhs_matrix, float* d_out, const void* d_plan, const void* d_plan_rows,
-                           const int* h_plan_counts, void* stream1, void* stream2)
+                           const int* h_plan_counts, const void* d_hub_plan, const int* h_hub_counts, void* stream1,
+                           void* stream2)
 {
     (void)n;
     if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
     if (m1 == 0 && m2 == 0) return hipSuccess;
     if (!aligned16(d_lhs_matrix) || !aligned16(d_rhs_matrix)) return hipErrorInvalidValue;
     rode::PlanRef plan;
-    if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, m2, plan)) return hipErrorInvalidValue;
+    if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, d_hub_plan, h_hub_counts, m2, plan)) return hipErrorInvalidValue;
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::sddmm_launch<float>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
@@ -255,7 +302,7 @@ int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_bl
 {
     return rode_hip_sddmm_planned(RODE_DENSE_F32, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
                                   d_row_offsets, d_column_indices, d_values, d_lhs_matrix, d_rhs_matrix, d_out, nullptr,
-                                  nullptr, nullptr, stream1, stream2);
+                                  nullptr, nullptr, nullptr, nullptr, stream1, stream2);
 }
 
 int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,
@@ -265,7 +312,7 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
 {
     return rode_hip_sddmm_planned(RODE_DENSE_F16, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
                                   d_row_offsets, d_column_indices, d_values, d_lhs_half, d_rhs_half, d_out, nullptr,
-                                  nullptr, nullptr, stream1, stream2);
+                                  nullptr, nullptr, nullptr, nullptr, stream1, stream2);
 }
 
 int rode_hip_csr_softmax_f32(int M, const int* d_row_offsets, const float* d_in, float* d_out, float scale,

@@ -31,7 +31,16 @@ struct PlanRef {
     const int* dev = nullptr;         // descriptors
     const void* rows = nullptr;       // planned rows of the chunks with a window
     const int* host_counts = nullptr;
+    // A hub plan (rode_hub.hip) and the host copy of its eight header ints (required with it).
+    const int* hub = nullptr;
+    const int* hub_counts = nullptr;
+    // SpMM only: room for one partial row of C per (slab, hub row), or null (atomics instead).
+    void* hub_workspace = nullptr;
+    size_t hub_workspace_bytes = 0;
 };
+
+hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, const int* col, int* plan,
+                           hipStream_t stream);
 
 size_t window_plan_ints(int m2);
 size_t window_plan_rows_bytes(int m2);

@@ -49,12 +49,15 @@ constexpr int kSpmmMergeSlots = 512;
 
 // SDDMM: merging needs no promise from the caller (an output computed twice at a slice
 // boundary is harmless).
-__device__ __forceinline__ bool sddmm_block_item(int seg, int m1, int lane, const int* __restrict__ block_rows,
-                                                 const int* __restrict__ st_off, const int* __restrict__ row_ptr,
-                                                 BlockItem& it)
+// hub_min_len > 0: rows of that aligned length or more belong to the hub kernels.
+__device__ __forceinline__ bool sddmm_block_item(int seg, int m1, int hub_min_len, int lane,
+                                                 const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                                                 const int* __restrict__ row_ptr, BlockItem& it)
 {
     const int row = block_rows[seg];
-    return merged_leader(kSddmmMergeSlots, seg, m1, lane, row, row_ptr[row], row_ptr[row + 1], block_rows, st_off, it);
+    const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
+    if (hub_min_len > 0 && row_end - row_start + (row_start & (kVecLen - 1)) >= hub_min_len) return false;
+    return merged_leader(kSddmmMergeSlots, seg, m1, lane, row, row_start, row_end, block_rows, st_off, it);
 }
 
 // SpMM.  owned_slots > 0 means that the caller promised complete lists: a row of at
@@ -66,12 +69,13 @@ __device__ __forceinline__ bool sddmm_block_item(int seg, int m1, int lane, cons
 // owned_slots == 0: every segment on its own, rounded to whole 32-slot units as in
 // RoDeSpmm.cu:210-234 (small launches: they need the waves more than they mind the
 // atomics).
-__device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots, int lane,
+__device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots, int hub_min_len, int lane,
                                                 const int* __restrict__ block_rows, const int* __restrict__ st_off,
                                                 const int* __restrict__ row_ptr, BlockItem& it)
 {
     const int row = block_rows[seg];
     const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
+    if (hub_min_len > 0 && row_end - row_start + (row_start & (kVecLen - 1)) >= hub_min_len) return false;
     if (row_end - row_start + (row_start & (kVecLen - 1)) <= owned_slots) {
         if (seg > 0 && block_rows[seg - 1] == row) return false;
         it.row = row;
@@ -94,15 +98,17 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
 // The row of segment `seg` if spmm_block_item() gives it a work item, else -1 (a follower,
 // or past the list).  The same rules, without the extent of the item: what the waves of a
 // workgroup need to know about each other.
-__device__ __forceinline__ int spmm_block_leader_row(int seg, int m1, int owned_slots,
+__device__ __forceinline__ int spmm_block_leader_row(int seg, int m1, int owned_slots, int hub_min_len,
                                                      const int* __restrict__ block_rows, const int* __restrict__ st_off,
                                                      const int* __restrict__ row_ptr)
 {
     if (seg >= m1) return -1;
     const int row = block_rows[seg];
-    if (seg == 0 || block_rows[seg - 1] != row || owned_slots == 0) return row;
+    if (hub_min_len <= 0 && (seg == 0 || block_rows[seg - 1] != row || owned_slots == 0)) return row;
     const int row_start = row_ptr[row];
     const int row_base = row_start - (row_start & (kVecLen - 1));
+    if (hub_min_len > 0 && row_ptr[row + 1] - row_base >= hub_min_len) return -1; // the hub kernel's
+    if (seg == 0 || block_rows[seg - 1] != row || owned_slots == 0) return row;
     if (row_ptr[row + 1] - row_base <= owned_slots) return -1; // summed whole by the wave of its first segment
     return (st_off[seg] - row_base) / kSpmmMergeSlots == (st_off[seg - 1] - row_base) / kSpmmMergeSlots ? -1 : row;
 }
@@ -185,6 +191,64 @@ __device__ __forceinline__ WindowDesc plan_residue_desc(const int* __restrict__ 
 {
     const int4 v = *reinterpret_cast<const int4*>(plan + kPlanHeaderInts + kPlanDescInts * chunk);
     return WindowDesc{v.x, v.y, v.z, v.w};
+}
+
+// ---- hub plan -------------------------------------------------------------------
+// Rows with very many nonzeros (hubs of a power-law graph) reference dense rows all over
+// the operand, and so does every other hub: the same dense rows, at other times, long
+// evicted from L2.  A hub plan cuts every hub row into pieces by column slab (a slab is
+// kHubSlabRows consecutive dense rows) and the hub kernels take the pieces slab by slab,
+// a few neighbouring slabs at a time (hub_merge: about 4 MB of the dense operand, the size
+// of an XCD's L2 - measured best on the power-law benchmark against half, twice and four
+// times that; smaller pieces cost more than they save): all hub rows' nonzeros of those
+// slabs at the same time on one XCD, so that a dense row is fetched from memory once and
+// then found in L2 by the other hubs.
+// Needs rows whose column indices ascend (the plan checks).  The standard kernels skip
+// the rows of a usable plan (by their length), so every nonzero is still processed once.
+// Layout, ints: header [0] hub rows  [1] slabs  [2] shortest hub row (aligned length)
+// [3] usable (every hub row's columns ascend)  [4] room for hub rows  [5..7] zero;
+// then the hub rows, ascending (room for [4] of them); then per hub row slabs + 1 piece
+// starts (indices into column_indices / values; the last one is the row's end).
+constexpr int kHubSlabRows = 2048;
+constexpr int kHubHeaderInts = 8;
+
+__host__ __device__ inline int hub_slabs(int dense_rows) { return (dense_rows + kHubSlabRows - 1) / kHubSlabRows; }
+__host__ __device__ inline int hub_room(int nnz, int min_len) { return min_len > 0 ? nnz / min_len + 1 : 0; }
+// (after the piece table: one int per 2048 rows of the matrix, scratch of the selection)
+constexpr int kHubSelectBlockRows = 2048;
+__host__ __device__ inline size_t hub_table_ints(int dense_rows, int nnz, int min_len)
+{
+    const size_t room = hub_room(nnz, min_len);
+    return kHubHeaderInts + room + room * (hub_slabs(dense_rows) + 1);
+}
+__host__ __device__ inline size_t hub_plan_ints(int M, int dense_rows, int nnz, int min_len)
+{
+    return hub_table_ints(dense_rows, nnz, min_len) + (M + kHubSelectBlockRows - 1) / kHubSelectBlockRows + 1;
+}
+
+// Slabs taken together by one work item of the hub kernels, for dense rows of `width`
+// 4-byte elements (16-bit operands count as 4 bytes too: the pieces matter more than the bytes).
+__host__ __device__ inline int hub_merge(int width)
+{
+    const int g = (4 << 20) / kHubSlabRows / (width > 0 ? width * 4 : 4);
+    return g < 1 ? 1 : (g > 64 ? 64 : g);
+}
+__host__ __device__ inline int hub_groups(int slabs, int merge) { return (slabs + merge - 1) / merge; }
+
+struct HubPlan {
+    int n_hub, slabs, min_len;
+    const int* rows;   // [n_hub]
+    const int* pieces; // [n_hub][slabs + 1]
+};
+__device__ __forceinline__ HubPlan hub_plan_view(const int* __restrict__ plan)
+{
+    HubPlan v;
+    v.n_hub = plan[0];
+    v.slabs = plan[1];
+    v.min_len = plan[2];
+    v.rows = plan + kHubHeaderInts;
+    v.pieces = plan + kHubHeaderInts + plan[4];
+    return v;
 }
 
 } // namespace rode

@@ -26,37 +26,19 @@ namespace rode {
 
 namespace {
 
-// One wave per block segment.  Segment s covers the aligned slots
-// [base, base + cnt) with base = st_off[s] & ~3 and cnt = floor((len + mask) / 32) * 32
-// (RoDeSddmm.cu:35-54); the first `mask` slots belong to the previous row and are
-// computed but never stored (RoDeSddmm.cu:56-58, 197).
-// (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
+// out[idx] = values[idx] * <lhs[row, :], rhs[col(idx), :]> for the aligned slots
+// [base, base + cnt) of one row, 64 slots per step; the first `mask` slots (the previous
+// row's) are computed but not stored.
 template <typename T, int KT, int NS, bool EDGE>
-__device__ __forceinline__ void
-sddmm_block_body(int bid, int nblocks, int m1, int k, const int* __restrict__ block_rows, const int* __restrict__ st_off,
-                 const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
-                 const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
+__device__ __forceinline__ void sddmm_row_slots(int row, int base, int mask, int cnt, int k, int lane, int* lds_cols,
+                                                const int* __restrict__ col, const float* __restrict__ val,
+                                                const T* __restrict__ lhs, const T* __restrict__ rhs,
+                                                float* __restrict__ out)
 {
     using S = SddmmShape<T, KT>;
-    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int seg = xcd_logical_block(bid, nblocks) * kWavesPerWg + wave;
-    if (seg >= m1) return;
-
-    // Consecutive segments of one row whose starts fall into the same window of
-    // kSddmmMergeSlots slots are handled by the wave of the first of them, so a decomposition
-    // with short segments (32 in the reference's K=128 parameter set) still fills whole
-    // 64-slot steps and loads the lhs row once.  Longer segments are unaffected.  (Outputs
-    // are pure functions of the inputs, so this is safe even when a caller passes a slice of
-    // the lists: the worst case is an output computed twice.)
-    BlockItem it;
-    if (!sddmm_block_item(seg, m1, lane, block_rows, st_off, row_ptr, it)) return;
-    const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
-
     float a[NS][S::kVec];
     load_lhs_slice<T, KT, NS, EDGE>(lhs, row, k, lane, a);
     const T* rhs_lane = rhs + (lane % S::kLpr) * S::kVec;
-    int* lds_cols = lds + wave * kWave;
 
     for (int off = 0; off < cnt; off += kWave) {
         if (off + (lane & 32) < cnt) { // the upper half sits out a trailing 32-slot step
@@ -75,13 +57,43 @@ sddmm_block_body(int bid, int nblocks, int m1, int k, const int* __restrict__ bl
     }
 }
 
+// One wave per block segment.  Segment s covers the aligned slots
+// [base, base + cnt) with base = st_off[s] & ~3 and cnt = floor((len + mask) / 32) * 32
+// (RoDeSddmm.cu:35-54); the first `mask` slots belong to the previous row and are
+// computed but never stored (RoDeSddmm.cu:56-58, 197).
+// (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
+template <typename T, int KT, int NS, bool EDGE>
+__device__ __forceinline__ void
+sddmm_block_body(int bid, int nblocks, int m1, int k, int hub_min_len, const int* __restrict__ block_rows,
+                 const int* __restrict__ st_off,
+                 const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
+                 const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
+{
+    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int seg = xcd_logical_block(bid, nblocks) * kWavesPerWg + wave;
+    if (seg >= m1) return;
+
+    // Consecutive segments of one row whose starts fall into the same window of
+    // kSddmmMergeSlots slots are handled by the wave of the first of them, so a decomposition
+    // with short segments (32 in the reference's K=128 parameter set) still fills whole
+    // 64-slot steps and loads the lhs row once.  Longer segments are unaffected.  (Outputs
+    // are pure functions of the inputs, so this is safe even when a caller passes a slice of
+    // the lists: the worst case is an output computed twice.)
+    BlockItem it;
+    if (!sddmm_block_item(seg, m1, hub_min_len, lane, block_rows, st_off, row_ptr, it)) return;
+    const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
+
+    sddmm_row_slots<T, KT, NS, EDGE>(row, base, mask, cnt, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
+}
+
 // One group of LPR lanes per residue row.  Tail selection follows RoDeSddmm.cu:237-243:
 // with N = len + (s & 3), rows with N >= 32 keep only their last N % 32 slots
 // starting at (s & ~3) + floor(N / 32) * 32; shorter rows are taken whole.
 // Lane ls of the group owns the slots ls, ls + LPR, ... (value, result, store).
 template <typename T, int KT, int NS, bool EDGE>
 __device__ __forceinline__ void
-sddmm_residue_body(int bid, int nblocks, int m2, int k, const int* __restrict__ residue_rows,
+sddmm_residue_body(int bid, int nblocks, int m2, int k, int hub_min_len, const int* __restrict__ residue_rows,
                    const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                    const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out,
                    const int* __restrict__ plan)
@@ -102,6 +114,7 @@ sddmm_residue_body(int bid, int nblocks, int m2, int k, const int* __restrict__ 
     const ResidueItem it = residue_item(row, row_ptr);
     const int first = it.first, cnt = it.cnt;
     if (cnt <= 0) return; // an empty, unaligned row is listed as a residue but owns no slot
+    if (hub_min_len > 0 && it.aligned >= hub_min_len) return; // the hub kernel has the whole row
 
     int* my_cols = lds + (wave * RPW + group) * kBlockItems;
     float v[OWN];
@@ -152,36 +165,59 @@ sddmm_residue_body(int bid, int nblocks, int m2, int k, const int* __restrict__ 
 
 template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_block_kernel(int m1, int k, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+sddmm_block_kernel(int m1, int k, int hub_min_len, const int* __restrict__ block_rows, const int* __restrict__ st_off,
                    const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                    const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
 {
-    sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+    sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m1, k, hub_min_len, block_rows, st_off, row_ptr, col, val, lhs,
+                                      rhs, out);
 }
 
 template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_residue_kernel(int m2, int k, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
+sddmm_residue_kernel(int m2, int k, int hub_min_len, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
                      const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
                      const T* __restrict__ rhs, float* __restrict__ out, const int* __restrict__ plan)
 {
-    sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out, plan);
+    sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m2, k, hub_min_len, residue_rows, row_ptr, col, val, lhs, rhs,
+                                        out, plan);
 }
 
 // Both lists in one launch: the first g1 workgroups work on block segments, the others on
 // residue rows.  For matrices so small that a launch costs as much as its kernel.
 template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_pair_kernel(int g1, int m1, int m2, int k, const int* __restrict__ block_rows, const int* __restrict__ residue_rows,
+sddmm_pair_kernel(int g1, int m1, int m2, int k, int hub_min_len, const int* __restrict__ block_rows,
+                  const int* __restrict__ residue_rows,
                   const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const float* __restrict__ val, const T* __restrict__ lhs, const T* __restrict__ rhs,
                   float* __restrict__ out, const int* __restrict__ plan)
 {
     if ((int)blockIdx.x < g1)
-        sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, g1, m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+        sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, g1, m1, k, hub_min_len, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
     else
-        sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, k, residue_rows, row_ptr, col, val, lhs,
+        sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, k, hub_min_len, residue_rows, row_ptr, col, val, lhs,
                                             rhs, out, plan);
+}
+
+// The rows of a hub plan, cut into pieces by column slab (rode_items.hpp): one wave per
+// piece, slab after slab, so that the hub rows' nonzeros of one slab of rhs are worked on
+// at the same time on one XCD and find its rows in that XCD's L2.
+template <typename T, int KT, int NS, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+sddmm_hub_kernel(int k, int merge, const int* __restrict__ hub, const int* __restrict__ col, const float* __restrict__ val,
+                 const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
+{
+    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const HubPlan hp = hub_plan_view(hub);
+    const long long item = (long long)xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
+    if (item >= (long long)hp.n_hub * hub_groups(hp.slabs, merge)) return;
+    const int slab = (int)(item / hp.n_hub) * merge, h = (int)(item % hp.n_hub);
+    const int* piece = hp.pieces + (size_t)h * (hp.slabs + 1);
+    const int base = piece[slab], cnt = piece[min(slab + merge, hp.slabs)] - base;
+    if (cnt <= 0) return;
+    sddmm_row_slots<T, KT, NS, EDGE>(hp.rows[h], base, 0, cnt, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
 }
 
 // Up to this many workgroups, and when both kernels go to the same stream, the two lists
@@ -212,20 +248,29 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
         standard_residue = plan.host_counts[1] < plan.host_counts[0];
         window_residue = plan.host_counts[1] > 0;
     }
+    const bool hubs = plan.hub != nullptr && plan.hub_counts != nullptr && plan.hub_counts[3] != 0 && plan.hub_counts[0] > 0;
+    const int hub_min_len = hubs ? plan.hub_counts[2] : 0;
     if (m1 > 0 && m2 > 0 && standard_residue && s1 == s2 && g1 + g2 <= kPairMaxWorkgroups) {
         sddmm_pair_kernel<T, KT, NS, EDGE><<<g1 + g2, kWgThreads, 0, s1>>>(
-            g1, m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);
+            g1, m1, m2, k, hub_min_len, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);
     } else {
         if (m1 > 0) {
             sddmm_block_kernel<T, KT, NS, EDGE><<<g1, kWgThreads, 0, s1>>>(
-                m1, k, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+                m1, k, hub_min_len, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
         }
         if (m2 > 0 && standard_residue) {
             sddmm_residue_kernel<T, KT, NS, EDGE><<<g2, kWgThreads, 0, s2>>>(
-                m2, k, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev);
+                m2, k, hub_min_len, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev);
         }
     }
     hipError_t e = hipGetLastError();
+    if (e == hipSuccess && hubs) {
+        const int merge = hub_merge(k);
+        const int gh = grid_for_waves((long long)plan.hub_counts[0] * hub_groups(plan.hub_counts[1], merge));
+        if (gh < 0) return hipErrorInvalidConfiguration;
+        sddmm_hub_kernel<T, KT, NS, EDGE><<<gh, kWgThreads, 0, s1>>>(k, merge, plan.hub, col, val, lhs, rhs, out);
+        e = hipGetLastError();
+    }
     if (e == hipSuccess && m2 > 0 && window_residue)
         e = sddmm_window_launch<T>(m2, k, col, val, lhs, rhs, out, plan.dev, plan.rows, s2);
     return e;

@@ -64,52 +64,20 @@ __device__ __forceinline__ void store_row(double* dst, const double (&acc)[VEC])
     for (int x = 0; x < VEC; x += 2) *reinterpret_cast<double2*>(dst + x) = make_double2(acc[x], acc[x + 1]);
 }
 
-// One wave per block segment (see sddmm_block_kernel for the slot arithmetic,
-// identical at RoDeSpmm.cu:210-234).
-// (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
-template <typename T, int TN, bool EDGE>
-__device__ __forceinline__ void
-spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, const int* __restrict__ block_rows,
-                const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
-                const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
-                typename DenseVec<T>::Acc* __restrict__ C)
+// Sum over the aligned slots [base, base + cnt) of values * B rows, for this lane's columns
+// of the tile; the first `mask` slots (the previous row's) and the slots past cnt in the
+// last quad are neutralised.  Every lane of the wave returns the wave's total.
+template <typename T, int TN>
+__device__ __forceinline__ void spmm_sum_slots(int base, int mask, int cnt, int lane, int* my_c,
+                                               typename DenseVec<T>::Acc* my_v, const T* b_lane, int n,
+                                               const int* __restrict__ col,
+                                               const typename DenseVec<T>::Acc* __restrict__ val,
+                                               typename DenseVec<T>::Acc (&total)[SpmmShape<T, TN>::kVec])
 {
     using S = SpmmShape<T, TN>;
     using A = typename S::Acc;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
-    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
-    __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int seg0 = xcd_logical_block(bid, nblocks) * kWavesPerWg;
-    const int seg = seg0 + wave;
-    BlockItem it{-1, 0, 0, 0};
-    const bool active = seg < m1 && spmm_block_item(seg, m1, owned_slots, lane, block_rows, st_off, row_ptr, it);
-    // A wave without a work item leaves at once (with the reference's 32-slot segments that
-    // is most waves); the barrier below then counts only the waves that are still running
-    // (S_BARRIER waits on the surviving waves of a workgroup).
-    if (!active) return;
-    // Do two work items of this workgroup add to the same row (neighbouring segments of a
-    // long row that are not merged into one leader)?  Every wave finds the same answer.  If
-    // so, the waves add their sums up in LDS and the row of C gets one update per run of
-    // such work items instead of one each.
-    int item_row[kWavesPerWg]; // the row of each wave's work item, -1: that wave has none (and has left)
-    bool shared_row = false;
-#pragma unroll
-    for (int i = 0; i < kWavesPerWg; ++i) {
-        item_row[i] = spmm_block_leader_row(seg0 + i, m1, owned_slots, block_rows, st_off, row_ptr);
-        if (i > 0) shared_row = shared_row || (item_row[i] >= 0 && item_row[i] == item_row[i - 1]);
-    }
-    const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
-
-    const int ls = lane % LPR, group = lane / LPR;
-    const int tile = blockIdx.y * TN;
-    // EDGE: n is not a multiple of TN; lanes past the last column re-read the tile's
-    // first columns (a valid address) and never write
-    const bool col_ok = !EDGE || tile + ls * VEC < n;
-    const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
-    int* my_c = lds_c + wave * kWave;
-    A* my_v = lds_v + wave * kWave;
-
+    const int group = lane / LPR;
     A acc[VEC];
 #pragma unroll
     for (int x = 0; x < VEC; ++x) acc[x] = A(0);
@@ -135,12 +103,60 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, const int*
             spmm_gather<T, TN, 16 / G, false>(b_lane, (size_t)n, acc, my_c, my_v, group, G, (live + 3) / 4);
         wave_lds_sync();
     }
+#pragma unroll
+    for (int x = 0; x < VEC; ++x) total[x] = butterfly_sum<LPR, kWave>(acc[x]);
+}
+
+// One wave per block segment (see sddmm_block_kernel for the slot arithmetic,
+// identical at RoDeSpmm.cu:210-234).
+// (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
+template <typename T, int TN, bool EDGE>
+__device__ __forceinline__ void
+spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int hub_min_len, const int* __restrict__ block_rows,
+                const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
+                const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
+                typename DenseVec<T>::Acc* __restrict__ C)
+{
+    using S = SpmmShape<T, TN>;
+    using A = typename S::Acc;
+    constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
+    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
+    __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int seg0 = xcd_logical_block(bid, nblocks) * kWavesPerWg;
+    const int seg = seg0 + wave;
+    BlockItem it{-1, 0, 0, 0};
+    const bool active = seg < m1 && spmm_block_item(seg, m1, owned_slots, hub_min_len, lane, block_rows, st_off, row_ptr, it);
+    // A wave without a work item leaves at once (with the reference's 32-slot segments that
+    // is most waves); the barrier below then counts only the waves that are still running
+    // (S_BARRIER waits on the surviving waves of a workgroup).
+    if (!active) return;
+    // Do two work items of this workgroup add to the same row (neighbouring segments of a
+    // long row that are not merged into one leader)?  Every wave finds the same answer.  If
+    // so, the waves add their sums up in LDS and the row of C gets one update per run of
+    // such work items instead of one each.
+    int item_row[kWavesPerWg]; // the row of each wave's work item, -1: that wave has none (and has left)
+    bool shared_row = false;
+#pragma unroll
+    for (int i = 0; i < kWavesPerWg; ++i) {
+        item_row[i] = spmm_block_leader_row(seg0 + i, m1, owned_slots, hub_min_len, block_rows, st_off, row_ptr);
+        if (i > 0) shared_row = shared_row || (item_row[i] >= 0 && item_row[i] == item_row[i - 1]);
+    }
+    const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
+
+    const int ls = lane % LPR, group = lane / LPR;
+    const int tile = blockIdx.y * TN;
+    // EDGE: n is not a multiple of TN; lanes past the last column re-read the tile's
+    // first columns (a valid address) and never write
+    const bool col_ok = !EDGE || tile + ls * VEC < n;
+    const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
+    int* my_c = lds_c + wave * kWave;
+    A* my_v = lds_v + wave * kWave;
 
     // combine the lane groups, then spread the atomics over them
     constexpr int EPG = VEC / G > 0 ? VEC / G : 1; // elements each group adds
     A total[VEC];
-#pragma unroll
-    for (int x = 0; x < VEC; ++x) total[x] = butterfly_sum<LPR, kWave>(acc[x]);
+    spmm_sum_slots<T, TN>(base, mask, cnt, lane, my_c, my_v, b_lane, n, col, val, total);
     if (shared_row) {
         __shared__ __attribute__((aligned(16))) A wg_sum[kWavesPerWg][TN];
         if (group == 0) {
@@ -173,7 +189,8 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, const int*
 // group walks its row's slot quads one after the other, no cross-lane reduction.
 template <typename T, int TN, bool EDGE>
 __device__ __forceinline__ void
-spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, const int* __restrict__ residue_rows,
+spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, int hub_min_len,
+                  const int* __restrict__ residue_rows,
                   const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                   typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
@@ -196,6 +213,7 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, const in
     const ResidueItem it = residue_item(row, row_ptr);
     const bool accumulate = it.accumulate; // the row also has block segments
     if (accumulate && it.aligned <= owned_slots) return; // summed entirely, tail included, by the block kernel
+    if (hub_min_len > 0 && it.aligned >= hub_min_len) return; // the hub kernel has the whole row
     const int first = it.first, cnt = it.cnt;
 
     const int tile = blockIdx.y * TN;
@@ -234,22 +252,25 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, const in
 
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_block_kernel(int m1, int n, int owned_slots, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+spmm_block_kernel(int m1, int n, int owned_slots, int hub_min_len, const int* __restrict__ block_rows,
+                  const int* __restrict__ st_off,
                   const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                   typename DenseVec<T>::Acc* __restrict__ C)
 {
-    spmm_block_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m1, n, owned_slots, block_rows, st_off, row_ptr, col, val, B, C);
+    spmm_block_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m1, n, owned_slots, hub_min_len, block_rows, st_off, row_ptr, col, val,
+                                 B, C);
 }
 
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ residue_rows,
+spmm_residue_kernel(int m2, int n, int owned_slots, int hub_min_len, const int* __restrict__ residue_rows,
                     const int* __restrict__ row_ptr, const int* __restrict__ col,
                     const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                     typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
-    spmm_residue_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m2, n, owned_slots, residue_rows, row_ptr, col, val, B, C, plan);
+    spmm_residue_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m2, n, owned_slots, hub_min_len, residue_rows, row_ptr, col, val, B,
+                                   C, plan);
 }
 
 // Both lists in one launch: the first g1 workgroups of a grid row work on block segments,
@@ -257,16 +278,107 @@ spmm_residue_kernel(int m2, int n, int owned_slots, const int* __restrict__ resi
 // kernel (a kernel of a few microseconds); the two parts then also fill the GPU together.
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, const int* __restrict__ block_rows,
+spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, int hub_min_len, const int* __restrict__ block_rows,
                  const int* __restrict__ residue_rows, const int* __restrict__ st_off, const int* __restrict__ row_ptr,
                  const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
                  const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
     if ((int)blockIdx.x < g1)
-        spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, block_rows, st_off, row_ptr, col, val, B, C);
+        spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, hub_min_len, block_rows, st_off, row_ptr, col, val, B, C);
     else
-        spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, max(owned_slots, 0), residue_rows, row_ptr, col, val,
+        spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, max(owned_slots, 0), hub_min_len, residue_rows,
+                                       row_ptr, col, val,
                                        B, C, plan);
+}
+
+// The rows of a hub plan, cut into pieces by column slab (rode_items.hpp): one wave per
+// piece, slab after slab, so that the hub rows' nonzeros of one slab of B are worked on at
+// the same time on one XCD and find B's rows in its L2.  A piece's sum goes to its own row
+// of `partial` (piece = slab group * hub rows + hub row; spmm_hub_reduce_kernel adds a row's
+// pieces up), or, without that workspace, is added to its row of C atomically (a hub row
+// then gets one atomic row update per slab: slower than the plain kernels at 512-byte rows).
+template <typename T, int TN, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+spmm_hub_kernel(int n, int merge, const int* __restrict__ hub, const int* __restrict__ col,
+                const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
+                typename DenseVec<T>::Acc* __restrict__ C, typename DenseVec<T>::Acc* __restrict__ partial)
+{
+    using S = SpmmShape<T, TN>;
+    using A = typename S::Acc;
+    constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
+    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
+    __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const HubPlan hp = hub_plan_view(hub);
+    const long long item = (long long)xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
+    if (item >= (long long)hp.n_hub * hub_groups(hp.slabs, merge)) return;
+    const int slab = (int)(item / hp.n_hub) * merge, h = (int)(item % hp.n_hub);
+    const int* piece = hp.pieces + (size_t)h * (hp.slabs + 1);
+    const int base = piece[slab], cnt = piece[min(slab + merge, hp.slabs)] - base;
+    if (cnt <= 0) return; // (the reduction skips empty pieces too)
+    const int row = hp.rows[h];
+    const int ls = lane % LPR, group = lane / LPR;
+    const int tile = blockIdx.y * TN;
+    const bool col_ok = !EDGE || tile + ls * VEC < n;
+    const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
+    constexpr int EPG = VEC / G > 0 ? VEC / G : 1; // elements each group adds
+    A total[VEC];
+    spmm_sum_slots<T, TN>(base, 0, cnt, lane, lds_c + wave * kWave, lds_v + wave * kWave, b_lane, n, col, val, total);
+    if (partial) {
+        if (group == 0 && col_ok) store_row<VEC>(partial + (size_t)item * n + tile + ls * VEC, total);
+        return;
+    }
+    A* c_lane = C + (size_t)row * n + tile + ls * VEC;
+#pragma unroll
+    for (int x = 0; x < VEC; ++x)
+        if (group == x / EPG && col_ok) atomicAdd(c_lane + x, total[x]);
+}
+
+// C[hub row, :] = sum of the row's pieces (a hub row is in no other work item, so this is
+// a plain store).  One workgroup per hub row: a group of n * sizeof / 16 threads reads a
+// piece's partial row 16 bytes per thread, the groups take the slabs in turn and their
+// sums are added up through LDS in a fixed order.
+template <typename A>
+__global__ void __launch_bounds__(kWgThreads)
+spmm_hub_reduce_kernel(int n, int merge, const int* __restrict__ hub, const A* __restrict__ partial, A* __restrict__ C)
+{
+    constexpr int V = 16 / sizeof(A);
+    __shared__ __attribute__((aligned(16))) A sums[kWgThreads * V];
+    const HubPlan hp = hub_plan_view(hub);
+    const int h = blockIdx.x;
+    if (h >= hp.n_hub) return;
+    const int* piece = hp.pieces + (size_t)h * (hp.slabs + 1);
+    A* c_row = C + (size_t)hp.rows[h] * n;
+    const int vecs = n / V; // 16-byte pieces of a row (n * sizeof(A) is a multiple of 16)
+    for (int v0 = 0; v0 < vecs; v0 += kWgThreads) {
+        const int width = min(vecs - v0, kWgThreads); // threads side by side on one partial row
+        const int groups = kWgThreads / width;
+        const int group = threadIdx.x / width, v = v0 + threadIdx.x % width;
+        A sum[V];
+#pragma unroll
+        for (int x = 0; x < V; ++x) sum[x] = A(0);
+        if (group < groups) {
+            for (int sg = group; sg * merge < hp.slabs; sg += groups) {
+                if (piece[min(sg * merge + merge, hp.slabs)] > piece[sg * merge]) {
+                    const A* src = partial + ((size_t)sg * hp.n_hub + h) * n + (size_t)v * V;
+#pragma unroll
+                    for (int x = 0; x < V; ++x) sum[x] += src[x];
+                }
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < V; ++x) sums[threadIdx.x * V + x] = sum[x];
+        __syncthreads();
+        if (group == 0) {
+            for (int g = 1; g < groups; ++g) {
+#pragma unroll
+                for (int x = 0; x < V; ++x) sum[x] += sums[(g * width + threadIdx.x) * V + x];
+            }
+#pragma unroll
+            for (int x = 0; x < V; ++x) c_row[(size_t)v * V + x] = sum[x];
+        }
+        __syncthreads();
+    }
 }
 
 constexpr int kClearRowsPerGroup = 8;
@@ -318,6 +430,10 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     // what the block kernel is told: rows it owns, or (negative) only that it may merge short
     // segments - which needs no promise, and with this many segments costs no parallelism
     const int block_owned = owned_slots > 0 ? owned_slots : (m1 >= kOwnedMinSegments ? -1 : 0);
+    // a usable hub plan takes its rows out of both lists (the caller promised whole lists with it)
+    const bool hubs = plan.hub != nullptr && plan.hub_counts != nullptr && plan.hub_counts[3] != 0 &&
+                      plan.hub_counts[0] > 0 && !(flags & (kSpmmOnlyBlock | kSpmmOnlyResidue));
+    const int hub_min_len = hubs ? plan.hub_counts[2] : 0;
     constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
     const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0 || tiles > 65535) return hipErrorInvalidConfiguration;
@@ -332,22 +448,35 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     hipError_t e = hipSuccess;
     if (block && residue && standard_residue && s1 == s2 && (long long)(g1 + g2) * tiles <= kPairMaxWorkgroups) {
         dim3 grid(g1 + g2, tiles);
-        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, block_rows, residue_rows,
+        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, hub_min_len, block_rows, residue_rows,
                                                                    st_off, row_ptr, col, val, B, C, plan.dev);
         e = hipGetLastError();
     } else {
         if (block) {
             dim3 grid(g1, tiles);
-            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, block_rows, st_off, row_ptr,
+            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, hub_min_len, block_rows, st_off, row_ptr,
                                                                         col, val, B, C);
             e = hipGetLastError();
         }
         if (residue && standard_residue) {
             dim3 grid(g2, tiles);
-            spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, residue_rows, row_ptr, col,
+            spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, hub_min_len, residue_rows, row_ptr, col,
                                                                           val, B, C, plan.dev);
             if (e == hipSuccess) e = hipGetLastError();
         }
+    }
+    if (e == hipSuccess && hubs) {
+        using A = typename DenseVec<T>::Acc;
+        const int merge = hub_merge(n * (int)sizeof(A) / 4);
+        const long long pieces = (long long)plan.hub_counts[0] * hub_groups(plan.hub_counts[1], merge);
+        const int gh = grid_for_waves(pieces);
+        if (gh < 0) return hipErrorInvalidConfiguration;
+        dim3 grid(gh, tiles);
+        const size_t need = (size_t)pieces * n * sizeof(A);
+        A* partial = plan.hub_workspace && plan.hub_workspace_bytes >= need ? static_cast<A*>(plan.hub_workspace) : nullptr;
+        spmm_hub_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(n, merge, plan.hub, col, val, B, C, partial);
+        if (partial) spmm_hub_reduce_kernel<A><<<plan.hub_counts[0], kWgThreads, 0, s1>>>(n, merge, plan.hub, partial, C);
+        e = hipGetLastError();
     }
     if constexpr (!std::is_same<T, double>::value) {
         if (e == hipSuccess && residue && window_residue)

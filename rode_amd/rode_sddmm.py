@@ -111,12 +111,37 @@ class RoDeCSR:
         # "auto" wants windows on at least half of the chunks and enough of them to fill the
         # GPU twice (a few windowed chunks only add launches); True keeps any plan with a
         # window; False makes none.
-        self.plan = None
-        if self.locality and m2 > 0:
+        self.plan = self._hub_plan() if self.locality else None
+        if self.plan is None and self.locality and m2 > 0:
             plan = rode_sddmm_hip.window_plan(res, m2, self.row_offsets, self.column_indices, self.n)
             enough = plan.windowed >= max(self.PLAN_MIN_CHUNKS, (plan.counts[0] + 1) // 2)
             if plan.windowed > 0 and (self.locality is True or enough):
                 self.plan = rode_sddmm_hip.window_plan_rows(plan, res, m2, self.row_offsets, self.column_indices)
+
+    # A hub plan is made when the rows of at least HUB_MIN_LEN nonzeros (and 8 per 4096
+    # columns) hold a tenth of the matrix and the matrix has at least HUB_MIN_SLABS times 4096
+    # columns (a smaller dense operand stays in the caches by itself).
+    HUB_MIN_LEN = 4096
+    HUB_MIN_SLABS = 16
+    HUB_MIN_SHARE = 0.1
+
+    def _hub_plan(self):
+        """Hub plan (rows with very many nonzeros are processed column slab by column slab so
+        that they share the dense rows they fetch), or None when the pattern has no use for it."""
+        slabs = (self.n + 4095) // 4096
+        if slabs < self.HUB_MIN_SLABS or self.nnz == 0:
+            return None
+        min_len = max(self.HUB_MIN_LEN, 8 * slabs)
+        ro = self.row_offsets_cpu.to(torch.int64)
+        aligned = ro[1:] - ro[:-1] + ro[:-1] % 4
+        hub = aligned >= min_len
+        share = float((ro[1:] - ro[:-1])[hub].sum()) / self.nnz
+        if self.locality is not True and share < self.HUB_MIN_SHARE:
+            return None
+        if not bool(hub.any()):
+            return None
+        plan = rode_sddmm_hip.hub_plan(self.row_offsets, self.column_indices, self.m, self.n, int(min_len))
+        return plan if plan.usable else None
 
     def with_values(self, values):
         """The same pattern and decomposition with other values (no preprocessing is

@@ -153,10 +153,79 @@ def csr_transpose(row_offsets, column_indices, m, n):
     return row_offsets_t, column_indices_t, perm
 
 
+class HubPlan:
+    """Hub plan of one pattern (``rode_hip_hub_plan``): the device array and a host copy
+    of its header ``[hub rows, slabs, min_len, usable, room, 0, 0, 0]``."""
+
+    def __init__(self, data, counts):
+        self.data = data
+        self.counts = counts
+        self._header = (ctypes.c_int * 8)(*counts)
+        self.rows = None  # (a matrix has a hub plan or a locality plan, never both)
+        self._workspaces = {}
+
+    def workspace(self, n, elem_bytes):
+        """Scratch for the SpMM hub kernels at dense width ``n`` (one partial row of C per
+        hub row and slab); kept for the next call.  Calls that overlap in time on different
+        streams must not share it."""
+        key = (n, elem_bytes)
+        if key not in self._workspaces:
+            nbytes = _lib.load().rode_hip_hub_workspace_bytes(ctypes.addressof(self._header), n, elem_bytes)
+            self._workspaces[key] = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.data.device)
+        return self._workspaces[key]
+
+    @property
+    def usable(self):
+        return self.counts[3] != 0 and self.counts[0] > 0
+
+    def hub_rows(self):
+        return self.data[8:8 + self.counts[0]].cpu().numpy()
+
+    def pieces(self):
+        """int32 array (hub rows, slabs + 1): where every hub row's nonzeros of each column slab start."""
+        first = 8 + self.counts[4]
+        return self.data[first:first + self.counts[0] * (self.counts[1] + 1)].cpu().numpy().reshape(self.counts[0], -1)
+
+
+def hub_plan(row_offsets, column_indices, m, n, min_len):
+    """Hub plan: the rows of at least ``min_len`` aligned nonzero slots, cut into pieces by
+    slab of 2048 columns.  Waits for its two kernels (it returns the counts)."""
+    for t, name in ((row_offsets, "row_offsets"), (column_indices, "column_indices")):
+        _check_input(t, name)
+        _check(t.dtype == torch.int32, f"{name} must be int32")
+    lib = _lib.load()
+    dev = row_offsets.device
+    nnz = column_indices.numel()
+    nbytes = lib.rode_hip_hub_plan_bytes(m, n, nnz, min_len)
+    _check(nbytes > 0, "min_len is too small for a hub plan")
+    with torch.cuda.device(dev):
+        data = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
+        counts = (ctypes.c_int * 8)()
+        _lib.check(lib.rode_hip_hub_plan(m, n, nnz, min_len, row_offsets.data_ptr(), column_indices.data_ptr(),
+                                         data.data_ptr(), nbytes, ctypes.addressof(counts), _stream_handle(dev)),
+                   "rode_hip_hub_plan")
+    return HubPlan(data, list(counts))
+
+
+def _spmm_plan_args(plan, whole_lists, n, out):
+    """The seven plan arguments of ``rode_hip_spmm_planned``: those of ``_plan_args`` and
+    the hub kernels' workspace."""
+    if isinstance(plan, HubPlan) and plan.usable and whole_lists:
+        ws = plan.workspace(n, out.element_size())
+        return (*_plan_args(plan), ws.data_ptr(), ws.numel())
+    return (*_plan_args(None if isinstance(plan, HubPlan) else plan), None, 0)
+
+
 def _plan_args(plan):
+    """The five plan arguments of the ``*_planned`` entry points: locality plan (descriptors,
+    rows, host header), hub plan (array, host header)."""
+    if isinstance(plan, HubPlan):
+        if not plan.usable:
+            return None, None, None, None, None
+        return None, None, None, plan.data.data_ptr(), ctypes.addressof(plan._header)
     if plan is None or plan.rows is None:
-        return None, None, None
-    return plan.data.data_ptr(), plan.rows.data_ptr(), ctypes.addressof(plan._header)
+        return None, None, None, None, None
+    return plan.data.data_ptr(), plan.rows.data_ptr(), ctypes.addressof(plan._header), None, None
 
 
 def preprocess(row_offsets, nnz, seg_length, k_block, vec_len):
@@ -233,7 +302,8 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     ``out`` accumulated in place the way the reference kernels do (long rows add,
     short rows overwrite).  ``whole_lists`` promises that the index tensors are the
     complete decomposition (always true for a ``RoDeCSR``); pass False for a slice.
-    ``plan``: a ``WindowPlan`` made from these very lists, or None."""
+    ``plan``: a ``WindowPlan`` made from these very lists, a ``HubPlan`` of this pattern
+    (used only with ``whole_lists``), or None."""
     for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
                     (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
                     (values, "values"), (dense_matrix, "dense_matrix")):
@@ -272,6 +342,7 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
         code = lib.rode_hip_spmm_planned(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
                                          values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
                                          block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
-                                         dense_matrix.data_ptr(), out.data_ptr(), *_plan_args(plan), s, s)
+                                         dense_matrix.data_ptr(), out.data_ptr(), *_spmm_plan_args(plan, whole_lists, n, out),
+                                         s, s)
     _lib.check(code, "rode_hip_spmm_planned")
     return out
