@@ -70,35 +70,42 @@ def parse_args():
     return p.parse_args()
 
 
-def work_split(row_ptr, col, ncols, owned_slots=0):
+def work_split(row_ptr, col, ncols, owned_slots=0, hub_min_len=0):
     """Which nonzeros the residue kernels own (tail rule of RoDeSpmm.cu:71-82) and how
     many distinct dense rows each kernel family touches.  ``owned_slots``: rows of
-    32..owned_slots aligned slots are summed, tail included, by the SpMM block kernel."""
+    32..owned_slots aligned slots are summed, tail included, by the SpMM block kernel.
+    ``hub_min_len`` > 0: rows of at least that many aligned slots belong, whole, to the
+    hub kernels."""
     rp = row_ptr.astype(np.int64)
     s, e = rp[:-1], rp[1:]
     pad = s % 4
     N = e - s + pad
+    hub_row = (N >= hub_min_len) if hub_min_len > 0 else np.zeros(len(N), dtype=bool)
     tail_first = np.where(N >= 32, s - pad + N // 32 * 32, s)
     tail_first = np.where((N >= 32) & (N <= owned_slots), e, tail_first)
-    in_res = np.arange(rp[-1], dtype=np.int64) >= np.repeat(tail_first, e - s)
-    nnz_res = int(in_res.sum())
-    distinct_res = int((np.bincount(col[in_res], minlength=ncols) > 0).sum())
-    distinct_blk = int((np.bincount(col[~in_res], minlength=ncols) > 0).sum())
-    rows_blk = int((N >= 32).sum())
-    rows_res = int((((N % 32) != 0) & (N > 0) & ~((N >= 32) & (N <= owned_slots))).sum())
-    return {"nnz_res": nnz_res, "nnz_blk": int(rp[-1]) - nnz_res, "distinct_res": distinct_res,
-            "distinct_blk": distinct_blk, "rows_blk": rows_blk, "rows_res": rows_res}
+    in_hub = np.repeat(hub_row, e - s)
+    in_res = (np.arange(rp[-1], dtype=np.int64) >= np.repeat(tail_first, e - s)) & ~in_hub
+    in_blk = ~in_res & ~in_hub
+    nnz_res, nnz_hub = int(in_res.sum()), int(in_hub.sum())
+    distinct = lambda mask: int((np.bincount(col[mask], minlength=ncols) > 0).sum())
+    rows_blk = int(((N >= 32) & ~hub_row).sum())
+    rows_res = int((((N % 32) != 0) & (N > 0) & ~((N >= 32) & (N <= owned_slots)) & ~hub_row).sum())
+    return {"nnz_res": nnz_res, "nnz_blk": int(rp[-1]) - nnz_res - nnz_hub, "nnz_hub": nnz_hub,
+            "distinct_res": distinct(in_res), "distinct_blk": distinct(in_blk), "distinct_hub": distinct(in_hub),
+            "rows_blk": rows_blk, "rows_res": rows_res, "rows_hub": int(hub_row.sum())}
 
 
 def algorithmic_bytes(kernel, split, m1, m2, k, elem):
     """Compulsory traffic of one launch: every array element it needs, once."""
     if kernel.endswith("block"):
         nnz, rows, distinct, meta = split["nnz_blk"], split["rows_blk"], split["distinct_blk"], m1 * 12 + 4
+    elif kernel.endswith("hub"):
+        nnz, rows, distinct, meta = split["nnz_hub"], split["rows_hub"], split["distinct_hub"], split["rows_hub"] * 12
     else:
         nnz, rows, distinct, meta = split["nnz_res"], m2, split["distinct_res"], m2 * 12
     if kernel.startswith("spmm"):
         # (col, val) + metadata + distinct B rows + C rows (atomic rows are read and written)
-        c_bytes = rows * k * 4 * (2 if kernel.endswith("block") else 1)
+        c_bytes = rows * k * 4 * (2 if kernel.endswith("block") else 1)  # (hub rows and short rows are stored)
         return nnz * 8 + meta + distinct * k * elem + c_bytes
     # sddmm: (col, val) + metadata + lhs rows + distinct rhs rows + out
     return nnz * 8 + meta + rows * k * elem + distinct * k * elem + nnz * 4
@@ -145,8 +152,8 @@ def main():
                                          *plan_args, hub_ws.data_ptr() if hub is not None else None,
                                          hub_ws.numel() if hub is not None else 0, *a[-2:])
 
-    def sddmm_fn(*a):
-        return lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[args.dtype], *a[:-2], *plan_args, *a[-2:])
+    def sddmm_fn(*a, flags=0):
+        return lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[args.dtype], flags, *a[:-2], *plan_args, *a[-2:])
 
     main_stream = torch.cuda.current_stream()
     side = torch.cuda.Stream() if args.two_streams else None
@@ -182,11 +189,11 @@ def main():
                            csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, s2), "spmm")
         join()
 
-    def sddmm(m1, m2):
+    def sddmm(m1, m2, flags=0):
         s2 = fork()
         _lib.check(sddmm_fn(m1, m2, n, k, csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
                             csr.st_offsets.data_ptr(), csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
-                            csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), out.data_ptr(), stream, s2),
+                            csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), out.data_ptr(), stream, s2, flags=flags),
                    "sddmm")
         join()
 
@@ -266,10 +273,13 @@ def main():
     kernels = {}
     if csr.m1 > 0:
         kernels["spmm_block"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_BLOCK), reps)  # incl. rows summed whole
-        kernels["sddmm_block"] = event_time(lambda: sddmm(csr.m1, 0), reps)
+        kernels["sddmm_block"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_BLOCK), reps)
     if csr.m2 > 0:
         kernels["spmm_residue"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_RESIDUE), reps)
-        kernels["sddmm_residue"] = event_time(lambda: sddmm(0, csr.m2), reps)
+        kernels["sddmm_residue"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_RESIDUE), reps)
+    if hub is not None:  # the rows of the hub plan: piece kernel (+ the sum of the partial rows of C for SpMM)
+        kernels["spmm_hub"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_HUB), reps)
+        kernels["sddmm_hub"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_HUB), reps)
     spmm_ms = event_time(lambda: (clear_c(), spmm(csr.m1, csr.m2)), reps)
     sddmm_ms = event_time(lambda: sddmm(csr.m1, csr.m2), reps)
     spmm_contract_ms = event_time(spmm_reference_contract, reps)
@@ -282,8 +292,9 @@ def main():
         del src, dst
 
     # the SpMM block kernel sums rows of 32..1024 slots whole when there are >= 16384 segments
-    split_sddmm = work_split(row_ptr, col, n)
-    split_spmm = work_split(row_ptr, col, n, 1024 if csr.m1 >= 16384 else 0)
+    hub_min_len = hub.counts[2] if hub is not None else 0
+    split_sddmm = work_split(row_ptr, col, n, 0, hub_min_len)
+    split_spmm = work_split(row_ptr, col, n, 1024 if csr.m1 >= 16384 else 0, hub_min_len)
     per_kernel = {}
     for name, ms in kernels.items():
         split = split_spmm if name.startswith("spmm") else split_sddmm
@@ -291,7 +302,7 @@ def main():
         if name == "spmm_residue":
             m2_eff = split["rows_res"]
         ab = algorithmic_bytes(name, split, csr.m1, m2_eff, k, elem)
-        knnz = split["nnz_blk"] if name.endswith("block") else split["nnz_res"]
+        knnz = split["nnz_" + {"block": "blk", "residue": "res", "hub": "hub"}[name.split("_")[1]]]
         per_kernel[name] = {"ms": round(ms, 4), "algorithmic_bytes": ab,
                             "algorithmic_GBs": round(ab / ms / 1e6, 1),
                             "gather_model_GBs": round((knnz * (8 + k * elem)) / ms / 1e6, 1),
@@ -303,7 +314,7 @@ def main():
         table = json.load(open(tpath))
         prefix = f"{args.workload}/k{k}/{args.dtype}/seg{csr.config['seg_length']}/"
         # with a locality plan the residue rows are the window kernel's
-        windowed = csr.plan is not None and dominant.endswith("residue") and k * elem > 128
+        windowed = csr.plan is not None and hub is None and dominant.endswith("residue") and k * elem > 128
         entry = table.get(prefix + dominant + "_window") if windowed else None
         entry = entry or table.get(prefix + dominant)
         if entry is not None and entry.get("sources") == kernel_sources_fingerprint():
@@ -435,8 +446,11 @@ def main():
                                   else "step = clear C rows + SpMM + SDDMM"),
                    "rows": m, "cols": n, "nnz": nnz, "K": k, "seg_length": csr.config["seg_length"],
                    "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale,
-                   "locality_plan": None if csr.plan is None else
-                   {"residue_chunks": csr.plan.counts[0], "chunks_with_lds_window": csr.plan.counts[1]}},
+                   "locality_plan": None if csr.plan is None or hub is not None else
+                   {"residue_chunks": csr.plan.counts[0], "chunks_with_lds_window": csr.plan.counts[1]},
+                   "hub_plan": None if hub is None else
+                   {"hub_rows": hub.counts[0], "shortest": hub.counts[2], "nnz_share": round(split_sddmm["nnz_hub"] / nnz, 3),
+                    "column_slabs": hub.counts[1], "slab_rows": 2048}},
         "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C",
                  "reference_contract_ms": round(spmm_contract_ms, 4),
                  "reference_contract": "memset of all of C + the typed entry point without the whole-lists promise "

@@ -131,12 +131,14 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
 #define RODE_DENSE_F16 1
 #define RODE_DENSE_F64 2
 #define RODE_SPMM_WHOLE_LISTS 1
-/* Launch only the block-segment kernel / only the residue kernel of the pair, with every
- * other decision (which rows a single wavefront sums whole) taken as if both were
- * launched: for measuring one kernel, and for callers that order the two themselves.
- * m1, m2 and all lists are passed as for a normal call. */
+/* Launch only the block-segment kernel / only the residue kernel / only the kernels of a
+ * hub plan, with every other decision (which rows a single wavefront sums whole, which rows
+ * the hub kernels take) made as if all were launched: for measuring one kernel, and for
+ * callers that order them themselves.  m1, m2, all lists and plans are passed as for a
+ * normal call; at most one of the three bits. */
 #define RODE_SPMM_ONLY_BLOCK 2
 #define RODE_SPMM_ONLY_RESIDUE 4
+#define RODE_SPMM_ONLY_HUB 8
 int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                      const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                      const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
@@ -214,8 +216,8 @@ int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_
  * rode_hip_window_plan returned; with it, kernels that would find no chunk to work on are
  * not launched at all.  fp64 operands, and dense rows of at most 128 bytes, ignore the
  * locality plan.  d_hub_plan / h_hub_counts: a hub plan of this matrix and its header, or
- * NULL; it needs RODE_SPMM_WHOLE_LISTS (the hub kernels replace work items of both lists)
- * and no RODE_SPMM_ONLY_* flag.  d_hub_workspace: rode_hip_hub_workspace_bytes(h_hub_counts,
+ * NULL; it needs RODE_SPMM_WHOLE_LISTS (the hub kernels replace work items of both lists).
+ * d_hub_workspace: rode_hip_hub_workspace_bytes(h_hub_counts,
  * n, 4 or 8) bytes of scratch, 16-byte aligned, that the hub kernels of this call may write
  * and read (one partial row of C per hub row and slab, summed by a second kernel), or NULL:
  * the pieces are then added to C atomically, which is slower for wide rows.  With every
@@ -281,10 +283,11 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
  * lhs / rhs; d_plan / d_plan_rows / h_plan_counts and d_hub_plan / h_hub_counts as for
  * rode_hip_spmm_planned (all NULL: exactly the typed functions above).  With a hub plan the
  * lists must be the complete decomposition (the hub kernels replace work items of both).
+ * flags: 0, or one of the RODE_SPMM_ONLY_* bits (one kernel family of the call).
  * Same results up to the order of the fp32 additions of a dot product.  No counterpart in
  * the reference.
  */
-int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d_row_indices_block,
+int rode_hip_sddmm_planned(int dtype, int flags, int m1, int m2, int n, int k, const int* d_row_indices_block,
                            const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                            const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
                            const void* d_rhs_matrix, float* d_out, const void* d_plan, const void* d_plan_rows,

@@ -35,7 +35,7 @@ SIGNATURES = {
     "rode_hip_spmm_clear_rows": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "rode_hip_sddmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 11),
     "rode_hip_sddmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 11),
-    "rode_hip_sddmm_planned": (c_int, [c_int] * 5 + [c_void_p] * 16),
+    "rode_hip_sddmm_planned": (c_int, [c_int] * 6 + [c_void_p] * 16),
     "rode_hip_csr_softmax_f32": (c_int, [c_int, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p]),
     "rode_hip_csr_softmax_backward_f32": (c_int, [c_int] + [c_void_p] * 4 + [ctypes.c_float, c_void_p]),
     "rode_hip_csr_transpose_workspace_bytes": (c_size_t, [c_int]),
@@ -44,7 +44,7 @@ SIGNATURES = {
 }
 
 DENSE_CODE = {"f32": 0, "f16": 1, "f64": 2}  # RODE_DENSE_* of include/rode_hip.h
-SPMM_WHOLE_LISTS, SPMM_ONLY_BLOCK, SPMM_ONLY_RESIDUE = 1, 2, 4  # RODE_SPMM_* flags
+SPMM_WHOLE_LISTS, SPMM_ONLY_BLOCK, SPMM_ONLY_RESIDUE, SPMM_ONLY_HUB = 1, 2, 4, 8  # RODE_SPMM_* flags
 
 _lib = None
 

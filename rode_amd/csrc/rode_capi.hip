@@ -199,11 +199,13 @@ int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, co
                           void* stream2)
 {
     (void)k;
-    constexpr int kKnown = RODE_SPMM_WHOLE_LISTS | RODE_SPMM_ONLY_BLOCK | RODE_SPMM_ONLY_RESIDUE;
+    constexpr int kKnown = RODE_SPMM_WHOLE_LISTS | RODE_SPMM_ONLY_BLOCK | RODE_SPMM_ONLY_RESIDUE | RODE_SPMM_ONLY_HUB;
     static_assert(RODE_SPMM_WHOLE_LISTS == rode::kSpmmWholeLists && RODE_SPMM_ONLY_BLOCK == rode::kSpmmOnlyBlock &&
-                      RODE_SPMM_ONLY_RESIDUE == rode::kSpmmOnlyResidue, "header and library disagree");
+                      RODE_SPMM_ONLY_RESIDUE == rode::kSpmmOnlyResidue && RODE_SPMM_ONLY_HUB == rode::kSpmmOnlyHub,
+                  "header and library disagree");
     if (m1 < 0 || m2 < 0 || (flags & ~kKnown)) return hipErrorInvalidValue;
-    if ((flags & RODE_SPMM_ONLY_BLOCK) && (flags & RODE_SPMM_ONLY_RESIDUE)) return hipErrorInvalidValue;
+    const int only = flags & rode::kOnlyMask;
+    if (only & (only - 1)) return hipErrorInvalidValue; // at most one ONLY bit
     if (m1 == 0 && m2 == 0) return hipSuccess;
     if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
     hipStream_t s1 = as_stream(stream1), s2 = as_stream(stream2);
@@ -266,7 +268,7 @@ int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const
                             d_row_indices2, d_row_seg_st_offsets, d_B_half, d_C, stream1, stream2);
 }
 
-int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d_row_indices_block,
+int rode_hip_sddmm_planned(int dtype, int flags, int m1, int m2, int n, int k, const int* d_row_indices_block,
                            const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                            const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
                            const void* d_rhs_matrix, float* d_out, const void* d_plan, const void* d_plan_rows,
@@ -274,11 +276,12 @@ int rode_hip_sddmm_planned(int dtype, int m1, int m2, int n, int k, const int* d
                            void* stream2)
 {
     (void)n;
-    if (m1 < 0 || m2 < 0) return hipErrorInvalidValue;
+    if (m1 < 0 || m2 < 0 || (flags & ~rode::kOnlyMask) || (flags & (flags - 1))) return hipErrorInvalidValue;
     if (m1 == 0 && m2 == 0) return hipSuccess;
     if (!aligned16(d_lhs_matrix) || !aligned16(d_rhs_matrix)) return hipErrorInvalidValue;
     rode::PlanRef plan;
     if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, d_hub_plan, h_hub_counts, m2, plan)) return hipErrorInvalidValue;
+    plan.only = flags;
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::sddmm_launch<float>(m1, m2, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
@@ -300,7 +303,7 @@ int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_bl
                        const float* d_values, const float* d_lhs_matrix, const float* d_rhs_matrix, float* d_out,
                        void* stream1, void* stream2)
 {
-    return rode_hip_sddmm_planned(RODE_DENSE_F32, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
+    return rode_hip_sddmm_planned(RODE_DENSE_F32, 0, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
                                   d_row_offsets, d_column_indices, d_values, d_lhs_matrix, d_rhs_matrix, d_out, nullptr,
                                   nullptr, nullptr, nullptr, nullptr, stream1, stream2);
 }
@@ -310,7 +313,7 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
                        const float* d_values, const void* d_lhs_half, const void* d_rhs_half, float* d_out,
                        void* stream1, void* stream2)
 {
-    return rode_hip_sddmm_planned(RODE_DENSE_F16, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
+    return rode_hip_sddmm_planned(RODE_DENSE_F16, 0, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
                                   d_row_offsets, d_column_indices, d_values, d_lhs_half, d_rhs_half, d_out, nullptr,
                                   nullptr, nullptr, nullptr, nullptr, stream1, stream2);
 }

@@ -23,7 +23,8 @@ template <typename T> struct SpmmAcc { using type = float; };
 template <> struct SpmmAcc<double> { using type = double; };
 
 // flags: the RODE_SPMM_* bits of the C ABI
-constexpr int kSpmmWholeLists = 1, kSpmmOnlyBlock = 2, kSpmmOnlyResidue = 4;
+constexpr int kSpmmWholeLists = 1, kSpmmOnlyBlock = 2, kSpmmOnlyResidue = 4, kSpmmOnlyHub = 8;
+constexpr int kOnlyMask = kSpmmOnlyBlock | kSpmmOnlyResidue | kSpmmOnlyHub;
 
 // A locality plan (rode_plan.hip): device array, and optionally a host copy of its four
 // header ints (chunk counts), with which launches that have nothing to do are left out.
@@ -37,6 +38,8 @@ struct PlanRef {
     // SpMM only: room for one partial row of C per (slab, hub row), or null (atomics instead).
     void* hub_workspace = nullptr;
     size_t hub_workspace_bytes = 0;
+    // SDDMM: the RODE_SPMM_ONLY_* bits of the call (SpMM carries them in its flags)
+    int only = 0;
 };
 
 hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, const int* col, int* plan,

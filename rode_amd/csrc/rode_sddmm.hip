@@ -248,8 +248,13 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
         standard_residue = plan.host_counts[1] < plan.host_counts[0];
         window_residue = plan.host_counts[1] > 0;
     }
-    const bool hubs = plan.hub != nullptr && plan.hub_counts != nullptr && plan.hub_counts[3] != 0 && plan.hub_counts[0] > 0;
-    const int hub_min_len = hubs ? plan.hub_counts[2] : 0;
+    const bool hub_plan = plan.hub != nullptr && plan.hub_counts != nullptr && plan.hub_counts[3] != 0 && plan.hub_counts[0] > 0;
+    const int hub_min_len = hub_plan ? plan.hub_counts[2] : 0;
+    const bool hubs = hub_plan && (plan.only == 0 || plan.only == kSpmmOnlyHub);
+    if (plan.only != 0) { // one kernel family of the call (timing each on its own)
+        if (plan.only != kSpmmOnlyBlock) m1 = 0;
+        if (plan.only != kSpmmOnlyResidue) m2 = 0;
+    }
     if (m1 > 0 && m2 > 0 && standard_residue && s1 == s2 && g1 + g2 <= kPairMaxWorkgroups) {
         sddmm_pair_kernel<T, KT, NS, EDGE><<<g1 + g2, kWgThreads, 0, s1>>>(
             g1, m1, m2, k, hub_min_len, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);

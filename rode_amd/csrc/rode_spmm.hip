@@ -431,9 +431,11 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     // segments - which needs no promise, and with this many segments costs no parallelism
     const int block_owned = owned_slots > 0 ? owned_slots : (m1 >= kOwnedMinSegments ? -1 : 0);
     // a usable hub plan takes its rows out of both lists (the caller promised whole lists with it)
-    const bool hubs = plan.hub != nullptr && plan.hub_counts != nullptr && plan.hub_counts[3] != 0 &&
-                      plan.hub_counts[0] > 0 && !(flags & (kSpmmOnlyBlock | kSpmmOnlyResidue));
-    const int hub_min_len = hubs ? plan.hub_counts[2] : 0;
+    const bool hub_plan = plan.hub != nullptr && plan.hub_counts != nullptr && plan.hub_counts[3] != 0 &&
+                          plan.hub_counts[0] > 0;
+    const int hub_min_len = hub_plan ? plan.hub_counts[2] : 0;
+    const int only = flags & kOnlyMask; // one kernel family of the call (timing each on its own)
+    const bool hubs = hub_plan && (only == 0 || only == kSpmmOnlyHub);
     constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
     const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0 || tiles > 65535) return hipErrorInvalidConfiguration;
@@ -444,7 +446,7 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
         standard_residue = plan.host_counts[1] < plan.host_counts[0];
         window_residue = plan.host_counts[1] > 0;
     }
-    const bool block = m1 > 0 && !(flags & kSpmmOnlyResidue), residue = m2 > 0 && !(flags & kSpmmOnlyBlock);
+    const bool block = m1 > 0 && (only == 0 || only == kSpmmOnlyBlock), residue = m2 > 0 && (only == 0 || only == kSpmmOnlyResidue);
     hipError_t e = hipSuccess;
     if (block && residue && standard_residue && s1 == s2 && (long long)(g1 + g2) * tiles <= kPairMaxWorkgroups) {
         dim3 grid(g1 + g2, tiles);

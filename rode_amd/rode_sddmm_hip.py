@@ -285,7 +285,7 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
     lib = _lib.load()
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
-        code = lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[kind], m1, m2, n, k, block_indices.data_ptr(),
+        code = lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[kind], 0, m1, m2, n, k, block_indices.data_ptr(),
                                           residue_indices.data_ptr(), st_offsets.data_ptr(), row_offsets.data_ptr(),
                                           column_indices.data_ptr(), values.data_ptr(), lhs_matrix.data_ptr(),
                                           rhs_matrix.data_ptr(), out.data_ptr(), *_plan_args(plan), s, s)

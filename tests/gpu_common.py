@@ -18,9 +18,9 @@ def t(a):
     return torch.from_numpy(np.ascontiguousarray(a))
 
 
-def make_csr(row_ptr, col, val, m, n, k, seg=None):
+def make_csr(row_ptr, col, val, m, n, k, seg=None, locality="auto"):
     cfg = None if seg is None else {"seg_length": seg, "k_block": 32, "vec_len": 4}
-    return RoDeCSR(t(row_ptr), t(col), t(val), DEV, m, n, k, config=cfg)
+    return RoDeCSR(t(row_ptr), t(col), t(val), DEV, m, n, k, config=cfg, locality=locality)
 
 
 def gpu_preprocess(row_ptr, seg, kb=32, vl=4):
