@@ -334,8 +334,8 @@ spmm_hub_kernel(int n, int merge, const int* __restrict__ hub, const int* __rest
         if (group == x / EPG && col_ok) atomicAdd(c_lane + x, total[x]);
 }
 
-// C[hub row, :] = sum of the row's pieces (a hub row is in no other work item, so this is
-// a plain store).  One workgroup per hub row: a group of n * sizeof / 16 threads reads a
+// C[hub row, :] += sum of the row's pieces (a hub row is in no other work item, so no
+// atomics; added, not stored, because long rows are accumulated into C by contract).  One workgroup per hub row: a group of n * sizeof / 16 threads reads a
 // piece's partial row 16 bytes per thread, the groups take the slabs in turn and their
 // sums are added up through LDS in a fixed order.
 template <typename A>
@@ -375,7 +375,7 @@ spmm_hub_reduce_kernel(int n, int merge, const int* __restrict__ hub, const A* _
                 for (int x = 0; x < V; ++x) sum[x] += sums[(g * width + threadIdx.x) * V + x];
             }
 #pragma unroll
-            for (int x = 0; x < V; ++x) c_row[(size_t)v * V + x] = sum[x];
+            for (int x = 0; x < V; ++x) c_row[(size_t)v * V + x] += sum[x];
         }
         __syncthreads();
     }

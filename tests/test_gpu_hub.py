@@ -74,6 +74,18 @@ def test_hub_rows_against_oracle(k, half):
     Bq, Lq = (round_half(B), round_half(L)) if half else (B, L)
     tol = TOL_F16 if half else TOL_F32
     assert spmm_row_l1_error(run_spmm(csr, B, half), oracle.spmm_f64(rp, col, val, Bq)) <= tol
+    if k == 64:  # fp64 through the same plan, and accumulation into a C that is not zero
+        from rode_amd import rode_sddmm_hip
+        dev = csr.device
+        C0 = torch.from_numpy(rng.standard_normal((m, k))).to(dev)
+        C = C0.clone()
+        rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                    csr.row_offsets, csr.column_indices, csr.values.double(), m, n,
+                                    torch.from_numpy(B).to(dev).double(), out=C, plan=csr.plan)
+        ref = oracle.spmm_f64(rp, col, val, B)
+        added = (np.diff(rp) + rp[:-1] % 4) >= 32  # long rows are added to, short rows overwritten
+        want = ref + np.where(added[:, None], C0.cpu().numpy(), 0.0)
+        assert spmm_row_l1_error(C.cpu().numpy(), want) <= 1e-12
     ref64, scale = oracle.sddmm_f64(rp, col, val, Lq, Bq, with_abs=True)
     out = run_sddmm(csr, L, B, half)
     err, cond = sddmm_row_l1_errors(out, ref64, scale, rp)
