@@ -78,6 +78,8 @@ class SpmmFunction(torch.autograd.Function):
 def _softmax_call(fn_name, row_offsets, a, b, scale):
     lib = _lib.load()
     out = torch.empty_like(a)
+    if a.numel() == 0:  # a pattern without nonzeros
+        return out
     m = row_offsets.numel() - 1
     with torch.cuda.device(a.device):
         s = torch.cuda.current_stream(a.device).cuda_stream
@@ -124,8 +126,10 @@ FUSED_MAX_ROW = 16384
 def _attention_call(csr, values, q, k, v, scale, want_probs):
     lib = _lib.load()
     m, d = q.shape
-    out = torch.empty((m, d), dtype=torch.float32, device=q.device)
     probs = torch.empty_like(values) if want_probs else None
+    if values.numel() == 0:  # no nonzeros: nothing attends to anything
+        return torch.zeros((m, d), dtype=torch.float32, device=q.device), probs
+    out = torch.empty((m, d), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         code = lib.rode_hip_attention_forward(
             _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"], m, d, csr.row_offsets.data_ptr(),

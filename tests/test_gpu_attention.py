@@ -199,9 +199,9 @@ def test_fused_attention_kernel_against_the_three_kernels(d, half):
     from rode_amd import csr_row_softmax, rode_sddmm, sparse_attention
     from rode_amd.autograd import _attention_call
     rng = np.random.default_rng(100 + d)
-    m, n = 300, 900
+    m, n = 300, 2000
     lens = rng.integers(0, 90, m)
-    lens[:8] = [0, 1, 63, 64, 65, 700, 0, 128]
+    lens[:9] = [0, 1, 63, 64, 65, 700, 0, 128, 1500 if d == 64 else 40]  # 1500: longer than the scores kept in LDS
     rp = np.zeros(m + 1, dtype=np.int32)
     rp[1:] = np.cumsum(lens)
     col = np.concatenate([np.sort(rng.choice(n, l, replace=False)) for l in lens]).astype(np.int32)
@@ -237,6 +237,18 @@ def test_fused_attention_kernel_against_the_three_kernels(d, half):
     assert (chain_p - probs).abs().max().item() <= tol
     chain = sparse_attention(mask, q, k, v, scale=scale, fused=False)
     assert (chain - out).abs().max().item() <= tol * max(1.0, chain.abs().max().item())
+
+
+def test_fused_attention_without_nonzeros():
+    from gpu_common import DEV, make_csr
+    from rode_amd import sparse_attention
+    m, n, d = 10, 12, 32
+    rp = np.zeros(m + 1, dtype=np.int32)
+    mask = make_csr(rp, np.zeros(0, dtype=np.int32), np.zeros(0, dtype=np.float32), m, n, d)
+    z = lambda r: torch.ones(r, d, device=DEV)
+    for fused in (True, False):
+        out = sparse_attention(mask, z(m), z(n), z(n), fused=fused)
+        assert out.shape == (m, d) and not out.any()
 
 
 def test_fused_attention_dispatch():
