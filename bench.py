@@ -65,6 +65,8 @@ def parse_args():
                    help="clear all of C before SpMM (the reference's contract) instead of only the rows SpMM adds to")
     p.add_argument("--no-plan", action="store_true",
                    help="do not use the locality plan (window kernels for chunks whose dense rows fit an LDS window)")
+    p.add_argument("--graph", action="store_true",
+                   help="capture one step in a HIP graph and time its replays (launch-bound workloads)")
     p.add_argument("--calibrate", action="store_true",
                    help="also run one plain device copy of 256 MiB (a known size to scale profiler counters by)")
     return p.parse_args()
@@ -228,12 +230,26 @@ def main():
         spmm(csr.m1, csr.m2)
         sddmm(csr.m1, csr.m2)
 
+    run_step = step
+    if args.graph:
+        # the step allocates nothing and never waits for the host, so it can be captured as it is
+        side_stream = torch.cuda.Stream()
+        side_stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side_stream):
+            stream = side_stream.cuda_stream
+            step()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side_stream):
+                step()
+        stream = torch.cuda.current_stream().cuda_stream
+        run_step = graph.replay
     for _ in range(args.warmup):
-        step()
+        run_step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run_step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
