@@ -305,7 +305,12 @@ hipError_t sddmm_launch(int m1, int m2, int k, const int* block_rows, const int*
                         float* out, PlanRef plan, hipStream_t s1, hipStream_t s2)
 {
     if (k <= 0 || k % DenseVec<T>::kElems != 0 || k > 512) return hipErrorInvalidValue;
-    if ((size_t)k * sizeof(T) <= 128) plan = PlanRef{};
+    // the window kernels are for rows of more than one 128-byte tile
+    if ((size_t)k * sizeof(T) <= 128) {
+        plan.dev = nullptr;
+        plan.rows = nullptr;
+        plan.host_counts = nullptr;
+    }
 #define RODE_SDDMM_CASE(KT, NS)                                                                                   \
     return launch_edge<T, KT, NS>(k != (KT) * (NS), m1, m2, k, block_rows, residue_rows, st_off, row_ptr, col, val, \
                                   lhs, rhs, out, plan, s1, s2)

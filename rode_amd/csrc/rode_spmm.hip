@@ -514,7 +514,12 @@ hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* 
 {
     static_assert(std::is_same<typename SpmmAcc<T>::type, typename DenseVec<T>::Acc>::value, "accumulation type");
     if (n <= 0 || n % DenseVec<T>::kElems != 0) return hipErrorInvalidValue;
-    if (std::is_same<T, double>::value || (size_t)n * sizeof(T) <= 128) plan = PlanRef{};
+    // the window kernels are for fp32 / fp16 operands with more than one 128-byte tile per row
+    if (std::is_same<T, double>::value || (size_t)n * sizeof(T) <= 128) {
+        plan.dev = nullptr;
+        plan.rows = nullptr;
+        plan.host_counts = nullptr;
+    }
     constexpr int kMaxTile = 32 * DenseVec<T>::kElems >= 128 ? 128 : 32 * DenseVec<T>::kElems;
     auto padded = [n](int tn) { return (n + tn - 1) / tn * tn; };
     int best = 32;
