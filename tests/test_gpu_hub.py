@@ -94,15 +94,17 @@ def test_hub_rows_against_oracle(k, half):
         assert (np.abs(out - ref64) / np.maximum(scale, 1e-30)).max() <= 2e-6
 
 
-def test_hub_plan_through_the_c_abi():
+@pytest.mark.parametrize("k", [64, 32])
+def test_hub_plan_through_the_c_abi(k):
     """The planned entry points with a hub plan against the same calls without one; the
-    atomic fallback of SpMM (no workspace); what is refused."""
+    atomic fallback of SpMM (no workspace); what is refused.  (k = 32: rows of one 128-byte
+    tile, for which a locality plan is ignored - a hub plan and the flags are not.)"""
     import ctypes
     from gpu_common import DEV, make_csr
     from rode_amd import RoDeCSR, _lib, rode_sddmm_hip
     lib = _lib.load()
     rng = np.random.default_rng(3)
-    m, n, k = 1500, 40000, 64
+    m, n = 1500, 40000
     rp, col, val, _ = _matrix(rng, m, n, [4500, 8000, 2000])
     csr = make_csr(rp, col, val, m, n, k, locality=False)
     assert csr.plan is None
