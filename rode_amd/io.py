@@ -2,18 +2,67 @@
 padding the reference's generators apply.  (The reference's own loader,
 ``matrix_utils.h`` / ``SPC::SparseMatrix`` used at Preprocess_opt/_preprocess.cu:2,406-413,
 is missing from its tree; this covers the same step: a SuiteSparse ``.mtx`` file in,
-CSR with ascending columns out.)  Host side, numpy only.
+CSR with ascending columns out.)  Host side: a multi-threaded C++ parser
+(``rode_amd/csrc/mtx.cpp``, in the host library next to the workload generators), with a
+numpy implementation of the same rules for a tree where that library is not built.
 """
+import ctypes
 import gzip
+import os
 
 import numpy as np
 
+from . import _lib
 
-def read_matrix_market(path):
+_native = None
+
+
+def _load_native():
+    global _native
+    if _native is None:
+        if not os.path.exists(_lib.WORKLOADS_PATH):
+            _native = False
+        else:
+            lib = ctypes.CDLL(_lib.WORKLOADS_PATH)
+            lib.rode_mtx_parse.restype = ctypes.c_void_p
+            lib.rode_mtx_parse.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_int),
+                                           ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_longlong),
+                                           ctypes.c_char_p, ctypes.c_int]
+            i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
+            f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+            lib.rode_mtx_copy.argtypes = [ctypes.c_void_p, i32p, i32p, f32p]
+            lib.rode_mtx_free.argtypes = [ctypes.c_void_p]
+            _native = lib
+    return _native
+
+
+def read_matrix_market(path, native=None):
     """Read a ``coordinate`` Matrix Market file (real / integer / pattern; general,
     symmetric or skew-symmetric) and return ``(m, n, row_ptr, col, val)`` as int32 /
     float32 CSR with ascending columns per row.  Pattern files get value 1.0;
-    duplicate entries are summed; the mirrored half of a symmetric file is added."""
+    duplicate entries are summed; the mirrored half of a symmetric file is added.
+    ``native``: True / False picks the C++ or the numpy parser, None the C++ one when its
+    library is built."""
+    lib = _load_native() if native is not False else False
+    if native is True and not lib:
+        raise RuntimeError(f"{_lib.WORKLOADS_PATH} is missing: build it with `make -C rode_amd/csrc`")
+    if lib:
+        opener = gzip.open if str(path).endswith(".gz") else open
+        with opener(path, "rb") as f:
+            text = f.read()
+        m, n, nnz = ctypes.c_int(), ctypes.c_int(), ctypes.c_longlong()
+        err = ctypes.create_string_buffer(256)
+        handle = lib.rode_mtx_parse(text, len(text), ctypes.byref(m), ctypes.byref(n), ctypes.byref(nnz), err, 256)
+        if not handle:
+            raise ValueError(f"{path}: {err.value.decode()}")
+        try:
+            row_ptr = np.empty(m.value + 1, dtype=np.int32)
+            col = np.empty(nnz.value, dtype=np.int32)
+            val = np.empty(nnz.value, dtype=np.float32)
+            lib.rode_mtx_copy(handle, row_ptr, col, val)
+        finally:
+            lib.rode_mtx_free(handle)
+        return m.value, n.value, row_ptr, col, val
     opener = gzip.open if str(path).endswith(".gz") else open
     with opener(path, "rt") as f:
         header = f.readline().strip().split()
@@ -30,7 +79,7 @@ def read_matrix_market(path):
         while line.startswith("%") or not line.strip():
             line = f.readline()
         m, n, entries = (int(t) for t in line.split()[:3])
-        data = np.loadtxt(f, dtype=np.float64, ndmin=2) if entries else np.zeros((0, 3))
+        data = np.loadtxt(f, dtype=np.float64, ndmin=2, comments="%") if entries else np.zeros((0, 3))
     if data.shape[0] != entries:
         raise ValueError(f"{path}: header promises {entries} entries, file has {data.shape[0]}")
     rows = data[:, 0].astype(np.int64) - 1

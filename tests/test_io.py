@@ -20,6 +20,14 @@ def _same(csr, ref):
     np.testing.assert_allclose(val, ref.data.astype(np.float32), rtol=1e-6)
 
 
+@pytest.fixture(params=[True, False], ids=["cxx", "numpy"], autouse=True)
+def parser(request, monkeypatch):
+    """Every test of the reader runs with the C++ parser and with the numpy one."""
+    read = rio.read_matrix_market
+    monkeypatch.setattr(rio, "read_matrix_market", lambda path, native=None: read(path, native=request.param))
+    return request.param
+
+
 @pytest.mark.parametrize("symmetry", ["general", "symmetric", "skew-symmetric"])
 def test_reads_what_scipy_reads(tmp_path, symmetry):
     rng = np.random.default_rng(0)
@@ -45,6 +53,24 @@ def test_pattern_rectangular_duplicates_and_gzip(tmp_path):
     empty.write_text("%%MatrixMarket matrix coordinate real general\n4 4 0\n")
     m, n, rp, col, val = rio.read_matrix_market(empty)
     assert rp.tolist() == [0] * 5 and len(col) == 0
+
+
+def test_large_file_in_parallel_pieces(tmp_path, parser):
+    """Several hundred thousand entries (the C++ parser cuts the text into one piece per
+    thread), integer field, exponent notation, CRLF line ends, a comment between entries."""
+    rng = np.random.default_rng(3)
+    m, n, e = 5000, 7000, 300000 if parser else 20000
+    rows, cols = rng.integers(1, m + 1, e), rng.integers(1, n + 1, e)
+    vals = rng.integers(-50, 50, e)
+    lines = [f"{r} {c} {v}" for r, c, v in zip(rows, cols, vals)]
+    lines.insert(e // 2, "% a comment in the middle")
+    path = tmp_path / "big.mtx"
+    path.write_bytes(("%%MatrixMarket matrix coordinate integer general\r\n" + f"{m} {n} {e}\r\n" + "\r\n".join(lines) + "\r\n").encode())
+    _same(rio.read_matrix_market(path), sp.coo_matrix((vals.astype(np.float64), (rows - 1, cols - 1)), shape=(m, n)))
+    small = tmp_path / "exp.mtx"
+    small.write_text("%%MatrixMarket matrix coordinate real general\n2 2 2\n1 2 1.5e+01\n2 1 -2.5E-1\n")
+    mm, nn, rp, col, val = rio.read_matrix_market(small)
+    assert rp.tolist() == [0, 1, 2] and col.tolist() == [1, 0] and val.tolist() == [15.0, -0.25]
 
 
 def test_rejects_bad_files(tmp_path):
