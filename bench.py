@@ -137,7 +137,6 @@ def main():
     cfg = "auto" if args.seg == 0 else None if args.seg < 0 else {"seg_length": args.seg, "k_block": 32, "vec_len": 4}
     csr = RoDeCSR(torch.from_numpy(row_ptr), torch.from_numpy(col), torch.from_numpy(val), dev, m, n,
                   k if k in RoDeCSR.CONFIGS else 128, config=cfg, locality=False if args.no_plan else "auto")
-    plan_args = rode_sddmm_hip._plan_args(csr.plan)
     gen = torch.Generator(device=dev).manual_seed(3000)
     B = torch.randn(n, k, device=dev, generator=gen).to(tdtype)     # SpMM dense operand, also SDDMM rhs
     L = torch.randn(m, k, device=dev, generator=gen).to(tdtype)     # SDDMM lhs
@@ -146,16 +145,17 @@ def main():
     setup_s = time.time() - t0
 
     stream = torch.cuda.current_stream().cuda_stream
+    import ctypes
     hub = csr.plan if isinstance(csr.plan, rode_sddmm_hip.HubPlan) else None
-    hub_ws = hub.workspace(k, 4) if hub is not None else None
+    spmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan, k, 4))
+    sddmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan))
 
     def spmm_fn(*a, flags=0):  # the whole decomposition is passed, and the library is told so
         return lib.rode_hip_spmm_planned(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS | flags, *a[:-2],
-                                         *plan_args, hub_ws.data_ptr() if hub is not None else None,
-                                         hub_ws.numel() if hub is not None else 0, *a[-2:])
+                                         spmm_plans, *a[-2:])
 
     def sddmm_fn(*a, flags=0):
-        return lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[args.dtype], flags, *a[:-2], *plan_args, *a[-2:])
+        return lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[args.dtype], flags, *a[:-2], sddmm_plans, *a[-2:])
 
     main_stream = torch.cuda.current_stream()
     side = torch.cuda.Stream() if args.two_streams else None

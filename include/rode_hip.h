@@ -211,25 +211,40 @@ int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_
                       const int* d_column_indices, void* d_plan, size_t plan_bytes, int* h_counts, void* stream);
 
 /*
- * rode_hip_spmm_ex with a plan.  d_plan / d_plan_rows: both parts of a locality plan made
- * from these lists, or NULL.  h_plan_counts: NULL, or the HOST int[4] header that
- * rode_hip_window_plan returned; with it, kernels that would find no chunk to work on are
- * not launched at all.  fp64 operands, and dense rows of at most 128 bytes, ignore the
- * locality plan.  d_hub_plan / h_hub_counts: a hub plan of this matrix and its header, or
- * NULL; it needs RODE_SPMM_WHOLE_LISTS (the hub kernels replace work items of both lists).
- * d_hub_workspace: rode_hip_hub_workspace_bytes(h_hub_counts,
- * n, 4 or 8) bytes of scratch, 16-byte aligned, that the hub kernels of this call may write
- * and read (one partial row of C per hub row and slab, summed by a second kernel), or NULL:
- * the pieces are then added to C atomically, which is slower for wide rows.  With every
- * plan pointer NULL: exactly rode_hip_spmm_ex.
+ * The plans of one matrix, as the *_planned entry points take them: a struct in HOST
+ * memory, read during the call only.  Every member may be NULL / 0; a struct of zeros (or
+ * a NULL struct pointer) makes the planned calls exactly the unplanned ones.
+ *   window, window_rows   both parts of a locality plan made from the lists of the call
+ *   window_counts         NULL, or the HOST int[4] header rode_hip_window_plan returned;
+ *                         with it, kernels that would find no chunk to work on are not
+ *                         launched at all.  fp64 operands, and dense rows of at most 128
+ *                         bytes, ignore the locality plan.
+ *   hub, hub_counts       a hub plan of this matrix and its HOST int[8] header (required
+ *                         with it).  Needs the complete decomposition: for SpMM the
+ *                         RODE_SPMM_WHOLE_LISTS promise, for SDDMM simply whole lists.
+ *                         Excludes a locality plan.
+ *   hub_workspace, hub_workspace_bytes   SpMM only: rode_hip_hub_workspace_bytes(hub_counts,
+ *                         n, 4 or 8) bytes of scratch, 16-byte aligned, that the hub kernels
+ *                         of this call may write and read (one partial row of C per hub
+ *                         row and slab group, summed by a second kernel), or NULL: the
+ *                         pieces are then added to C atomically, slower for wide rows.
  * Same results as without a plan, up to the order of the fp32 additions inside a row.
  */
+typedef struct rode_hip_plans {
+    const void* window;
+    const void* window_rows;
+    const int* window_counts;
+    const void* hub;
+    const int* hub_counts;
+    void* hub_workspace;
+    size_t hub_workspace_bytes;
+} rode_hip_plans;
+
+/* rode_hip_spmm_ex with plans. */
 int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                           const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                           const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
-                          const void* d_plan, const void* d_plan_rows, const int* h_plan_counts,
-                          const void* d_hub_plan, const int* h_hub_counts, void* d_hub_workspace,
-                          size_t hub_workspace_bytes, void* stream1, void* stream2);
+                          const rode_hip_plans* plans, void* stream1, void* stream2);
 
 /*
  * Prepares an uninitialised C[M x n] for one of the SpMM calls: zeroes exactly the rows
@@ -279,10 +294,8 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
                        const void* d_rhs_half, float* d_out, void* stream1, void* stream2);
 
 /*
- * SDDMM with a plan: dtype RODE_DENSE_F32 or RODE_DENSE_F16 selects the element type of
- * lhs / rhs; d_plan / d_plan_rows / h_plan_counts and d_hub_plan / h_hub_counts as for
- * rode_hip_spmm_planned (all NULL: exactly the typed functions above).  With a hub plan the
- * lists must be the complete decomposition (the hub kernels replace work items of both).
+ * SDDMM with plans: dtype RODE_DENSE_F32 or RODE_DENSE_F16 selects the element type of
+ * lhs / rhs; plans as for rode_hip_spmm_planned (NULL: exactly the typed functions above).
  * flags: 0, or one of the RODE_SPMM_ONLY_* bits (one kernel family of the call).
  * Same results up to the order of the fp32 additions of a dot product.  No counterpart in
  * the reference.
@@ -290,8 +303,7 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
 int rode_hip_sddmm_planned(int dtype, int flags, int m1, int m2, int n, int k, const int* d_row_indices_block,
                            const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                            const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
-                           const void* d_rhs_matrix, float* d_out, const void* d_plan, const void* d_plan_rows,
-                           const int* h_plan_counts, const void* d_hub_plan, const int* h_hub_counts, void* stream1,
+                           const void* d_rhs_matrix, float* d_out, const rode_hip_plans* plans, void* stream1,
                            void* stream2);
 
 /*

@@ -31,17 +31,24 @@ SIGNATURES = {
     "rode_hip_hub_plan_bytes": (c_size_t, [c_int] * 4),
     "rode_hip_hub_plan": (c_int, [c_int] * 4 + [c_void_p] * 3 + [c_size_t, c_void_p, c_void_p]),
     "rode_hip_hub_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
-    "rode_hip_spmm_planned": (c_int, [c_int] * 6 + [c_void_p] * 14 + [c_size_t] + [c_void_p] * 2),
+    "rode_hip_spmm_planned": (c_int, [c_int] * 6 + [c_void_p] * 11),
     "rode_hip_spmm_clear_rows": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "rode_hip_sddmm_f32": (c_int, [c_int] * 4 + [c_void_p] * 11),
     "rode_hip_sddmm_f16": (c_int, [c_int] * 4 + [c_void_p] * 11),
-    "rode_hip_sddmm_planned": (c_int, [c_int] * 6 + [c_void_p] * 16),
+    "rode_hip_sddmm_planned": (c_int, [c_int] * 6 + [c_void_p] * 12),
     "rode_hip_csr_softmax_f32": (c_int, [c_int, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_void_p]),
     "rode_hip_csr_softmax_backward_f32": (c_int, [c_int] + [c_void_p] * 4 + [ctypes.c_float, c_void_p]),
     "rode_hip_csr_transpose_workspace_bytes": (c_size_t, [c_int]),
     "rode_hip_csr_transpose": (c_int, [c_int] * 3 + [c_void_p] * 6 + [c_size_t, c_void_p]),
     "rode_hip_attention_forward": (c_int, [c_int] * 3 + [c_void_p] * 6 + [ctypes.c_float] + [c_void_p] * 3),
 }
+
+class Plans(ctypes.Structure):
+    """``rode_hip_plans`` of include/rode_hip.h."""
+    _fields_ = [("window", c_void_p), ("window_rows", c_void_p), ("window_counts", c_void_p),
+                ("hub", c_void_p), ("hub_counts", c_void_p), ("hub_workspace", c_void_p),
+                ("hub_workspace_bytes", c_size_t)]
+
 
 DENSE_CODE = {"f32": 0, "f16": 1, "f64": 2}  # RODE_DENSE_* of include/rode_hip.h
 SPMM_WHOLE_LISTS, SPMM_ONLY_BLOCK, SPMM_ONLY_RESIDUE, SPMM_ONLY_HUB = 1, 2, 4, 8  # RODE_SPMM_* flags

@@ -158,25 +158,30 @@ size_t rode_hip_hub_workspace_bytes(const int* h_hub_counts, int n, int elem_byt
 
 namespace {
 // The caller's plans as the launchers take them; false if they cannot belong to these lists.
-bool plan_ref(const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, const void* d_hub_plan,
-              const int* h_hub_counts, int m2, rode::PlanRef& plan)
+bool plan_ref(const rode_hip_plans* p, int m2, rode::PlanRef& plan)
 {
-    if (d_hub_plan) {
+    if (!p) return true;
+    const bool window = p->window && p->window_rows; // (one without rows: the standard kernels do everything)
+    if (p->hub) {
         // a hub plan needs its header on the host, and excludes a locality plan (the window
         // kernels do not know which rows the hub kernels have taken)
-        if (!h_hub_counts || !aligned16(d_hub_plan) || (d_plan && d_plan_rows)) return false;
-        if (h_hub_counts[0] < 0 || h_hub_counts[0] > h_hub_counts[4] || h_hub_counts[1] < 0 ||
-            h_hub_counts[2] < RODE_HIP_HUB_MIN_LEN)
+        if (!p->hub_counts || !aligned16(p->hub) || window) return false;
+        if (p->hub_counts[0] < 0 || p->hub_counts[0] > p->hub_counts[4] || p->hub_counts[1] < 0 ||
+            p->hub_counts[2] < RODE_HIP_HUB_MIN_LEN)
             return false;
-        plan.hub = static_cast<const int*>(d_hub_plan);
-        plan.hub_counts = h_hub_counts;
+        plan.hub = static_cast<const int*>(p->hub);
+        plan.hub_counts = p->hub_counts;
+        if (p->hub_workspace && aligned16(p->hub_workspace)) {
+            plan.hub_workspace = p->hub_workspace;
+            plan.hub_workspace_bytes = p->hub_workspace_bytes;
+        }
     }
-    if (!d_plan || !d_plan_rows) return true; // no plan, or one without rows: the standard kernels do everything
-    if (!aligned16(d_plan) || !aligned16(d_plan_rows)) return false;
-    if (h_plan_counts && h_plan_counts[0] != rode::plan_residue_chunks(m2)) return false;
-    plan.dev = static_cast<const int*>(d_plan);
-    plan.rows = d_plan_rows;
-    plan.host_counts = h_plan_counts;
+    if (!window) return true;
+    if (!aligned16(p->window) || !aligned16(p->window_rows)) return false;
+    if (p->window_counts && p->window_counts[0] != rode::plan_residue_chunks(m2)) return false;
+    plan.dev = static_cast<const int*>(p->window);
+    plan.rows = p->window_rows;
+    plan.host_counts = p->window_counts;
     return true;
 }
 } // namespace
@@ -187,16 +192,13 @@ int rode_hip_spmm_ex(int dtype, int flags, int m1, int m2, int k, int n, const v
                      void* stream1, void* stream2)
 {
     return rode_hip_spmm_planned(dtype, flags, m1, m2, k, n, d_values, d_column_indices, d_row_offsets, d_row_indices1,
-                                 d_row_indices2, d_row_seg_st_offsets, d_B, d_C, nullptr, nullptr, nullptr, nullptr, nullptr,
-                                 nullptr, 0, stream1, stream2);
+                                 d_row_indices2, d_row_seg_st_offsets, d_B, d_C, nullptr, stream1, stream2);
 }
 
 int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, const void* d_values,
                           const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                           const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
-                          const void* d_plan, const void* d_plan_rows, const int* h_plan_counts, const void* d_hub_plan,
-                          const int* h_hub_counts, void* d_hub_workspace, size_t hub_workspace_bytes, void* stream1,
-                          void* stream2)
+                          const rode_hip_plans* plans, void* stream1, void* stream2)
 {
     (void)k;
     constexpr int kKnown = RODE_SPMM_WHOLE_LISTS | RODE_SPMM_ONLY_BLOCK | RODE_SPMM_ONLY_RESIDUE | RODE_SPMM_ONLY_HUB;
@@ -210,13 +212,9 @@ int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, co
     if (!aligned16(d_B) || !aligned16(d_C)) return hipErrorInvalidValue;
     hipStream_t s1 = as_stream(stream1), s2 = as_stream(stream2);
     rode::PlanRef plan;
-    if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, d_hub_plan, h_hub_counts, m2, plan)) return hipErrorInvalidValue;
+    if (!plan_ref(plans, m2, plan)) return hipErrorInvalidValue;
     // the hub kernels replace work items of both lists: only with the complete decomposition
     if (plan.hub && !(flags & RODE_SPMM_WHOLE_LISTS)) return hipErrorInvalidValue;
-    if (plan.hub && d_hub_workspace && aligned16(d_hub_workspace)) {
-        plan.hub_workspace = d_hub_workspace;
-        plan.hub_workspace_bytes = hub_workspace_bytes;
-    }
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,
@@ -271,8 +269,7 @@ int rode_hip_spmm_f16(int m1, int m2, int k, int n, const float* d_values, const
 int rode_hip_sddmm_planned(int dtype, int flags, int m1, int m2, int n, int k, const int* d_row_indices_block,
                            const int* d_row_indices_residue, const int* d_st_offsets, const int* d_row_offsets,
                            const int* d_column_indices, const float* d_values, const void* d_lhs_matrix,
-                           const void* d_rhs_matrix, float* d_out, const void* d_plan, const void* d_plan_rows,
-                           const int* h_plan_counts, const void* d_hub_plan, const int* h_hub_counts, void* stream1,
+                           const void* d_rhs_matrix, float* d_out, const rode_hip_plans* plans, void* stream1,
                            void* stream2)
 {
     (void)n;
@@ -280,7 +277,7 @@ int rode_hip_sddmm_planned(int dtype, int flags, int m1, int m2, int n, int k, c
     if (m1 == 0 && m2 == 0) return hipSuccess;
     if (!aligned16(d_lhs_matrix) || !aligned16(d_rhs_matrix)) return hipErrorInvalidValue;
     rode::PlanRef plan;
-    if (!plan_ref(d_plan, d_plan_rows, h_plan_counts, d_hub_plan, h_hub_counts, m2, plan)) return hipErrorInvalidValue;
+    if (!plan_ref(plans, m2, plan)) return hipErrorInvalidValue;
     plan.only = flags;
     switch (dtype) {
     case RODE_DENSE_F32:
@@ -305,7 +302,7 @@ int rode_hip_sddmm_f32(int m1, int m2, int n, int k, const int* d_row_indices_bl
 {
     return rode_hip_sddmm_planned(RODE_DENSE_F32, 0, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
                                   d_row_offsets, d_column_indices, d_values, d_lhs_matrix, d_rhs_matrix, d_out, nullptr,
-                                  nullptr, nullptr, nullptr, nullptr, stream1, stream2);
+                                  stream1, stream2);
 }
 
 int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_block, const int* d_row_indices_residue,
@@ -315,7 +312,7 @@ int rode_hip_sddmm_f16(int m1, int m2, int n, int k, const int* d_row_indices_bl
 {
     return rode_hip_sddmm_planned(RODE_DENSE_F16, 0, m1, m2, n, k, d_row_indices_block, d_row_indices_residue, d_st_offsets,
                                   d_row_offsets, d_column_indices, d_values, d_lhs_half, d_rhs_half, d_out, nullptr,
-                                  nullptr, nullptr, nullptr, nullptr, stream1, stream2);
+                                  stream1, stream2);
 }
 
 int rode_hip_csr_softmax_f32(int M, const int* d_row_offsets, const float* d_in, float* d_out, float scale,

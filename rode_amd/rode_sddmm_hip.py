@@ -207,25 +207,22 @@ def hub_plan(row_offsets, column_indices, m, n, min_len):
     return HubPlan(data, list(counts))
 
 
-def _spmm_plan_args(plan, whole_lists, n, out):
-    """The seven plan arguments of ``rode_hip_spmm_planned``: those of ``_plan_args`` and
-    the hub kernels' workspace."""
-    if isinstance(plan, HubPlan) and plan.usable and whole_lists:
-        ws = plan.workspace(n, out.element_size())
-        return (*_plan_args(plan), ws.data_ptr(), ws.numel())
-    return (*_plan_args(None if isinstance(plan, HubPlan) else plan), None, 0)
-
-
-def _plan_args(plan):
-    """The five plan arguments of the ``*_planned`` entry points: locality plan (descriptors,
-    rows, host header), hub plan (array, host header)."""
+def plans_struct(plan, spmm_width=None, spmm_elem_bytes=4, whole_lists=True):
+    """The ``rode_hip_plans`` struct of one call (keep it alive until the call returns; pass
+    it with ``ctypes.byref``).  ``plan``: a ``WindowPlan``, a ``HubPlan`` or None.
+    ``spmm_width``: for an SpMM call the dense width, so that a hub plan's workspace is
+    attached; a hub plan is left out of an SpMM call without the whole-lists promise."""
+    p = _lib.Plans()
     if isinstance(plan, HubPlan):
-        if not plan.usable:
-            return None, None, None, None, None
-        return None, None, None, plan.data.data_ptr(), ctypes.addressof(plan._header)
-    if plan is None or plan.rows is None:
-        return None, None, None, None, None
-    return plan.data.data_ptr(), plan.rows.data_ptr(), ctypes.addressof(plan._header), None, None
+        if plan.usable and (spmm_width is None or whole_lists):
+            p.hub, p.hub_counts = plan.data.data_ptr(), ctypes.addressof(plan._header)
+            if spmm_width is not None:
+                ws = plan.workspace(spmm_width, spmm_elem_bytes)
+                p.hub_workspace, p.hub_workspace_bytes = ws.data_ptr(), ws.numel()
+    elif plan is not None and plan.rows is not None:
+        p.window, p.window_rows = plan.data.data_ptr(), plan.rows.data_ptr()
+        p.window_counts = ctypes.addressof(plan._header)
+    return p
 
 
 def preprocess(row_offsets, nnz, seg_length, k_block, vec_len):
@@ -285,10 +282,11 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
     lib = _lib.load()
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
+        plans = plans_struct(plan)
         code = lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[kind], 0, m1, m2, n, k, block_indices.data_ptr(),
                                           residue_indices.data_ptr(), st_offsets.data_ptr(), row_offsets.data_ptr(),
                                           column_indices.data_ptr(), values.data_ptr(), lhs_matrix.data_ptr(),
-                                          rhs_matrix.data_ptr(), out.data_ptr(), *_plan_args(plan), s, s)
+                                          rhs_matrix.data_ptr(), out.data_ptr(), ctypes.byref(plans), s, s)
     _lib.check(code, "rode_hip_sddmm_planned")
     return out
 
@@ -339,10 +337,10 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     dtype = {torch.float32: 0, torch.float16: 1, torch.float64: 2}[dense_matrix.dtype]  # RODE_DENSE_*
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
+        plans = plans_struct(plan, n, out.element_size(), whole_lists)
         code = lib.rode_hip_spmm_planned(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
                                          values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
                                          block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
-                                         dense_matrix.data_ptr(), out.data_ptr(), *_spmm_plan_args(plan, whole_lists, n, out),
-                                         s, s)
+                                         dense_matrix.data_ptr(), out.data_ptr(), ctypes.byref(plans), s, s)
     _lib.check(code, "rode_hip_spmm_planned")
     return out

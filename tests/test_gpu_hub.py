@@ -112,16 +112,23 @@ def test_hub_plan_through_the_c_abi(k):
     assert plan.usable and plan.counts[0] == 3
     B = torch.from_numpy(rng.standard_normal((n, k)).astype(np.float32)).to(DEV)
     L = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(DEV)
-    hub_args = (plan.data.data_ptr(), ctypes.addressof(plan._header))
+
+    def plans(hub, ws=None, window=None):
+        p = _lib.Plans()
+        if hub:
+            p.hub, p.hub_counts = plan.data.data_ptr(), ctypes.addressof(plan._header)
+        if ws is not None:
+            p.hub_workspace, p.hub_workspace_bytes = ws.data_ptr(), ws.numel()
+        if window is not None:
+            p.window, p.window_rows = window.data_ptr(), window.data_ptr()
+        return p
 
     def spmm(flags, hub, ws):
         C = torch.zeros(m, k, device=DEV)
         code = lib.rode_hip_spmm_planned(0, flags, csr.m1, csr.m2, n, k, csr.values.data_ptr(), csr.column_indices.data_ptr(),
                                          csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(),
                                          csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(), B.data_ptr(),
-                                         C.data_ptr(), None, None, None, *(hub_args if hub else (None, None)),
-                                         ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-                                         None, None)
+                                         C.data_ptr(), ctypes.byref(plans(hub, ws)), None, None)
         torch.cuda.synchronize()
         return code, C
 
@@ -141,13 +148,13 @@ def test_hub_plan_through_the_c_abi(k):
     assert spmm(0, True, ws)[0] != 0
     assert spmm(_lib.SPMM_WHOLE_LISTS | _lib.SPMM_ONLY_BLOCK | _lib.SPMM_ONLY_HUB, True, ws)[0] != 0
 
-    def sddmm(flags, hub, window=(None, None, None)):
+    def sddmm(flags, hub, window=None):
         out = torch.full((len(val),), float("nan"), device=DEV)
         code = lib.rode_hip_sddmm_planned(0, flags, csr.m1, csr.m2, n, k, csr.block_indices.data_ptr(),
                                           csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(),
                                           csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
-                                          L.data_ptr(), B.data_ptr(), out.data_ptr(), *window,
-                                          *(hub_args if hub else (None, None)), None, None)
+                                          L.data_ptr(), B.data_ptr(), out.data_ptr(), ctypes.byref(plans(hub, None, window)),
+                                          None, None)
         torch.cuda.synchronize()
         return code, out
 
@@ -159,4 +166,4 @@ def test_hub_plan_through_the_c_abi(k):
     written = [~torch.isnan(sddmm(f, True)[1]) for f in (_lib.SPMM_ONLY_BLOCK, _lib.SPMM_ONLY_RESIDUE, _lib.SPMM_ONLY_HUB)]
     assert (written[0].int() + written[1].int() + written[2].int() == 1).all()
     fake = torch.zeros(64, dtype=torch.int32, device=DEV)
-    assert sddmm(0, True, (fake.data_ptr(), fake.data_ptr(), None))[0] != 0
+    assert sddmm(0, True, fake)[0] != 0
