@@ -211,6 +211,26 @@ int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_
                       const int* d_column_indices, void* d_plan, size_t plan_bytes, int* h_counts, void* stream);
 
 /*
+ * Group plan (no counterpart in the reference either).  For matrices whose adjacent rows
+ * share long runs of consecutive column indices (sliding-window attention masks, dense
+ * bands, block structure): groups of RODE_HIP_GROUP_ROWS adjacent rows whose common run
+ * has at least 64 columns and holds at least three quarters of their nonzeros are
+ * processed by kernels of their own, which load every dense row of the run once for all
+ * rows of the group (and compute its address instead of reading column indices).  The
+ * other kernels leave those rows out.  Same results up to the order of the fp32 additions.
+ *   d_plan       rode_hip_group_plan_bytes(M) bytes, 16-byte aligned, out
+ *   h_counts     HOST int[4], out (the call waits for its kernels): [0] groups (M / 4,
+ *                whole groups only), [1] groups with a run; the *_planned entry points
+ *                need it and ignore a plan with [1] == 0
+ * A group plan belongs to the pattern it was made from and excludes the other two plans.
+ * SDDMM uses it for k <= 128 (fp32) / 256 (fp16) elements, SpMM for any width.
+ */
+#define RODE_HIP_GROUP_ROWS 4
+size_t rode_hip_group_plan_bytes(int M);
+int rode_hip_group_plan(int M, const int* d_row_offsets, const int* d_column_indices, void* d_plan, size_t plan_bytes,
+                        int* h_counts, void* stream);
+
+/*
  * The plans of one matrix, as the *_planned entry points take them: a struct in HOST
  * memory, read during the call only.  Every member may be NULL / 0; a struct of zeros (or
  * a NULL struct pointer) makes the planned calls exactly the unplanned ones.
@@ -228,6 +248,9 @@ int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_
  *                         of this call may write and read (one partial row of C per hub
  *                         row and slab group, summed by a second kernel), or NULL: the
  *                         pieces are then added to C atomically, slower for wide rows.
+ *   groups, group_counts  a group plan of this matrix and its HOST int[4] header (required
+ *                         with it).  Needs the complete decomposition, like a hub plan,
+ *                         and excludes both other plans.
  * Same results as without a plan, up to the order of the fp32 additions inside a row.
  */
 typedef struct rode_hip_plans {
@@ -238,6 +261,8 @@ typedef struct rode_hip_plans {
     const int* hub_counts;
     void* hub_workspace;
     size_t hub_workspace_bytes;
+    const void* groups;
+    const int* group_counts;
 } rode_hip_plans;
 
 /* rode_hip_spmm_ex with plans. */

@@ -28,6 +28,8 @@ SIGNATURES = {
     "rode_hip_window_plan": (c_int, [c_int] * 2 + [c_void_p] * 4 + [c_size_t, c_void_p, c_void_p]),
     "rode_hip_window_rows_bytes": (c_size_t, [c_int]),
     "rode_hip_window_rows": (c_int, [c_int] + [c_void_p] * 5 + [c_size_t, c_void_p]),
+    "rode_hip_group_plan_bytes": (c_size_t, [c_int]),
+    "rode_hip_group_plan": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "rode_hip_hub_plan_bytes": (c_size_t, [c_int] * 4),
     "rode_hip_hub_plan": (c_int, [c_int] * 4 + [c_void_p] * 3 + [c_size_t, c_void_p, c_void_p]),
     "rode_hip_hub_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
@@ -47,7 +49,7 @@ class Plans(ctypes.Structure):
     """``rode_hip_plans`` of include/rode_hip.h."""
     _fields_ = [("window", c_void_p), ("window_rows", c_void_p), ("window_counts", c_void_p),
                 ("hub", c_void_p), ("hub_counts", c_void_p), ("hub_workspace", c_void_p),
-                ("hub_workspace_bytes", c_size_t)]
+                ("hub_workspace_bytes", c_size_t), ("groups", c_void_p), ("group_counts", c_void_p)]
 
 
 DENSE_CODE = {"f32": 0, "f16": 1, "f64": 2}  # RODE_DENSE_* of include/rode_hip.h

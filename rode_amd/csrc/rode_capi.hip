@@ -156,12 +156,34 @@ size_t rode_hip_hub_workspace_bytes(const int* h_hub_counts, int n, int elem_byt
     return (size_t)h_hub_counts[0] * rode::hub_groups(h_hub_counts[1], merge) * n * elem_bytes;
 }
 
+size_t rode_hip_group_plan_bytes(int M) { return M < 0 ? 0 : rode::group_plan_ints(M) * sizeof(int); }
+
+int rode_hip_group_plan(int M, const int* d_row_offsets, const int* d_column_indices, void* d_plan, size_t plan_bytes,
+                        int* h_counts, void* stream)
+{
+    if (M < 0 || !d_plan || !aligned16(d_plan) || !h_counts || plan_bytes < rode_hip_group_plan_bytes(M))
+        return hipErrorInvalidValue;
+    if (M > 0 && (!d_row_offsets || !d_column_indices)) return hipErrorInvalidValue;
+    hipError_t e = rode::group_plan_launch(M, d_row_offsets, d_column_indices, static_cast<int*>(d_plan), as_stream(stream));
+    if (e == hipSuccess) e = hipMemcpyAsync(h_counts, d_plan, 4 * sizeof(int), hipMemcpyDeviceToHost, as_stream(stream));
+    if (e == hipSuccess) e = hipStreamSynchronize(as_stream(stream));
+    return e;
+}
+
 namespace {
 // The caller's plans as the launchers take them; false if they cannot belong to these lists.
 bool plan_ref(const rode_hip_plans* p, int m2, rode::PlanRef& plan)
 {
     if (!p) return true;
     const bool window = p->window && p->window_rows; // (one without rows: the standard kernels do everything)
+    if (p->groups) {
+        // a group plan needs its header on the host, and excludes the other plans (their
+        // kernels do not know which rows the group kernels have taken)
+        if (!p->group_counts || !aligned16(p->groups) || window || p->hub) return false;
+        if (p->group_counts[0] < 0 || p->group_counts[1] < 0 || p->group_counts[1] > p->group_counts[0]) return false;
+        plan.groups = static_cast<const int*>(p->groups);
+        plan.group_counts = p->group_counts;
+    }
     if (p->hub) {
         // a hub plan needs its header on the host, and excludes a locality plan (the window
         // kernels do not know which rows the hub kernels have taken)
@@ -213,8 +235,8 @@ int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, co
     hipStream_t s1 = as_stream(stream1), s2 = as_stream(stream2);
     rode::PlanRef plan;
     if (!plan_ref(plans, m2, plan)) return hipErrorInvalidValue;
-    // the hub kernels replace work items of both lists: only with the complete decomposition
-    if (plan.hub && !(flags & RODE_SPMM_WHOLE_LISTS)) return hipErrorInvalidValue;
+    // the hub and group kernels replace work items of both lists: only with the complete decomposition
+    if ((plan.hub || plan.groups) && !(flags & RODE_SPMM_WHOLE_LISTS)) return hipErrorInvalidValue;
     switch (dtype) {
     case RODE_DENSE_F32:
         return rode::spmm_launch<float>(m1, m2, n, d_row_indices1, d_row_indices2, d_row_seg_st_offsets, d_row_offsets,

@@ -1,0 +1,106 @@
+// Group plan: groups of kGroupRows adjacent rows that share a long run of consecutive
+// column indices (sliding-window attention masks, dense bands, block structure).  The
+// group kernels (spmm_group_kernel, sddmm_group_kernel) walk the shared run once for all
+// rows of a group: one gather of a dense row serves every row of the group, and the dense
+// rows of a run are consecutive in memory, so no column index is read for them.  The
+// nonzeros of a row outside the run are processed as usual, by the same workgroup; the
+// standard kernels leave grouped rows out.  No counterpart in the reference, whose kernels
+// gather the dense row of every nonzero of every row (RoDe_SpMM/RoDeSpmm.cu:140-160,
+// RoDe_SDDMM/RoDeSddmm.cu:96-140).  The plan changes no result.
+//
+//   group_runs_kernel   per row: its longest run of consecutive columns (first column,
+//                       length, position in the row); one thread per row.
+//   group_desc_kernel   per group: the intersection of its rows' runs; the group is kept
+//                       if that run has at least kGroupMinRun columns and holds at least
+//                       three quarters of the group's nonzeros.
+#include "rode_items.hpp"
+#include "rode_internal.hpp"
+
+namespace rode {
+
+namespace {
+
+constexpr int kGroupMinRun = 64;
+
+__global__ void __launch_bounds__(kWgThreads)
+group_runs_kernel(int M, const int* __restrict__ row_ptr, const int* __restrict__ col, int* __restrict__ runs)
+{
+    const int row = blockIdx.x * kWgThreads + threadIdx.x;
+    if (row >= M) return;
+    const int s = row_ptr[row], e = row_ptr[row + 1];
+    int best_first = 0, best_len = 0, best_pos = 0;
+    int first = 0, len = 0, pos = 0, prev = -2;
+    for (int i = s; i < e; ++i) {
+        const int c = col[i];
+        if (c == prev + 1) {
+            ++len;
+        } else {
+            first = c;
+            len = 1;
+            pos = i - s;
+        }
+        if (len > best_len) {
+            best_first = first;
+            best_len = len;
+            best_pos = pos;
+        }
+        prev = c;
+    }
+    runs[3 * row] = best_first;
+    runs[3 * row + 1] = best_len;
+    runs[3 * row + 2] = best_pos;
+}
+
+__global__ void __launch_bounds__(kWgThreads)
+group_desc_kernel(int groups, const int* __restrict__ row_ptr, const int* __restrict__ runs, int* __restrict__ plan)
+{
+    const int g = blockIdx.x * kWgThreads + threadIdx.x;
+    if (g >= groups) return;
+    RowGroup d;
+    int lo = 0, hi = 0x7fffffff;
+    long long slots = 0;
+#pragma unroll
+    for (int r = 0; r < kGroupRows; ++r) {
+        const int row = g * kGroupRows + r;
+        lo = max(lo, runs[3 * row]);
+        hi = min(hi, runs[3 * row] + runs[3 * row + 1]);
+        slots += row_ptr[row + 1] - row_ptr[row];
+    }
+    const int len = hi - lo;
+    const bool keep = len >= kGroupMinRun && 4ll * kGroupRows * len >= 3 * slots;
+    d.lo = keep ? lo : 0;
+    d.len = keep ? len : 0;
+#pragma unroll
+    for (int r = 0; r < kGroupRows; ++r) {
+        const int row = g * kGroupRows + r;
+        d.pos[r] = keep ? runs[3 * row + 2] + (lo - runs[3 * row]) : 0;
+    }
+    d.reserved[0] = d.reserved[1] = 0;
+    reinterpret_cast<RowGroup*>(plan + kGroupHeaderInts)[g] = d;
+    if (keep) atomicAdd(plan + 1, 1);
+}
+
+__global__ void group_header_kernel(int groups, int* __restrict__ plan)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        plan[0] = groups;
+        plan[1] = 0;
+        for (int i = 2; i < kGroupHeaderInts; ++i) plan[i] = 0;
+    }
+}
+
+} // namespace
+
+hipError_t group_plan_launch(int M, const int* row_ptr, const int* col, int* plan, hipStream_t stream)
+{
+    const int groups = row_groups(M);
+    group_header_kernel<<<1, kWave, 0, stream>>>(groups, plan);
+    if (groups > 0) {
+        int* runs = plan + kGroupHeaderInts + (size_t)groups * (sizeof(RowGroup) / sizeof(int)); // scratch behind the table
+        group_runs_kernel<<<(M + kWgThreads - 1) / kWgThreads, kWgThreads, 0, stream>>>(M, row_ptr, col, runs);
+        group_desc_kernel<<<(groups + kWgThreads - 1) / kWgThreads, kWgThreads, 0, stream>>>(groups, row_ptr, runs, plan);
+    }
+    return hipGetLastError();
+}
+
+} // namespace rode

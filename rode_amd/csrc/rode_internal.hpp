@@ -38,9 +38,14 @@ struct PlanRef {
     // SpMM only: room for one partial row of C per (slab, hub row), or null (atomics instead).
     void* hub_workspace = nullptr;
     size_t hub_workspace_bytes = 0;
+    // A group plan (rode_group.hip) and the host copy of its four header ints (required with it).
+    const int* groups = nullptr;
+    const int* group_counts = nullptr;
     // SDDMM: the RODE_SPMM_ONLY_* bits of the call (SpMM carries them in its flags)
     int only = 0;
 };
+
+hipError_t group_plan_launch(int M, const int* row_ptr, const int* col, int* plan, hipStream_t stream);
 
 hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, const int* col, int* plan,
                            hipStream_t stream);

@@ -8,6 +8,25 @@
 
 namespace rode {
 
+// Rows that the kernels of a plan have taken out of the two lists (see the hub plan and the
+// group plan below): the standard kernels ask before they touch a row.
+constexpr int kGroupRows = 4; // rows of one group of the group plan
+struct RowGroup {
+    int lo, len;          // the run of consecutive columns [lo, lo + len) that all rows of the group hold; len 0: no group
+    int pos[kGroupRows];  // where the run starts in each row (slots from the row's first nonzero)
+    int reserved[2];
+};
+struct RowOwners {
+    int hub_min_len = 0;              // > 0: rows of that aligned length or more belong to the hub kernels
+    const RowGroup* groups = nullptr; // the groups of a group plan, or null
+    int n_groups = 0;
+};
+__device__ __forceinline__ bool owned_elsewhere(const RowOwners& o, int row, int aligned_len)
+{
+    if (o.hub_min_len > 0 && aligned_len >= o.hub_min_len) return true;
+    return o.groups != nullptr && row / kGroupRows < o.n_groups && o.groups[row / kGroupRows].len > 0;
+}
+
 // Aligned slot range [base, base + cnt) of one block work item; the first `mask` slots
 // belong to the previous row (unaligned start) and must not contribute.
 struct BlockItem {
@@ -49,14 +68,13 @@ constexpr int kSpmmMergeSlots = 512;
 
 // SDDMM: merging needs no promise from the caller (an output computed twice at a slice
 // boundary is harmless).
-// hub_min_len > 0: rows of that aligned length or more belong to the hub kernels.
-__device__ __forceinline__ bool sddmm_block_item(int seg, int m1, int hub_min_len, int lane,
+__device__ __forceinline__ bool sddmm_block_item(int seg, int m1, const RowOwners& owners, int lane,
                                                  const int* __restrict__ block_rows, const int* __restrict__ st_off,
                                                  const int* __restrict__ row_ptr, BlockItem& it)
 {
     const int row = block_rows[seg];
     const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
-    if (hub_min_len > 0 && row_end - row_start + (row_start & (kVecLen - 1)) >= hub_min_len) return false;
+    if (owned_elsewhere(owners, row, row_end - row_start + (row_start & (kVecLen - 1)))) return false;
     return merged_leader(kSddmmMergeSlots, seg, m1, lane, row, row_start, row_end, block_rows, st_off, it);
 }
 
@@ -69,13 +87,13 @@ __device__ __forceinline__ bool sddmm_block_item(int seg, int m1, int hub_min_le
 // owned_slots == 0: every segment on its own, rounded to whole 32-slot units as in
 // RoDeSpmm.cu:210-234 (small launches: they need the waves more than they mind the
 // atomics).
-__device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots, int hub_min_len, int lane,
+__device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots, const RowOwners& owners, int lane,
                                                 const int* __restrict__ block_rows, const int* __restrict__ st_off,
                                                 const int* __restrict__ row_ptr, BlockItem& it)
 {
     const int row = block_rows[seg];
     const int row_start = row_ptr[row], row_end = row_ptr[row + 1];
-    if (hub_min_len > 0 && row_end - row_start + (row_start & (kVecLen - 1)) >= hub_min_len) return false;
+    if (owned_elsewhere(owners, row, row_end - row_start + (row_start & (kVecLen - 1)))) return false;
     if (row_end - row_start + (row_start & (kVecLen - 1)) <= owned_slots) {
         if (seg > 0 && block_rows[seg - 1] == row) return false;
         it.row = row;
@@ -98,16 +116,17 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
 // The row of segment `seg` if spmm_block_item() gives it a work item, else -1 (a follower,
 // or past the list).  The same rules, without the extent of the item: what the waves of a
 // workgroup need to know about each other.
-__device__ __forceinline__ int spmm_block_leader_row(int seg, int m1, int owned_slots, int hub_min_len,
+__device__ __forceinline__ int spmm_block_leader_row(int seg, int m1, int owned_slots, const RowOwners& owners,
                                                      const int* __restrict__ block_rows, const int* __restrict__ st_off,
                                                      const int* __restrict__ row_ptr)
 {
     if (seg >= m1) return -1;
     const int row = block_rows[seg];
-    if (hub_min_len <= 0 && (seg == 0 || block_rows[seg - 1] != row || owned_slots == 0)) return row;
+    const bool asks = owners.hub_min_len > 0 || owners.groups != nullptr;
+    if (!asks && (seg == 0 || block_rows[seg - 1] != row || owned_slots == 0)) return row;
     const int row_start = row_ptr[row];
     const int row_base = row_start - (row_start & (kVecLen - 1));
-    if (hub_min_len > 0 && row_ptr[row + 1] - row_base >= hub_min_len) return -1; // the hub kernel's
+    if (asks && owned_elsewhere(owners, row, row_ptr[row + 1] - row_base)) return -1; // another kernel's
     if (seg == 0 || block_rows[seg - 1] != row || owned_slots == 0) return row;
     if (row_ptr[row + 1] - row_base <= owned_slots) return -1; // summed whole by the wave of its first segment
     return (st_off[seg] - row_base) / kSpmmMergeSlots == (st_off[seg - 1] - row_base) / kSpmmMergeSlots ? -1 : row;
@@ -191,6 +210,19 @@ __device__ __forceinline__ WindowDesc plan_residue_desc(const int* __restrict__ 
 {
     const int4 v = *reinterpret_cast<const int4*>(plan + kPlanHeaderInts + kPlanDescInts * chunk);
     return WindowDesc{v.x, v.y, v.z, v.w};
+}
+
+// ---- group plan -----------------------------------------------------------------
+// Groups of kGroupRows adjacent rows that share a long run of consecutive columns (see
+// rode_group.hip).  Layout, ints: header [0] groups (= rows / kGroupRows, whole groups
+// only)  [1] groups with a run  [2], [3] zero; then one RowGroup per group; then three
+// ints per row of scratch for the plan's own kernels.
+constexpr int kGroupHeaderInts = 4;
+static_assert(sizeof(RowGroup) == 32 && kGroupRows == kWavesPerWg, "one wave per row of a group");
+__host__ __device__ inline int row_groups(int M) { return M / kGroupRows; }
+__host__ __device__ inline size_t group_plan_ints(int M)
+{
+    return kGroupHeaderInts + (size_t)row_groups(M) * (sizeof(RowGroup) / sizeof(int)) + 3 * (size_t)M;
 }
 
 // ---- hub plan -------------------------------------------------------------------

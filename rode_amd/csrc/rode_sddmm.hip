@@ -64,7 +64,7 @@ __device__ __forceinline__ void sddmm_row_slots(int row, int base, int mask, int
 // (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
 template <typename T, int KT, int NS, bool EDGE>
 __device__ __forceinline__ void
-sddmm_block_body(int bid, int nblocks, int m1, int k, int hub_min_len, const int* __restrict__ block_rows,
+sddmm_block_body(int bid, int nblocks, int m1, int k, RowOwners owners, const int* __restrict__ block_rows,
                  const int* __restrict__ st_off,
                  const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                  const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
@@ -81,7 +81,7 @@ sddmm_block_body(int bid, int nblocks, int m1, int k, int hub_min_len, const int
     // are pure functions of the inputs, so this is safe even when a caller passes a slice of
     // the lists: the worst case is an output computed twice.)
     BlockItem it;
-    if (!sddmm_block_item(seg, m1, hub_min_len, lane, block_rows, st_off, row_ptr, it)) return;
+    if (!sddmm_block_item(seg, m1, owners, lane, block_rows, st_off, row_ptr, it)) return;
     const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
 
     sddmm_row_slots<T, KT, NS, EDGE>(row, base, mask, cnt, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
@@ -93,7 +93,7 @@ sddmm_block_body(int bid, int nblocks, int m1, int k, int hub_min_len, const int
 // Lane ls of the group owns the slots ls, ls + LPR, ... (value, result, store).
 template <typename T, int KT, int NS, bool EDGE>
 __device__ __forceinline__ void
-sddmm_residue_body(int bid, int nblocks, int m2, int k, int hub_min_len, const int* __restrict__ residue_rows,
+sddmm_residue_body(int bid, int nblocks, int m2, int k, RowOwners owners, const int* __restrict__ residue_rows,
                    const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                    const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out,
                    const int* __restrict__ plan)
@@ -114,7 +114,7 @@ sddmm_residue_body(int bid, int nblocks, int m2, int k, int hub_min_len, const i
     const ResidueItem it = residue_item(row, row_ptr);
     const int first = it.first, cnt = it.cnt;
     if (cnt <= 0) return; // an empty, unaligned row is listed as a residue but owns no slot
-    if (hub_min_len > 0 && it.aligned >= hub_min_len) return; // the hub kernel has the whole row
+    if (owned_elsewhere(owners, row, it.aligned)) return; // another kernel has the whole row
 
     int* my_cols = lds + (wave * RPW + group) * kBlockItems;
     float v[OWN];
@@ -165,21 +165,21 @@ sddmm_residue_body(int bid, int nblocks, int m2, int k, int hub_min_len, const i
 
 template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_block_kernel(int m1, int k, int hub_min_len, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+sddmm_block_kernel(int m1, int k, RowOwners owners, const int* __restrict__ block_rows, const int* __restrict__ st_off,
                    const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                    const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
 {
-    sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m1, k, hub_min_len, block_rows, st_off, row_ptr, col, val, lhs,
+    sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m1, k, owners, block_rows, st_off, row_ptr, col, val, lhs,
                                       rhs, out);
 }
 
 template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_residue_kernel(int m2, int k, int hub_min_len, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
+sddmm_residue_kernel(int m2, int k, RowOwners owners, const int* __restrict__ residue_rows, const int* __restrict__ row_ptr,
                      const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
                      const T* __restrict__ rhs, float* __restrict__ out, const int* __restrict__ plan)
 {
-    sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m2, k, hub_min_len, residue_rows, row_ptr, col, val, lhs, rhs,
+    sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m2, k, owners, residue_rows, row_ptr, col, val, lhs, rhs,
                                         out, plan);
 }
 
@@ -187,17 +187,103 @@ sddmm_residue_kernel(int m2, int k, int hub_min_len, const int* __restrict__ res
 // residue rows.  For matrices so small that a launch costs as much as its kernel.
 template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_pair_kernel(int g1, int m1, int m2, int k, int hub_min_len, const int* __restrict__ block_rows,
+sddmm_pair_kernel(int g1, int m1, int m2, int k, RowOwners owners, const int* __restrict__ block_rows,
                   const int* __restrict__ residue_rows,
                   const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const float* __restrict__ val, const T* __restrict__ lhs, const T* __restrict__ rhs,
                   float* __restrict__ out, const int* __restrict__ plan)
 {
     if ((int)blockIdx.x < g1)
-        sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, g1, m1, k, hub_min_len, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+        sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, g1, m1, k, owners, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
     else
-        sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, k, hub_min_len, residue_rows, row_ptr, col, val, lhs,
+        sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, k, owners, residue_rows, row_ptr, col, val, lhs,
                                             rhs, out, plan);
+}
+
+// The groups of a group plan (rode_group.hip): one workgroup per group of four adjacent
+// rows that share a run of consecutive columns.  The waves split the run; every rhs row of
+// it is loaded once (its address follows from the run, no column index is read) and
+// multiplied with the lhs rows of all four rows of the group, which stay in registers.
+// Wave w then computes row w's nonzeros outside the run as usual.  Single-slab rows only
+// (k <= 128 elements per lane tile): four lhs slices of more slabs would not fit.
+template <typename T, int KT, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
+                   const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
+                   const T* __restrict__ rhs, float* __restrict__ out)
+{
+    using S = SddmmShape<T, KT>;
+    constexpr int LPR = S::kLpr, VEC = S::kVec, R = kGroupRows;
+    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
+    const int g = xcd_logical_block(blockIdx.x, gridDim.x);
+    if (g >= n_groups) return;
+    const RowGroup d = groups[g];
+    if (d.len <= 0) return; // not a group: its rows are in the lists
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int ls = lane % LPR;
+    const int row0 = g * R;
+    float a[R][1][VEC];
+    int first[R]; // where the run starts in column_indices / values, per row
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
+        first[r] = row_ptr[row0 + r] + d.pos[r];
+    }
+    const T* rhs_lane = rhs + ls * VEC;
+    // this wave's quarter of the run, in quads of columns; lane e of a step has column j0 + e
+    const int quads = (d.len + 3) / 4;
+    const int q_begin = quads * wave / kWavesPerWg, q_end = quads * (wave + 1) / kWavesPerWg;
+    const int j_end = min(d.len, 4 * q_end);
+    const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
+    for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
+        if (j0 + (lane & 32) < j_end) { // the upper half sits out a step that has nothing for it
+            float result[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) result[r] = 0.f;
+#pragma unroll
+            for (int q = 0; q < S::kQuads; ++q) {
+                float p[R][4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int c = d.lo + min(j0 + group_first + 4 * q + t, d.len - 1);
+                    float b[VEC];
+                    if (!EDGE || ls * VEC < k) {
+                        DenseVec<T>::load(rhs_lane + (size_t)c * k, b);
+                    } else {
+#pragma unroll
+                        for (int x = 0; x < VEC; ++x) b[x] = 0.f;
+                    }
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        float sum = 0.f;
+#pragma unroll
+                        for (int x = 0; x < VEC; ++x) sum = fmaf(a[r][0][x], b[x], sum);
+                        p[r][t] = sum;
+                    }
+                }
+                // transpose-reduce per row: afterwards lane (ls & 3) == t holds column t of the quad
+                const bool hi2 = ls & 2, hi1 = ls & 1;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const float q0 = (hi2 ? p[r][2] : p[r][0]) + lane_xor2(hi2 ? p[r][0] : p[r][2]);
+                    const float q1 = (hi2 ? p[r][3] : p[r][1]) + lane_xor2(hi2 ? p[r][1] : p[r][3]);
+                    float v = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
+                    v = butterfly_sum<4, LPR>(v);
+                    if ((ls >> 2) == q) result[r] = v;
+                }
+            }
+            const int j = j0 + lane;
+            if (j < j_end) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) out[first[r] + j] = val[first[r] + j] * result[r];
+            }
+        }
+    }
+    // row `wave`: its nonzeros before and after the run
+    const int row = row0 + wave, s = row_ptr[row], e = row_ptr[row + 1];
+    const int run_first = s + d.pos[wave], run_end = run_first + d.len;
+    sddmm_row_slots<T, KT, 1, EDGE>(row, s, 0, run_first - s, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
+    sddmm_row_slots<T, KT, 1, EDGE>(row, run_end, 0, e - run_end, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
 }
 
 // The rows of a hub plan, cut into pieces by column slab (rode_items.hpp): one wave per
@@ -249,23 +335,31 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
         window_residue = plan.host_counts[1] > 0;
     }
     const bool hub_plan = plan.hub != nullptr && plan.hub_counts != nullptr && plan.hub_counts[3] != 0 && plan.hub_counts[0] > 0;
-    const int hub_min_len = hub_plan ? plan.hub_counts[2] : 0;
+    // (the group kernel keeps four lhs slices in registers: rows of one slab only)
+    const bool group_plan = NS == 1 && plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] > 0;
+    RowOwners owners;
+    owners.hub_min_len = hub_plan ? plan.hub_counts[2] : 0;
+    if (group_plan) {
+        owners.groups = reinterpret_cast<const RowGroup*>(plan.groups + kGroupHeaderInts);
+        owners.n_groups = plan.group_counts[0];
+    }
     const bool hubs = hub_plan && (plan.only == 0 || plan.only == kSpmmOnlyHub);
+    const bool grouped = group_plan && (plan.only == 0 || plan.only == kSpmmOnlyHub); // (timed with the hub kernels)
     if (plan.only != 0) { // one kernel family of the call (timing each on its own)
         if (plan.only != kSpmmOnlyBlock) m1 = 0;
         if (plan.only != kSpmmOnlyResidue) m2 = 0;
     }
     if (m1 > 0 && m2 > 0 && standard_residue && s1 == s2 && g1 + g2 <= kPairMaxWorkgroups) {
         sddmm_pair_kernel<T, KT, NS, EDGE><<<g1 + g2, kWgThreads, 0, s1>>>(
-            g1, m1, m2, k, hub_min_len, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);
+            g1, m1, m2, k, owners, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);
     } else {
         if (m1 > 0) {
             sddmm_block_kernel<T, KT, NS, EDGE><<<g1, kWgThreads, 0, s1>>>(
-                m1, k, hub_min_len, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+                m1, k, owners, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
         }
         if (m2 > 0 && standard_residue) {
             sddmm_residue_kernel<T, KT, NS, EDGE><<<g2, kWgThreads, 0, s2>>>(
-                m2, k, hub_min_len, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev);
+                m2, k, owners, residue_rows, row_ptr, col, val, lhs, rhs, out, plan.dev);
         }
     }
     hipError_t e = hipGetLastError();
@@ -275,6 +369,14 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
         if (gh < 0) return hipErrorInvalidConfiguration;
         sddmm_hub_kernel<T, KT, NS, EDGE><<<gh, kWgThreads, 0, s1>>>(k, merge, plan.hub, col, val, lhs, rhs, out);
         e = hipGetLastError();
+    }
+    if constexpr (NS == 1) {
+        if (e == hipSuccess && grouped) {
+            const int gg = (owners.n_groups + kXcds - 1) / kXcds * kXcds;
+            sddmm_group_kernel<T, KT, EDGE><<<gg, kWgThreads, 0, s1>>>(k, owners.n_groups, owners.groups, row_ptr, col, val,
+                                                                        lhs, rhs, out);
+            e = hipGetLastError();
+        }
     }
     if (e == hipSuccess && m2 > 0 && window_residue)
         e = sddmm_window_launch<T>(m2, k, col, val, lhs, rhs, out, plan.dev, plan.rows, s2);

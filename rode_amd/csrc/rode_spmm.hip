@@ -112,7 +112,7 @@ __device__ __forceinline__ void spmm_sum_slots(int base, int mask, int cnt, int 
 // (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
 template <typename T, int TN, bool EDGE>
 __device__ __forceinline__ void
-spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int hub_min_len, const int* __restrict__ block_rows,
+spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, RowOwners owners, const int* __restrict__ block_rows,
                 const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
                 const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                 typename DenseVec<T>::Acc* __restrict__ C)
@@ -126,7 +126,7 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int hub_mi
     const int seg0 = xcd_logical_block(bid, nblocks) * kWavesPerWg;
     const int seg = seg0 + wave;
     BlockItem it{-1, 0, 0, 0};
-    const bool active = seg < m1 && spmm_block_item(seg, m1, owned_slots, hub_min_len, lane, block_rows, st_off, row_ptr, it);
+    const bool active = seg < m1 && spmm_block_item(seg, m1, owned_slots, owners, lane, block_rows, st_off, row_ptr, it);
     // A wave without a work item leaves at once (with the reference's 32-slot segments that
     // is most waves); the barrier below then counts only the waves that are still running
     // (S_BARRIER waits on the surviving waves of a workgroup).
@@ -139,7 +139,7 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int hub_mi
     bool shared_row = false;
 #pragma unroll
     for (int i = 0; i < kWavesPerWg; ++i) {
-        item_row[i] = spmm_block_leader_row(seg0 + i, m1, owned_slots, hub_min_len, block_rows, st_off, row_ptr);
+        item_row[i] = spmm_block_leader_row(seg0 + i, m1, owned_slots, owners, block_rows, st_off, row_ptr);
         if (i > 0) shared_row = shared_row || (item_row[i] >= 0 && item_row[i] == item_row[i - 1]);
     }
     const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
@@ -189,7 +189,7 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int hub_mi
 // group walks its row's slot quads one after the other, no cross-lane reduction.
 template <typename T, int TN, bool EDGE>
 __device__ __forceinline__ void
-spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, int hub_min_len,
+spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, RowOwners owners,
                   const int* __restrict__ residue_rows,
                   const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
@@ -213,7 +213,7 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, int hub_
     const ResidueItem it = residue_item(row, row_ptr);
     const bool accumulate = it.accumulate; // the row also has block segments
     if (accumulate && it.aligned <= owned_slots) return; // summed entirely, tail included, by the block kernel
-    if (hub_min_len > 0 && it.aligned >= hub_min_len) return; // the hub kernel has the whole row
+    if (owned_elsewhere(owners, row, it.aligned)) return; // another kernel has the whole row
     const int first = it.first, cnt = it.cnt;
 
     const int tile = blockIdx.y * TN;
@@ -252,24 +252,24 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, int hub_
 
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_block_kernel(int m1, int n, int owned_slots, int hub_min_len, const int* __restrict__ block_rows,
+spmm_block_kernel(int m1, int n, int owned_slots, RowOwners owners, const int* __restrict__ block_rows,
                   const int* __restrict__ st_off,
                   const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                   typename DenseVec<T>::Acc* __restrict__ C)
 {
-    spmm_block_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m1, n, owned_slots, hub_min_len, block_rows, st_off, row_ptr, col, val,
+    spmm_block_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m1, n, owned_slots, owners, block_rows, st_off, row_ptr, col, val,
                                  B, C);
 }
 
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_residue_kernel(int m2, int n, int owned_slots, int hub_min_len, const int* __restrict__ residue_rows,
+spmm_residue_kernel(int m2, int n, int owned_slots, RowOwners owners, const int* __restrict__ residue_rows,
                     const int* __restrict__ row_ptr, const int* __restrict__ col,
                     const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                     typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
-    spmm_residue_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m2, n, owned_slots, hub_min_len, residue_rows, row_ptr, col, val, B,
+    spmm_residue_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m2, n, owned_slots, owners, residue_rows, row_ptr, col, val, B,
                                    C, plan);
 }
 
@@ -278,17 +278,113 @@ spmm_residue_kernel(int m2, int n, int owned_slots, int hub_min_len, const int* 
 // kernel (a kernel of a few microseconds); the two parts then also fill the GPU together.
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, int hub_min_len, const int* __restrict__ block_rows,
+spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, RowOwners owners, const int* __restrict__ block_rows,
                  const int* __restrict__ residue_rows, const int* __restrict__ st_off, const int* __restrict__ row_ptr,
                  const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
                  const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
     if ((int)blockIdx.x < g1)
-        spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, hub_min_len, block_rows, st_off, row_ptr, col, val, B, C);
+        spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, owners, block_rows, st_off, row_ptr, col, val, B, C);
     else
-        spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, max(owned_slots, 0), hub_min_len, residue_rows,
+        spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, max(owned_slots, 0), owners, residue_rows,
                                        row_ptr, col, val,
                                        B, C, plan);
+}
+
+// The groups of a group plan (rode_group.hip): one workgroup per group of four adjacent
+// rows that share a run of consecutive columns.  The waves split the run; every dense row
+// of it is loaded once and multiplied into the sums of all four rows (its address follows
+// from the run, no column index is read).  Wave w then adds row w's nonzeros outside the
+// run, the waves' sums meet in LDS, and wave w adds the total of row w to C (the row is in
+// no other work item: no atomics).
+template <typename T, int TN, bool EDGE>
+__global__ void __launch_bounds__(kWgThreads)
+spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
+                  const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
+                  const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C)
+{
+    using S = SpmmShape<T, TN>;
+    using A = typename S::Acc;
+    constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
+    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
+    __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg][R][kWave];
+    __shared__ __attribute__((aligned(16))) A sums[kWavesPerWg][R][TN];
+    const int g = xcd_logical_block(blockIdx.x, gridDim.x);
+    if (g >= n_groups) return;
+    const RowGroup d = groups[g];
+    if (d.len <= 0) return; // not a group: its rows are in the lists
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int ls = lane % LPR, group = lane / LPR;
+    const int tile = blockIdx.y * TN;
+    const bool col_ok = !EDGE || tile + ls * VEC < n;
+    const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
+    const int row0 = g * R;
+    int first[R]; // where the run starts in column_indices / values, per row
+#pragma unroll
+    for (int r = 0; r < R; ++r) first[r] = row_ptr[row0 + r] + d.pos[r];
+
+    // this wave's quarter of the run, in quads of columns
+    const int quads = (d.len + 3) / 4;
+    const int q_begin = quads * wave / kWavesPerWg, q_end = quads * (wave + 1) / kWavesPerWg;
+    const int j_end = min(d.len, 4 * q_end);
+    A acc[R][VEC];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) acc[r][x] = A(0);
+    for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
+        const int j = j0 + lane;
+#pragma unroll
+        for (int r = 0; r < R; ++r) lds_v[wave][r][lane] = j < j_end ? val[first[r] + j] : A(0);
+        wave_lds_sync();
+        const int nq = min(kWave / 4, (j_end - j0 + 3) / 4);
+#pragma unroll
+        for (int i = 0; i < kWave / 4 / G; ++i) {
+            const int q = group + i * G;
+            if (q < nq) {
+                A b[4][VEC];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    DenseVec<T>::load(b_lane + (size_t)(d.lo + min(j0 + 4 * q + t, d.len - 1)) * n, b[t]);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    A v[4];
+                    load_quad(&lds_v[wave][r][4 * q], v);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+#pragma unroll
+                        for (int x = 0; x < VEC; ++x) acc[r][x] = fma(v[t], b[t][x], acc[r][x]);
+                }
+            }
+        }
+        wave_lds_sync();
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) acc[r][x] = butterfly_sum<LPR, kWave>(acc[r][x]);
+        if (group == 0) {
+#pragma unroll
+            for (int x = 0; x < VEC; ++x) sums[wave][r][ls * VEC + x] = acc[r][x];
+        }
+    }
+    // row `wave`: its nonzeros before and after the run
+    const int row = row0 + wave, s = row_ptr[row], e = row_ptr[row + 1];
+    const int run_first = s + d.pos[wave], run_end = run_first + d.len;
+    A before[VEC], after[VEC];
+    spmm_sum_slots<T, TN>(s, 0, run_first - s, lane, lds_c + wave * kWave, &lds_v[wave][0][0], b_lane, n, col, val, before);
+    spmm_sum_slots<T, TN>(run_end, 0, e - run_end, lane, lds_c + wave * kWave, &lds_v[wave][0][0], b_lane, n, col, val, after);
+    __syncthreads();
+    if (group == 0 && col_ok) {
+        A* c_lane = C + (size_t)row * n + tile + ls * VEC;
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) {
+            A total = before[x] + after[x];
+#pragma unroll
+            for (int w = 0; w < kWavesPerWg; ++w) total += sums[w][wave][ls * VEC + x];
+            c_lane[x] += total; // (long rows are accumulated into C by contract)
+        }
+    }
 }
 
 // The rows of a hub plan, cut into pieces by column slab (rode_items.hpp): one wave per
@@ -433,9 +529,16 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     // a usable hub plan takes its rows out of both lists (the caller promised whole lists with it)
     const bool hub_plan = plan.hub != nullptr && plan.hub_counts != nullptr && plan.hub_counts[3] != 0 &&
                           plan.hub_counts[0] > 0;
-    const int hub_min_len = hub_plan ? plan.hub_counts[2] : 0;
+    const bool group_plan = plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] > 0;
+    RowOwners owners;
+    owners.hub_min_len = hub_plan ? plan.hub_counts[2] : 0;
+    if (group_plan) {
+        owners.groups = reinterpret_cast<const RowGroup*>(plan.groups + kGroupHeaderInts);
+        owners.n_groups = plan.group_counts[0];
+    }
     const int only = flags & kOnlyMask; // one kernel family of the call (timing each on its own)
     const bool hubs = hub_plan && (only == 0 || only == kSpmmOnlyHub);
+    const bool grouped = group_plan && (only == 0 || only == kSpmmOnlyHub); // (timed with the hub kernels)
     constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
     const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0 || tiles > 65535) return hipErrorInvalidConfiguration;
@@ -450,19 +553,19 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     hipError_t e = hipSuccess;
     if (block && residue && standard_residue && s1 == s2 && (long long)(g1 + g2) * tiles <= kPairMaxWorkgroups) {
         dim3 grid(g1 + g2, tiles);
-        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, hub_min_len, block_rows, residue_rows,
+        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, owners, block_rows, residue_rows,
                                                                    st_off, row_ptr, col, val, B, C, plan.dev);
         e = hipGetLastError();
     } else {
         if (block) {
             dim3 grid(g1, tiles);
-            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, hub_min_len, block_rows, st_off, row_ptr,
+            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, owners, block_rows, st_off, row_ptr,
                                                                         col, val, B, C);
             e = hipGetLastError();
         }
         if (residue && standard_residue) {
             dim3 grid(g2, tiles);
-            spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, hub_min_len, residue_rows, row_ptr, col,
+            spmm_residue_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s2>>>(m2, n, owned_slots, owners, residue_rows, row_ptr, col,
                                                                           val, B, C, plan.dev);
             if (e == hipSuccess) e = hipGetLastError();
         }
@@ -478,6 +581,12 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
         A* partial = plan.hub_workspace && plan.hub_workspace_bytes >= need ? static_cast<A*>(plan.hub_workspace) : nullptr;
         spmm_hub_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(n, merge, plan.hub, col, val, B, C, partial);
         if (partial) spmm_hub_reduce_kernel<A><<<plan.hub_counts[0], kWgThreads, 0, s1>>>(n, merge, plan.hub, partial, C);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess && grouped) {
+        const int gg = (owners.n_groups + kXcds - 1) / kXcds * kXcds;
+        dim3 grid(gg, tiles);
+        spmm_group_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(n, owners.n_groups, owners.groups, row_ptr, col, val, B, C);
         e = hipGetLastError();
     }
     if constexpr (!std::is_same<T, double>::value) {

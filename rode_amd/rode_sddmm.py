@@ -111,7 +111,7 @@ class RoDeCSR:
         # "auto" wants windows on at least half of the chunks and enough of them to fill the
         # GPU twice (a few windowed chunks only add launches); True keeps any plan with a
         # window; False makes none.
-        self.plan = self._hub_plan() if self.locality else None
+        self.plan = (self._group_plan() or self._hub_plan()) if self.locality else None
         if self.plan is None and self.locality and m2 > 0:
             plan = rode_sddmm_hip.window_plan(res, m2, self.row_offsets, self.column_indices, self.n)
             enough = plan.windowed >= max(self.PLAN_MIN_CHUNKS, (plan.counts[0] + 1) // 2)
@@ -124,6 +124,20 @@ class RoDeCSR:
     HUB_MIN_LEN = 4096
     HUB_MIN_SLABS = 16
     HUB_MIN_SHARE = 0.1
+
+    # A group plan is kept when at least half of the groups of four rows share a run (or any,
+    # with locality=True), and is only looked for in matrices with at least GROUP_MIN_MEAN
+    # nonzeros per row (a shared run has at least 64 columns).
+    GROUP_MIN_MEAN = 64
+
+    def _group_plan(self):
+        """Group plan (adjacent rows that share a long run of consecutive columns are processed
+        together, each dense row of the run loaded once for all of them), or None."""
+        if self.m < 4 or self.nnz < self.GROUP_MIN_MEAN * self.m:
+            return None
+        plan = rode_sddmm_hip.group_plan(self.row_offsets, self.column_indices, self.m)
+        enough = 2 * plan.counts[1] >= plan.counts[0]
+        return plan if plan.usable and (self.locality is True or enough) else None
 
     def _hub_plan(self):
         """Hub plan (rows with very many nonzeros are processed column slab by column slab so

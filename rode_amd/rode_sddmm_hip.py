@@ -207,13 +207,53 @@ def hub_plan(row_offsets, column_indices, m, n, min_len):
     return HubPlan(data, list(counts))
 
 
+class GroupPlan:
+    """Group plan of one pattern (``rode_hip_group_plan``): the device array and a host copy
+    of its header ``[groups, groups with a shared run, 0, 0]``."""
+
+    def __init__(self, data, counts):
+        self.data = data
+        self.counts = counts
+        self._header = (ctypes.c_int * 4)(*counts)
+        self.rows = None  # (a matrix has one kind of plan)
+
+    @property
+    def usable(self):
+        return self.counts[1] > 0
+
+    def groups(self):
+        """int32 array (groups, 8): first column and length of the shared run (0: none), its
+        position in each of the four rows, two unused."""
+        return self.data[4:4 + 8 * self.counts[0]].cpu().numpy().reshape(-1, 8)
+
+
+def group_plan(row_offsets, column_indices, m):
+    """Group plan: which groups of four adjacent rows share a long run of consecutive
+    columns.  Waits for its kernels (it returns the counts)."""
+    for t, name in ((row_offsets, "row_offsets"), (column_indices, "column_indices")):
+        _check_input(t, name)
+        _check(t.dtype == torch.int32, f"{name} must be int32")
+    lib = _lib.load()
+    dev = row_offsets.device
+    nbytes = lib.rode_hip_group_plan_bytes(m)
+    with torch.cuda.device(dev):
+        data = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
+        counts = (ctypes.c_int * 4)()
+        _lib.check(lib.rode_hip_group_plan(m, row_offsets.data_ptr(), column_indices.data_ptr(), data.data_ptr(), nbytes,
+                                           ctypes.addressof(counts), _stream_handle(dev)), "rode_hip_group_plan")
+    return GroupPlan(data, list(counts))
+
+
 def plans_struct(plan, spmm_width=None, spmm_elem_bytes=4, whole_lists=True):
     """The ``rode_hip_plans`` struct of one call (keep it alive until the call returns; pass
-    it with ``ctypes.byref``).  ``plan``: a ``WindowPlan``, a ``HubPlan`` or None.
+    it with ``ctypes.byref``).  ``plan``: a ``WindowPlan``, a ``HubPlan``, a ``GroupPlan`` or None.
     ``spmm_width``: for an SpMM call the dense width, so that a hub plan's workspace is
     attached; a hub plan is left out of an SpMM call without the whole-lists promise."""
     p = _lib.Plans()
-    if isinstance(plan, HubPlan):
+    if isinstance(plan, GroupPlan):
+        if plan.usable and (spmm_width is None or whole_lists):
+            p.groups, p.group_counts = plan.data.data_ptr(), ctypes.addressof(plan._header)
+    elif isinstance(plan, HubPlan):
         if plan.usable and (spmm_width is None or whole_lists):
             p.hub, p.hub_counts = plan.data.data_ptr(), ctypes.addressof(plan._header)
             if spmm_width is not None:

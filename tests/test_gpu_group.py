@@ -1,0 +1,157 @@
+"""Group plan: groups of four adjacent rows that share a long run of consecutive columns
+are processed by kernels of their own (rode_group.hip, spmm_group_kernel,
+sddmm_group_kernel).  The plan changes which kernel processes a row, never a result:
+everything here is checked against the fp64 oracle with the tolerances of the unplanned
+kernels."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _window_matrix(rng, m, n, window, extra, ragged=True):
+    """Sliding window of `window` columns around the diagonal plus `extra` random columns
+    per row; with `ragged`, some rows get holes in their window, some are empty, some short."""
+    rows = []
+    for r in range(m):
+        lo, hi = max(0, r * n // m - window // 2), min(n, r * n // m + window // 2)
+        c = set(range(lo, hi)) | set(rng.choice(n, extra, replace=False).tolist())
+        if ragged and r % 37 == 5:
+            c -= set(range(lo + 10, lo + 13))          # a hole: the longest run is only part of the window
+        if ragged and r % 53 == 7:
+            c = set()                                  # an empty row inside a group
+        if ragged and r % 61 == 9:
+            c = set(rng.choice(n, 5, replace=False).tolist())  # a short row without a run
+        rows.append(np.array(sorted(c), dtype=np.int32))
+    rp = np.zeros(m + 1, dtype=np.int32)
+    rp[1:] = np.cumsum([len(c) for c in rows])
+    col = np.concatenate(rows).astype(np.int32) if rp[-1] else np.zeros(0, dtype=np.int32)
+    val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
+    return rp, col, val
+
+
+def test_plan_contents():
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(0)
+    m, n = 203, 900   # 203 rows: the last three are in no group
+    rp, col, val = _window_matrix(rng, m, n, 200, 12)
+    dev = torch.device("cuda:0")
+    plan = rode_sddmm_hip.group_plan(torch.from_numpy(rp).to(dev), torch.from_numpy(col).to(dev), m)
+    assert plan.counts[0] == m // 4
+    desc = plan.groups()
+    kept = 0
+    for g in range(m // 4):
+        runs = []
+        for r in range(4 * g, 4 * g + 4):
+            c = col[rp[r]:rp[r + 1]]
+            best = (0, 0, 0)
+            i = 0
+            while i < len(c):                      # longest run of consecutive columns (the first of equals)
+                j = i
+                while j + 1 < len(c) and c[j + 1] == c[j] + 1:
+                    j += 1
+                if j - i + 1 > best[1]:
+                    best = (int(c[i]), j - i + 1, i)
+                i = j + 1
+            runs.append(best)
+        lo, hi = max(a for a, _, _ in runs), min(a + l for a, l, _ in runs)
+        slots = rp[4 * g + 4] - rp[4 * g]
+        keep = hi - lo >= 64 and 16 * (hi - lo) >= 3 * slots
+        if keep:
+            kept += 1
+            assert desc[g, 0] == lo and desc[g, 1] == hi - lo
+            assert desc[g, 2:6].tolist() == [p + lo - a for a, _, p in runs]
+        else:
+            assert desc[g, 1] == 0
+    assert plan.counts[1] == kept and 0 < kept < m // 4   # the ragged rows break some groups
+
+
+@pytest.mark.parametrize("k,half", [(64, False), (128, False), (32, False), (64, True), (128, True), (200, False)])
+def test_grouped_rows_against_oracle(k, half):
+    import oracle
+    from gpu_common import TOL_F16, TOL_F32, make_csr, round_half, run_sddmm, run_spmm
+    from helpers import spmm_row_l1_error, sddmm_row_l1_errors
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(k)
+    m, n = 1001, 1500
+    rp, col, val = _window_matrix(rng, m, n, 300 if k != 32 else 77, 20)
+    csr = make_csr(rp, col, val, m, n, k, locality=True)
+    assert isinstance(csr.plan, rode_sddmm_hip.GroupPlan) and csr.plan.usable
+    B = rng.standard_normal((n, k)).astype(np.float32)
+    L = rng.standard_normal((m, k)).astype(np.float32)
+    Bq, Lq = (round_half(B), round_half(L)) if half else (B, L)
+    tol = TOL_F16 if half else TOL_F32
+    assert spmm_row_l1_error(run_spmm(csr, B, half), oracle.spmm_f64(rp, col, val, Bq)) <= tol
+    ref64, scale = oracle.sddmm_f64(rp, col, val, Lq, Bq, with_abs=True)
+    out = run_sddmm(csr, L, B, half)
+    err, cond = sddmm_row_l1_errors(out, ref64, scale, rp)
+    assert float(err[cond <= 100].max(initial=0.0)) <= tol
+    if not half:
+        assert (np.abs(out - ref64) / np.maximum(scale, 1e-30)).max() <= 2e-6
+    if k == 64 and not half:  # fp64, and accumulation into a C that is not zero
+        dev = csr.device
+        C0 = torch.from_numpy(rng.standard_normal((m, k))).to(dev)
+        C = C0.clone()
+        rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
+                                    csr.row_offsets, csr.column_indices, csr.values.double(), m, n,
+                                    torch.from_numpy(B).to(dev).double(), out=C, plan=csr.plan)
+        aligned = np.diff(rp) + rp[:-1] % 4
+        kept = (aligned >= 32) | (aligned == 0)  # long rows are added to, rows in no list untouched, short rows overwritten
+        want = oracle.spmm_f64(rp, col, val, B) + np.where(kept[:, None], C0.cpu().numpy(), 0.0)
+        assert np.abs(C.cpu().numpy() - want).max() <= 1e-12 * max(1.0, np.abs(want).max())
+
+
+def test_every_nonzero_has_one_owner_and_what_is_refused():
+    import ctypes
+    from gpu_common import DEV, make_csr
+    from rode_amd import _lib, rode_sddmm_hip
+    lib = _lib.load()
+    rng = np.random.default_rng(9)
+    m, n, k = 400, 1200, 64
+    rp, col, val = _window_matrix(rng, m, n, 256, 16)
+    csr = make_csr(rp, col, val, m, n, k, locality=False)
+    plan = rode_sddmm_hip.group_plan(csr.row_offsets, csr.column_indices, m)
+    assert plan.usable
+    L = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(DEV)
+    B = torch.from_numpy(rng.standard_normal((n, k)).astype(np.float32)).to(DEV)
+
+    def plans(groups=True, hub=False):
+        p = _lib.Plans()
+        if groups:
+            p.groups, p.group_counts = plan.data.data_ptr(), ctypes.addressof(plan._header)
+        if hub:
+            p.hub, p.hub_counts = plan.data.data_ptr(), ctypes.addressof(plan._header)
+        return p
+
+    def sddmm(flags, p):
+        out = torch.full((len(val),), float("nan"), device=DEV)
+        code = lib.rode_hip_sddmm_planned(0, flags, csr.m1, csr.m2, n, k, csr.block_indices.data_ptr(),
+                                          csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(),
+                                          csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
+                                          L.data_ptr(), B.data_ptr(), out.data_ptr(), ctypes.byref(p), None, None)
+        torch.cuda.synchronize()
+        return code, out
+
+    code, plain = sddmm(0, plans(False))
+    code2, grouped = sddmm(0, plans())
+    assert code == 0 and code2 == 0 and not torch.isnan(grouped).any()
+    assert (grouped - plain).abs().max().item() <= 2e-5 * plain.abs().max().item()
+    written = [~torch.isnan(sddmm(f, plans())[1]) for f in (_lib.SPMM_ONLY_BLOCK, _lib.SPMM_ONLY_RESIDUE, _lib.SPMM_ONLY_HUB)]
+    assert (written[0].int() + written[1].int() + written[2].int() == 1).all()
+    assert sddmm(0, plans(True, True))[0] != 0   # a group plan next to a hub plan
+
+    def spmm(flags, p):
+        C = torch.zeros(m, k, device=DEV)
+        code = lib.rode_hip_spmm_planned(0, flags, csr.m1, csr.m2, n, k, csr.values.data_ptr(), csr.column_indices.data_ptr(),
+                                         csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(),
+                                         csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(), B.data_ptr(),
+                                         C.data_ptr(), ctypes.byref(p), None, None)
+        torch.cuda.synchronize()
+        return code, C
+
+    code, plain_c = spmm(_lib.SPMM_WHOLE_LISTS, plans(False))
+    parts = [spmm(_lib.SPMM_WHOLE_LISTS | f, plans()) for f in (_lib.SPMM_ONLY_BLOCK, _lib.SPMM_ONLY_RESIDUE, _lib.SPMM_ONLY_HUB)]
+    assert code == 0 and all(c == 0 for c, _ in parts)
+    assert (sum(p for _, p in parts) - plain_c).abs().max().item() <= 2e-5 * plain_c.abs().max().item()
+    assert spmm(0, plans())[0] != 0  # a group plan without the whole-lists promise
