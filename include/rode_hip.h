@@ -220,8 +220,9 @@ int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_
  * other kernels leave those rows out.  Same results up to the order of the fp32 additions.
  *   d_plan       rode_hip_group_plan_bytes(M) bytes, 16-byte aligned, out
  *   h_counts     HOST int[4], out (the call waits for its kernels): [0] groups (M / 4,
- *                whole groups only), [1] groups with a run; the *_planned entry points
- *                need it and ignore a plan with [1] == 0
+ *                whole groups only), [1] groups with a run, [2] rows outside those groups
+ *                (0: the other kernels have nothing to do and are not launched); the
+ *                *_planned entry points need it and ignore a plan with [1] == 0
  * A group plan belongs to the pattern it was made from and excludes the other two plans.
  * SDDMM uses it for k <= 128 (fp32) / 256 (fp16) elements, SpMM for any width.
  */

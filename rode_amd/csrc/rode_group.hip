@@ -77,15 +77,19 @@ group_desc_kernel(int groups, const int* __restrict__ row_ptr, const int* __rest
     }
     d.reserved[0] = d.reserved[1] = 0;
     reinterpret_cast<RowGroup*>(plan + kGroupHeaderInts)[g] = d;
-    if (keep) atomicAdd(plan + 1, 1);
+    if (keep) {
+        atomicAdd(plan + 1, 1);
+        atomicSub(plan + 2, kGroupRows);
+    }
 }
 
-__global__ void group_header_kernel(int groups, int* __restrict__ plan)
+__global__ void group_header_kernel(int M, int groups, int* __restrict__ plan)
 {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         plan[0] = groups;
         plan[1] = 0;
-        for (int i = 2; i < kGroupHeaderInts; ++i) plan[i] = 0;
+        plan[2] = M; // rows outside the groups with a run: counted down as groups are kept
+        plan[3] = 0;
     }
 }
 
@@ -94,7 +98,7 @@ __global__ void group_header_kernel(int groups, int* __restrict__ plan)
 hipError_t group_plan_launch(int M, const int* row_ptr, const int* col, int* plan, hipStream_t stream)
 {
     const int groups = row_groups(M);
-    group_header_kernel<<<1, kWave, 0, stream>>>(groups, plan);
+    group_header_kernel<<<1, kWave, 0, stream>>>(M, groups, plan);
     if (groups > 0) {
         int* runs = plan + kGroupHeaderInts + (size_t)groups * (sizeof(RowGroup) / sizeof(int)); // scratch behind the table
         group_runs_kernel<<<(M + kWgThreads - 1) / kWgThreads, kWgThreads, 0, stream>>>(M, row_ptr, col, runs);

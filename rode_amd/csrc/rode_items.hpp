@@ -215,7 +215,7 @@ __device__ __forceinline__ WindowDesc plan_residue_desc(const int* __restrict__ 
 // ---- group plan -----------------------------------------------------------------
 // Groups of kGroupRows adjacent rows that share a long run of consecutive columns (see
 // rode_group.hip).  Layout, ints: header [0] groups (= rows / kGroupRows, whole groups
-// only)  [1] groups with a run  [2], [3] zero; then one RowGroup per group; then three
+// only)  [1] groups with a run  [2] rows outside those groups  [3] zero; then one RowGroup per group; then three
 // ints per row of scratch for the plan's own kernels.
 constexpr int kGroupHeaderInts = 4;
 static_assert(sizeof(RowGroup) == 32 && kGroupRows == kWavesPerWg, "one wave per row of a group");

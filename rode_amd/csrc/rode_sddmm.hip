@@ -349,6 +349,7 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
         if (plan.only != kSpmmOnlyBlock) m1 = 0;
         if (plan.only != kSpmmOnlyResidue) m2 = 0;
     }
+    if (group_plan && plan.group_counts[2] == 0) m1 = m2 = 0; // every row in a group with a run: nothing for the lists' kernels
     if (m1 > 0 && m2 > 0 && standard_residue && s1 == s2 && g1 + g2 <= kPairMaxWorkgroups) {
         sddmm_pair_kernel<T, KT, NS, EDGE><<<g1 + g2, kWgThreads, 0, s1>>>(
             g1, m1, m2, k, owners, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);

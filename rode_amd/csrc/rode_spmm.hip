@@ -67,8 +67,10 @@ __device__ __forceinline__ void store_row(double* dst, const double (&acc)[VEC])
 // Sum over the aligned slots [base, base + cnt) of values * B rows, for this lane's columns
 // of the tile; the first `mask` slots (the previous row's) and the slots past cnt in the
 // last quad are neutralised.  Every lane of the wave returns the wave's total.
+// (split, jump: the slots are [base, base + split) followed by [base + split + jump, ...):
+// a row with a hole that somebody else works on; split >= cnt for one plain range.)
 template <typename T, int TN>
-__device__ __forceinline__ void spmm_sum_slots(int base, int mask, int cnt, int lane, int* my_c,
+__device__ __forceinline__ void spmm_sum_slots(int base, int mask, int cnt, int split, int jump, int lane, int* my_c,
                                                typename DenseVec<T>::Acc* my_v, const T* b_lane, int n,
                                                const int* __restrict__ col,
                                                const typename DenseVec<T>::Acc* __restrict__ val,
@@ -91,8 +93,10 @@ __device__ __forceinline__ void spmm_sum_slots(int base, int mask, int cnt, int 
             // slots of the previous row (head) and slots past the end (last quad) are
             // neutralised: value 0, column of a real slot
             const bool head = slot < mask, past = slot >= cnt;
-            c = col[base + (head ? mask : (past ? cnt - 1 : slot))];
-            v = (head || past) ? A(0) : val[base + slot];
+            const int at = head ? mask : (past ? cnt - 1 : slot);
+            const int idx = base + at + (at >= split ? jump : 0);
+            c = col[idx];
+            v = (head || past) ? A(0) : val[idx];
         }
         my_c[lane] = c;
         my_v[lane] = v;
@@ -156,7 +160,7 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, RowOwners 
     // combine the lane groups, then spread the atomics over them
     constexpr int EPG = VEC / G > 0 ? VEC / G : 1; // elements each group adds
     A total[VEC];
-    spmm_sum_slots<T, TN>(base, mask, cnt, lane, my_c, my_v, b_lane, n, col, val, total);
+    spmm_sum_slots<T, TN>(base, mask, cnt, cnt, 0, lane, my_c, my_v, b_lane, n, col, val, total);
     if (shared_row) {
         __shared__ __attribute__((aligned(16))) A wg_sum[kWavesPerWg][TN];
         if (group == 0) {
@@ -342,10 +346,13 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
         for (int i = 0; i < kWave / 4 / G; ++i) {
             const int q = group + i * G;
             if (q < nq) {
+                // four consecutive rows of B (the last quad of a run may be cut short: its rows
+                // past the run repeat the run's last row, their values are zero)
+                const T* b_quad = b_lane + (size_t)(d.lo + j0 + 4 * q) * n;
+                const int room = d.len - 1 - (j0 + 4 * q);
                 A b[4][VEC];
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    DenseVec<T>::load(b_lane + (size_t)(d.lo + min(j0 + 4 * q + t, d.len - 1)) * n, b[t]);
+                for (int t = 0; t < 4; ++t) DenseVec<T>::load(b_quad + (size_t)min(t, room) * n, b[t]);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     A v[4];
@@ -371,15 +378,15 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     // row `wave`: its nonzeros before and after the run
     const int row = row0 + wave, s = row_ptr[row], e = row_ptr[row + 1];
     const int run_first = s + d.pos[wave], run_end = run_first + d.len;
-    A before[VEC], after[VEC];
-    spmm_sum_slots<T, TN>(s, 0, run_first - s, lane, lds_c + wave * kWave, &lds_v[wave][0][0], b_lane, n, col, val, before);
-    spmm_sum_slots<T, TN>(run_end, 0, e - run_end, lane, lds_c + wave * kWave, &lds_v[wave][0][0], b_lane, n, col, val, after);
+    A outside[VEC]; // the slots before the run and, in the same pass, those after it
+    spmm_sum_slots<T, TN>(s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, lane, lds_c + wave * kWave,
+                          &lds_v[wave][0][0], b_lane, n, col, val, outside);
     __syncthreads();
     if (group == 0 && col_ok) {
         A* c_lane = C + (size_t)row * n + tile + ls * VEC;
 #pragma unroll
         for (int x = 0; x < VEC; ++x) {
-            A total = before[x] + after[x];
+            A total = outside[x];
 #pragma unroll
             for (int w = 0; w < kWavesPerWg; ++w) total += sums[w][wave][ls * VEC + x];
             c_lane[x] += total; // (long rows are accumulated into C by contract)
@@ -419,7 +426,7 @@ spmm_hub_kernel(int n, int merge, const int* __restrict__ hub, const int* __rest
     const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
     constexpr int EPG = VEC / G > 0 ? VEC / G : 1; // elements each group adds
     A total[VEC];
-    spmm_sum_slots<T, TN>(base, 0, cnt, lane, lds_c + wave * kWave, lds_v + wave * kWave, b_lane, n, col, val, total);
+    spmm_sum_slots<T, TN>(base, 0, cnt, cnt, 0, lane, lds_c + wave * kWave, lds_v + wave * kWave, b_lane, n, col, val, total);
     if (partial) {
         if (group == 0 && col_ok) store_row<VEC>(partial + (size_t)item * n + tile + ls * VEC, total);
         return;
@@ -549,7 +556,10 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
         standard_residue = plan.host_counts[1] < plan.host_counts[0];
         window_residue = plan.host_counts[1] > 0;
     }
-    const bool block = m1 > 0 && (only == 0 || only == kSpmmOnlyBlock), residue = m2 > 0 && (only == 0 || only == kSpmmOnlyResidue);
+    // (every row in a group with a run: the lists' kernels would find nothing to do)
+    const bool lists = !(group_plan && plan.group_counts[2] == 0);
+    const bool block = lists && m1 > 0 && (only == 0 || only == kSpmmOnlyBlock);
+    const bool residue = lists && m2 > 0 && (only == 0 || only == kSpmmOnlyResidue);
     hipError_t e = hipSuccess;
     if (block && residue && standard_residue && s1 == s2 && (long long)(g1 + g2) * tiles <= kPairMaxWorkgroups) {
         dim3 grid(g1 + g2, tiles);

@@ -65,6 +65,7 @@ def test_plan_contents():
         else:
             assert desc[g, 1] == 0
     assert plan.counts[1] == kept and 0 < kept < m // 4   # the ragged rows break some groups
+    assert plan.counts[2] == m - 4 * kept                 # rows left to the other kernels
 
 
 @pytest.mark.parametrize("k,half", [(64, False), (128, False), (32, False), (64, True), (128, True), (200, False)])
