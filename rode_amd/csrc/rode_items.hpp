@@ -218,6 +218,7 @@ __device__ __forceinline__ WindowDesc plan_residue_desc(const int* __restrict__ 
 // only)  [1] groups with a run  [2] rows outside those groups  [3] zero; then one RowGroup per group; then three
 // ints per row of scratch for the plan's own kernels.
 constexpr int kGroupHeaderInts = 4;
+constexpr int kGroupWaveEach = 2048; // from this many groups with a run on, a group is one wave's work, below it a workgroup's
 static_assert(sizeof(RowGroup) == 32 && kGroupRows == kWavesPerWg, "one wave per row of a group");
 __host__ __device__ inline int row_groups(int M) { return M / kGroupRows; }
 __host__ __device__ inline size_t group_plan_ints(int M)

@@ -29,8 +29,11 @@ namespace {
 // out[idx] = values[idx] * <lhs[row, :], rhs[col(idx), :]> for the aligned slots
 // [base, base + cnt) of one row, 64 slots per step; the first `mask` slots (the previous
 // row's) are computed but not stored.
+// (split, jump: the slots are [base, base + split) followed by [base + split + jump, ...):
+// a row with a hole that somebody else works on; split >= cnt for one plain range.)
 template <typename T, int KT, int NS, bool EDGE>
-__device__ __forceinline__ void sddmm_row_slots(int row, int base, int mask, int cnt, int k, int lane, int* lds_cols,
+__device__ __forceinline__ void sddmm_row_slots(int row, int base, int mask, int cnt, int split, int jump, int k, int lane,
+                                                int* lds_cols,
                                                 const int* __restrict__ col, const float* __restrict__ val,
                                                 const T* __restrict__ lhs, const T* __restrict__ rhs,
                                                 float* __restrict__ out)
@@ -48,7 +51,8 @@ __device__ __forceinline__ void sddmm_row_slots(int row, int base, int mask, int
             // still never make a lane read or write beyond its row's block part: such lanes
             // repeat the last slot and store nothing.
             const bool live = slot < cnt;
-            const int idx = base + (live ? slot : cnt - 1);
+            const int at = live ? slot : cnt - 1;
+            const int idx = base + at + (at >= split ? jump : 0);
             const int c = col[idx];
             const float v = val[idx];
             const float d = sddmm_unit<T, KT, NS, EDGE>(rhs_lane, a, c, k, lds_cols, lane);
@@ -84,7 +88,7 @@ sddmm_block_body(int bid, int nblocks, int m1, int k, RowOwners owners, const in
     if (!sddmm_block_item(seg, m1, owners, lane, block_rows, st_off, row_ptr, it)) return;
     const int row = it.row, mask = it.mask, base = it.base, cnt = it.cnt;
 
-    sddmm_row_slots<T, KT, NS, EDGE>(row, base, mask, cnt, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
+    sddmm_row_slots<T, KT, NS, EDGE>(row, base, mask, cnt, cnt, 0, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
 }
 
 // One group of LPR lanes per residue row.  Tail selection follows RoDeSddmm.cu:237-243:
@@ -206,7 +210,7 @@ sddmm_pair_kernel(int g1, int m1, int m2, int k, RowOwners owners, const int* __
 // multiplied with the lhs rows of all four rows of the group, which stay in registers.
 // Wave w then computes row w's nonzeros outside the run as usual.  Single-slab rows only
 // (k <= 128 elements per lane tile): four lhs slices of more slabs would not fit.
-template <typename T, int KT, bool EDGE>
+template <typename T, int KT, bool EDGE, int WPG>
 __global__ void __launch_bounds__(kWgThreads)
 sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
                    const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ lhs,
@@ -214,12 +218,14 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
 {
     using S = SddmmShape<T, KT>;
     constexpr int LPR = S::kLpr, VEC = S::kVec, R = kGroupRows;
+    static_assert(WPG == 1 || WPG == kWavesPerWg, "a group has one wave, or one workgroup");
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
-    const int g = xcd_logical_block(blockIdx.x, gridDim.x);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int g = xcd_logical_block(blockIdx.x, gridDim.x) * (kWavesPerWg / WPG) + wave / WPG;
     if (g >= n_groups) return;
     const RowGroup d = groups[g];
     if (d.len <= 0) return; // not a group: its rows are in the lists
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int w = wave % WPG; // this wave among the waves of its group
     const int ls = lane % LPR;
     const int row0 = g * R;
     float a[R][1][VEC];
@@ -230,9 +236,9 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
         first[r] = row_ptr[row0 + r] + d.pos[r];
     }
     const T* rhs_lane = rhs + ls * VEC;
-    // this wave's quarter of the run, in quads of columns; lane e of a step has column j0 + e
+    // this wave's share of the run, in quads of columns; lane e of a step has column j0 + e
     const int quads = (d.len + 3) / 4;
-    const int q_begin = quads * wave / kWavesPerWg, q_end = quads * (wave + 1) / kWavesPerWg;
+    const int q_begin = quads * w / WPG, q_end = quads * (w + 1) / WPG;
     const int j_end = min(d.len, 4 * q_end);
     const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
     for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
@@ -279,11 +285,15 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
             }
         }
     }
-    // row `wave`: its nonzeros before and after the run
-    const int row = row0 + wave, s = row_ptr[row], e = row_ptr[row + 1];
-    const int run_first = s + d.pos[wave], run_end = run_first + d.len;
-    sddmm_row_slots<T, KT, 1, EDGE>(row, s, 0, run_first - s, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
-    sddmm_row_slots<T, KT, 1, EDGE>(row, run_end, 0, e - run_end, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
+    // the rows this wave finishes: their nonzeros before and after the run
+#pragma unroll
+    for (int r = w; r < R; r += WPG) {
+        const int row = row0 + r, s = row_ptr[row], e = row_ptr[row + 1];
+        const int run_first = s + d.pos[r], run_end = run_first + d.len;
+        // (the slots before the run and, in the same pass, those after it)
+        sddmm_row_slots<T, KT, 1, EDGE>(row, s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, k, lane,
+                                        lds + wave * kWave, col, val, lhs, rhs, out);
+    }
 }
 
 // The rows of a hub plan, cut into pieces by column slab (rode_items.hpp): one wave per
@@ -303,7 +313,7 @@ sddmm_hub_kernel(int k, int merge, const int* __restrict__ hub, const int* __res
     const int* piece = hp.pieces + (size_t)h * (hp.slabs + 1);
     const int base = piece[slab], cnt = piece[min(slab + merge, hp.slabs)] - base;
     if (cnt <= 0) return;
-    sddmm_row_slots<T, KT, NS, EDGE>(hp.rows[h], base, 0, cnt, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
+    sddmm_row_slots<T, KT, NS, EDGE>(hp.rows[h], base, 0, cnt, cnt, 0, k, lane, lds + wave * kWave, col, val, lhs, rhs, out);
 }
 
 // Up to this many workgroups, and when both kernels go to the same stream, the two lists
@@ -373,9 +383,15 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
     }
     if constexpr (NS == 1) {
         if (e == hipSuccess && grouped) {
-            const int gg = (owners.n_groups + kXcds - 1) / kXcds * kXcds;
-            sddmm_group_kernel<T, KT, EDGE><<<gg, kWgThreads, 0, s1>>>(k, owners.n_groups, owners.groups, row_ptr, col, val,
-                                                                        lhs, rhs, out);
+            // one wave per group when there are groups enough to fill the GPU that way, else a workgroup
+            if (plan.group_counts[1] >= kGroupWaveEach) {
+                const int wgs = (owners.n_groups + kWavesPerWg - 1) / kWavesPerWg;
+                sddmm_group_kernel<T, KT, EDGE, 1><<<(wgs + kXcds - 1) / kXcds * kXcds, kWgThreads, 0, s1>>>(
+                    k, owners.n_groups, owners.groups, row_ptr, col, val, lhs, rhs, out);
+            } else {
+                sddmm_group_kernel<T, KT, EDGE, kWavesPerWg><<<(owners.n_groups + kXcds - 1) / kXcds * kXcds, kWgThreads, 0, s1>>>(
+                    k, owners.n_groups, owners.groups, row_ptr, col, val, lhs, rhs, out);
+            }
             e = hipGetLastError();
         }
     }

@@ -301,7 +301,7 @@ spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, RowOwners owner
 // from the run, no column index is read).  Wave w then adds row w's nonzeros outside the
 // run, the waves' sums meet in LDS, and wave w adds the total of row w to C (the row is in
 // no other work item: no atomics).
-template <typename T, int TN, bool EDGE>
+template <typename T, int TN, bool EDGE, int WPG>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
                   const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
@@ -310,14 +310,17 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     using S = SpmmShape<T, TN>;
     using A = typename S::Acc;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
+    constexpr int GPW = kWavesPerWg / WPG; // groups per workgroup
+    static_assert(WPG == 1 || WPG == kWavesPerWg, "a group has one wave, or one workgroup");
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg][R][kWave];
-    __shared__ __attribute__((aligned(16))) A sums[kWavesPerWg][R][TN];
-    const int g = xcd_logical_block(blockIdx.x, gridDim.x);
+    __shared__ __attribute__((aligned(16))) A sums[WPG > 1 ? kWavesPerWg : 1][R][TN];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int g = xcd_logical_block(blockIdx.x, gridDim.x) * GPW + wave / WPG;
     if (g >= n_groups) return;
     const RowGroup d = groups[g];
     if (d.len <= 0) return; // not a group: its rows are in the lists
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int w = wave % WPG; // this wave among the waves of its group
     const int ls = lane % LPR, group = lane / LPR;
     const int tile = blockIdx.y * TN;
     const bool col_ok = !EDGE || tile + ls * VEC < n;
@@ -327,9 +330,9 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
 #pragma unroll
     for (int r = 0; r < R; ++r) first[r] = row_ptr[row0 + r] + d.pos[r];
 
-    // this wave's quarter of the run, in quads of columns
+    // this wave's share of the run, in quads of columns
     const int quads = (d.len + 3) / 4;
-    const int q_begin = quads * wave / kWavesPerWg, q_end = quads * (wave + 1) / kWavesPerWg;
+    const int q_begin = quads * w / WPG, q_end = quads * (w + 1) / WPG;
     const int j_end = min(d.len, 4 * q_end);
     A acc[R][VEC];
 #pragma unroll
@@ -370,26 +373,33 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     for (int r = 0; r < R; ++r) {
 #pragma unroll
         for (int x = 0; x < VEC; ++x) acc[r][x] = butterfly_sum<LPR, kWave>(acc[r][x]);
-        if (group == 0) {
+        if (WPG > 1 && group == 0) {
 #pragma unroll
             for (int x = 0; x < VEC; ++x) sums[wave][r][ls * VEC + x] = acc[r][x];
         }
     }
-    // row `wave`: its nonzeros before and after the run
-    const int row = row0 + wave, s = row_ptr[row], e = row_ptr[row + 1];
-    const int run_first = s + d.pos[wave], run_end = run_first + d.len;
-    A outside[VEC]; // the slots before the run and, in the same pass, those after it
-    spmm_sum_slots<T, TN>(s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, lane, lds_c + wave * kWave,
-                          &lds_v[wave][0][0], b_lane, n, col, val, outside);
-    __syncthreads();
-    if (group == 0 && col_ok) {
-        A* c_lane = C + (size_t)row * n + tile + ls * VEC;
+    if (WPG > 1) __syncthreads();
+    // the rows this wave finishes: their nonzeros before and after the run, then the update of C
 #pragma unroll
-        for (int x = 0; x < VEC; ++x) {
-            A total = outside[x];
+    for (int r = w; r < R; r += WPG) {
+        const int row = row0 + r, s = row_ptr[row], e = row_ptr[row + 1];
+        const int run_first = s + d.pos[r], run_end = run_first + d.len;
+        A outside[VEC]; // the slots before the run and, in the same pass, those after it
+        spmm_sum_slots<T, TN>(s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, lane, lds_c + wave * kWave,
+                              &lds_v[wave][0][0], b_lane, n, col, val, outside);
+        if (group == 0 && col_ok) {
+            A* c_lane = C + (size_t)row * n + tile + ls * VEC;
 #pragma unroll
-            for (int w = 0; w < kWavesPerWg; ++w) total += sums[w][wave][ls * VEC + x];
-            c_lane[x] += total; // (long rows are accumulated into C by contract)
+            for (int x = 0; x < VEC; ++x) {
+                A total = outside[x];
+                if (WPG > 1) {
+#pragma unroll
+                    for (int v = 0; v < WPG; ++v) total += sums[v][r][ls * VEC + x];
+                } else {
+                    total += acc[r][x];
+                }
+                c_lane[x] += total; // (long rows are accumulated into C by contract)
+            }
         }
     }
 }
@@ -594,9 +604,18 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
         e = hipGetLastError();
     }
     if (e == hipSuccess && grouped) {
-        const int gg = (owners.n_groups + kXcds - 1) / kXcds * kXcds;
-        dim3 grid(gg, tiles);
-        spmm_group_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(n, owners.n_groups, owners.groups, row_ptr, col, val, B, C);
+        // one wave per group when there are groups enough to fill the GPU that way (measured on
+        // the attention-mask benchmark, 4096 groups: 0.042 against 0.062 ms), else a workgroup
+        if (plan.group_counts[1] >= kGroupWaveEach) {
+            const int wgs = (owners.n_groups + kWavesPerWg - 1) / kWavesPerWg;
+            dim3 grid((wgs + kXcds - 1) / kXcds * kXcds, tiles);
+            spmm_group_kernel<T, TN, EDGE, 1><<<grid, kWgThreads, 0, s1>>>(n, owners.n_groups, owners.groups, row_ptr, col,
+                                                                           val, B, C);
+        } else {
+            dim3 grid((owners.n_groups + kXcds - 1) / kXcds * kXcds, tiles);
+            spmm_group_kernel<T, TN, EDGE, kWavesPerWg><<<grid, kWgThreads, 0, s1>>>(n, owners.n_groups, owners.groups, row_ptr,
+                                                                                     col, val, B, C);
+        }
         e = hipGetLastError();
     }
     if constexpr (!std::is_same<T, double>::value) {

@@ -103,6 +103,30 @@ def test_grouped_rows_against_oracle(k, half):
         assert np.abs(C.cpu().numpy() - want).max() <= 1e-12 * max(1.0, np.abs(want).max())
 
 
+@pytest.mark.parametrize("half", [False, True])
+def test_one_wave_per_group(half):
+    """From 2048 groups with a run on, a group is the work of one wave instead of one
+    workgroup (no sums through LDS): the same checks on a matrix with about 2250 such groups."""
+    import oracle
+    from gpu_common import TOL_F16, TOL_F32, make_csr, round_half, run_sddmm, run_spmm
+    from helpers import spmm_row_l1_error, sddmm_row_l1_errors
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(11)
+    m, n, k = 12002, 12500, 64
+    rp, col, val = _window_matrix(rng, m, n, 96, 6)
+    csr = make_csr(rp, col, val, m, n, k, locality=True)
+    assert isinstance(csr.plan, rode_sddmm_hip.GroupPlan) and csr.plan.counts[1] >= 2048
+    assert 0 < csr.plan.counts[2] < m   # some rows are left to the other kernels
+    B = rng.standard_normal((n, k)).astype(np.float32)
+    L = rng.standard_normal((m, k)).astype(np.float32)
+    Bq, Lq = (round_half(B), round_half(L)) if half else (B, L)
+    tol = TOL_F16 if half else TOL_F32
+    assert spmm_row_l1_error(run_spmm(csr, B, half), oracle.spmm_f64(rp, col, val, Bq)) <= tol
+    ref64, scale = oracle.sddmm_f64(rp, col, val, Lq, Bq, with_abs=True)
+    err, cond = sddmm_row_l1_errors(run_sddmm(csr, L, B, half), ref64, scale, rp)
+    assert float(err[cond <= 100].max(initial=0.0)) <= tol
+
+
 def test_every_nonzero_has_one_owner_and_what_is_refused():
     import ctypes
     from gpu_common import DEV, make_csr
