@@ -217,7 +217,7 @@ def main():
             _lib.check(lib.rode_hip_attention_forward(
                 _lib.DENSE_CODE[args.dtype], m, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
                 csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), B.data_ptr(), float(k) ** -0.5, C.data_ptr(),
-                probs.data_ptr() if args.fused == "probs" else None, stream), "attention")
+                probs.data_ptr() if args.fused == "probs" else None, sddmm_plans, stream), "attention")
             return
         if args.chain:
             sddmm(csr.m1, csr.m2)

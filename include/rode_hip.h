@@ -360,10 +360,14 @@ int rode_hip_csr_softmax_backward_f32(int M, const int* d_row_offsets, const flo
  *   d_q [M x d], d_k, d_v [columns x d]   row-major, 16-byte aligned
  *   d_out        float [M x d]; rows without nonzeros are written as zeros
  *   d_probs      NULL, or float [nnz] that receives p (what a gradient needs)
+ *   plans        NULL, or the plans of this pattern: a group plan with at least 2048 groups
+ *                with a run is used (the rows of a group then share one wave, and every k
+ *                and v row of the group's run is loaded once for its four rows); the other
+ *                plans are ignored
  */
 int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
                                const float* d_values, const void* d_q, const void* d_k, const void* d_v,
-                               float scale, float* d_out, float* d_probs, void* stream);
+                               float scale, float* d_out, float* d_probs, const rode_hip_plans* plans, void* stream);
 
 /*
  * The transposed pattern of a CSR matrix (M rows, N columns, nnz nonzeros): what the

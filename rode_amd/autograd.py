@@ -130,11 +130,14 @@ def _attention_call(csr, values, q, k, v, scale, want_probs):
     if values.numel() == 0:  # no nonzeros: nothing attends to anything
         return torch.zeros((m, d), dtype=torch.float32, device=q.device), probs
     out = torch.empty((m, d), dtype=torch.float32, device=q.device)
+    import ctypes
+    plans = rode_sddmm_hip.plans_struct(csr.plan if isinstance(csr.plan, rode_sddmm_hip.GroupPlan) else None)
     with torch.cuda.device(q.device):
         code = lib.rode_hip_attention_forward(
             _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"], m, d, csr.row_offsets.data_ptr(),
             csr.column_indices.data_ptr(), values.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale),
-            out.data_ptr(), probs.data_ptr() if want_probs else None, torch.cuda.current_stream(q.device).cuda_stream)
+            out.data_ptr(), probs.data_ptr() if want_probs else None, ctypes.byref(plans),
+            torch.cuda.current_stream(q.device).cuda_stream)
     _lib.check(code, "rode_hip_attention_forward")
     return out, probs
 

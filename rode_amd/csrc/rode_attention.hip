@@ -20,6 +20,7 @@
 // request (the gradient needs them): the raw scores of a row's first 1024 slots wait in
 // LDS (those of longer rows in the output array itself) until maximum and sum are known,
 // then the lanes that produced them normalise and store them.
+#include "rode_items.hpp"
 #include "rode_units.hpp"
 #include "rode_internal.hpp"
 
@@ -46,7 +47,7 @@ template <typename T, int D, bool WRITE_P>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                       const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, float scale,
-                      float* __restrict__ out, float* probs)
+                      float* __restrict__ out, float* probs, RowOwners owners)
 {
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
@@ -56,6 +57,7 @@ attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restr
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int row = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (row >= M) return;
+    if (owned_elsewhere(owners, row, 0)) return; // a row of a group: attention_group_kernel has it
     const int s = row_ptr[row], e = row_ptr[row + 1];
     const int ls = lane % LPR, group = lane / LPR;
     float* out_lane = out + (size_t)row * D + ls * VEC;
@@ -130,17 +132,222 @@ attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restr
     }
 }
 
+// One step of the running softmax of a row: the scores of up to 64 slots (sc, -inf for a
+// lane without a slot) move the maximum; the row's sum and accumulated output are rescaled.
+// Returns this lane's probability relative to the new maximum.
+template <int VEC>
+__device__ __forceinline__ float softmax_step(float sc, bool live, float& m_run, float& l_lane, float (&acc)[VEC])
+{
+    const float m_new = fmaxf(m_run, wave_max_f(sc));
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = __expf(m_run - m_safe);
+    const float p = live ? __expf(sc - m_safe) : 0.f;
+    l_lane = fmaf(l_lane, corr, p);
+#pragma unroll
+    for (int x = 0; x < VEC; ++x) acc[x] *= corr;
+    m_run = m_new;
+    return p;
+}
+
+// The groups of a group plan (rode_group.hip): one wave per group of four adjacent rows
+// that share a run of consecutive columns.  Along the run every k row and every v row is
+// loaded once for the four rows (the score part is the SDDMM group kernel's, the output
+// part the SpMM group kernel's, with a running softmax per row in between); then the wave
+// takes the nonzeros outside the run, row by row, the way attention_rows_kernel does.
+// Raw scores wait in the probs array itself; the lanes that wrote them normalise them.
+template <typename T, int D, bool WRITE_P>
+__global__ void __launch_bounds__(kWgThreads)
+attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
+                       const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ q,
+                       const T* __restrict__ k, const T* __restrict__ v, float scale, float* __restrict__ out,
+                       float* probs)
+{
+    using S = SpmmShape<T, D>;
+    constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
+    constexpr int QUADS = LPR / 4; // slot quads per lane group per 32-slot unit (SddmmShape::kQuads)
+    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
+    __shared__ __attribute__((aligned(16))) float lds_p[kWavesPerWg][R][kWave];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int g = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
+    if (g >= n_groups) return;
+    const RowGroup d = groups[g];
+    if (d.len <= 0) return; // not a group: attention_rows_kernel has its rows
+    const int ls = lane % LPR, group = lane / LPR;
+    const int row0 = g * R;
+    float a[R][1][VEC];
+    int first[R]; // where the run starts in column_indices / values, per row
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        load_lhs_slice<T, D, 1, false>(q, row0 + r, D, lane, a[r]);
+        first[r] = row_ptr[row0 + r] + d.pos[r];
+    }
+    const T* k_lane = k + ls * VEC;
+    const T* v_lane = v + ls * VEC;
+    int* my_c = lds_c + wave * kWave;
+    float m_run[R], l_lane[R], acc[R][VEC];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        m_run[r] = -INFINITY;
+        l_lane[r] = 0.f;
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) acc[r][x] = 0.f;
+    }
+
+    // the run: lane e of a step has column j0 + e
+    const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
+    for (int j0 = 0; j0 < d.len; j0 += kWave) {
+        const int j = j0 + lane;
+        const bool live = j < d.len;
+        float dot[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) dot[r] = 0.f;
+        if (j0 + (lane & 32) < d.len) { // the upper half sits out a step that has nothing for it
+#pragma unroll
+            for (int qd = 0; qd < QUADS; ++qd) {
+                float p4[R][4];
+                const T* k_quad = k_lane + (size_t)(d.lo + j0 + group_first + 4 * qd) * D;
+                const int room = d.len - 1 - (j0 + group_first + 4 * qd); // (rows past the run repeat its last row)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    float b[VEC];
+                    DenseVec<T>::load(k_quad + (ptrdiff_t)min(t, room) * D, b);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        float sum = 0.f;
+#pragma unroll
+                        for (int x = 0; x < VEC; ++x) sum = fmaf(a[r][0][x], b[x], sum);
+                        p4[r][t] = sum;
+                    }
+                }
+                const bool hi2 = ls & 2, hi1 = ls & 1;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const float q0 = (hi2 ? p4[r][2] : p4[r][0]) + lane_xor2(hi2 ? p4[r][0] : p4[r][2]);
+                    const float q1 = (hi2 ? p4[r][3] : p4[r][1]) + lane_xor2(hi2 ? p4[r][1] : p4[r][3]);
+                    float sum = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
+                    sum = butterfly_sum<4, LPR>(sum);
+                    if ((ls >> 2) == qd) dot[r] = sum;
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float sc = live ? scale * (val[first[r] + j] * dot[r]) : -INFINITY;
+            lds_p[wave][r][lane] = softmax_step<VEC>(sc, live, m_run[r], l_lane[r], acc[r]);
+            if (WRITE_P && live) probs[first[r] + j] = sc;
+        }
+        wave_lds_sync();
+        const int nq = min(kWave / 4, (d.len - j0 + 3) / 4);
+#pragma unroll
+        for (int i = 0; i < kWave / 4 / G; ++i) {
+            const int qd = group + i * G;
+            if (qd < nq) {
+                const T* v_quad = v_lane + (size_t)(d.lo + j0 + 4 * qd) * D;
+                const int room = d.len - 1 - (j0 + 4 * qd);
+                float b[4][VEC];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) DenseVec<T>::load(v_quad + (ptrdiff_t)min(t, room) * D, b[t]);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const float4 p4 = *reinterpret_cast<const float4*>(&lds_p[wave][r][4 * qd]);
+                    const float pv[4] = {p4.x, p4.y, p4.z, p4.w};
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+#pragma unroll
+                        for (int x = 0; x < VEC; ++x) acc[r][x] = fmaf(pv[t], b[t][x], acc[r][x]);
+                }
+            }
+        }
+        wave_lds_sync();
+    }
+
+    // the nonzeros outside the run, row by row: the slots before it and, in the same pass, those after it
+    float* my_p = lds_p[wave][0];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int s = row_ptr[row0 + r], e = row_ptr[row0 + r + 1];
+        const int split = d.pos[r], cnt = split + (e - (s + split + d.len));
+        for (int off = 0; off < cnt; off += kWave) {
+            const int slot = off + lane;
+            const bool live = slot < cnt;
+            const int at = live ? slot : cnt - 1;
+            const int idx = s + at + (at >= split ? d.len : 0);
+            const int c = col[idx];
+            const float w = val[idx];
+            float sc = -INFINITY;
+            if (off + (lane & 32) < cnt) {
+                const float dd = sddmm_unit<T, D, 1, false>(k_lane, a[r], c, D, my_c, lane);
+                if (live) sc = scale * (w * dd);
+            }
+            my_p[lane] = softmax_step<VEC>(sc, live, m_run[r], l_lane[r], acc[r]);
+            if (WRITE_P && live) probs[idx] = sc;
+            wave_lds_sync();
+            const int nlive = min(cnt - off, kWave);
+            if (nlive == kWave)
+                spmm_gather<T, D, 16 / G, true>(v_lane, (size_t)D, acc[r], my_c, my_p, group, G, 16);
+            else
+                spmm_gather<T, D, 16 / G, false>(v_lane, (size_t)D, acc[r], my_c, my_p, group, G, (nlive + 3) / 4);
+            wave_lds_sync();
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float inv = 1.0f / butterfly_sum<1, kWave>(l_lane[r]);
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) acc[r][x] = butterfly_sum<LPR, kWave>(acc[r][x]) * inv;
+        if (group == 0) {
+            float* out_lane = out + (size_t)(row0 + r) * D + ls * VEC;
+#pragma unroll
+            for (int x = 0; x < VEC; x += 4)
+                *reinterpret_cast<float4*>(out_lane + x) = make_float4(acc[r][x], acc[r][x + 1], acc[r][x + 2], acc[r][x + 3]);
+        }
+        if (WRITE_P) {
+            // every lane normalises the scores it wrote itself: same walk over the run and over the rest
+            const float m_safe = m_run[r] == -INFINITY ? 0.f : m_run[r];
+            for (int j = lane; j < d.len; j += kWave) probs[first[r] + j] = __expf(probs[first[r] + j] - m_safe) * inv;
+            const int s = row_ptr[row0 + r], e = row_ptr[row0 + r + 1];
+            const int split = d.pos[r], cnt = split + (e - (s + split + d.len));
+            for (int slot = lane; slot < cnt; slot += kWave) {
+                const int idx = s + slot + (slot >= split ? d.len : 0);
+                probs[idx] = __expf(probs[idx] - m_safe) * inv;
+            }
+        }
+    }
+}
+
 template <typename T, int D>
 hipError_t launch_rows(int M, const int* row_ptr, const int* col, const float* val, const T* q, const T* k, const T* v,
-                       float scale, float* out, float* probs, hipStream_t stream)
+                       float scale, float* out, float* probs, PlanRef plan, hipStream_t stream)
 {
     long long wgs = ((long long)M + kWavesPerWg - 1) / kWavesPerWg;
     wgs = (wgs + kXcds - 1) / kXcds * kXcds;
     if (wgs * kWgThreads >= (1ll << 32)) return hipErrorInvalidConfiguration;
-    if (probs)
-        attention_rows_kernel<T, D, true><<<(int)wgs, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out, probs);
-    else
-        attention_rows_kernel<T, D, false><<<(int)wgs, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out, probs);
+    // a group plan is used when a wave per group fills the GPU
+    RowOwners owners;
+    const bool grouped = plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] >= kGroupWaveEach;
+    if (grouped) {
+        owners.groups = reinterpret_cast<const RowGroup*>(plan.groups + kGroupHeaderInts);
+        owners.n_groups = plan.group_counts[0];
+    }
+    if (!(grouped && plan.group_counts[2] == 0)) { // (else every row is in a group)
+        if (probs)
+            attention_rows_kernel<T, D, true><<<(int)wgs, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out,
+                                                                                   probs, owners);
+        else
+            attention_rows_kernel<T, D, false><<<(int)wgs, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out,
+                                                                                    probs, owners);
+    }
+    if (grouped) {
+        int gw = (owners.n_groups + kWavesPerWg - 1) / kWavesPerWg;
+        gw = (gw + kXcds - 1) / kXcds * kXcds;
+        if (probs)
+            attention_group_kernel<T, D, true><<<gw, kWgThreads, 0, stream>>>(owners.n_groups, owners.groups, row_ptr, col, val,
+                                                                              q, k, v, scale, out, probs);
+        else
+            attention_group_kernel<T, D, false><<<gw, kWgThreads, 0, stream>>>(owners.n_groups, owners.groups, row_ptr, col,
+                                                                               val, q, k, v, scale, out, probs);
+    }
     return hipGetLastError();
 }
 
@@ -149,20 +356,20 @@ hipError_t launch_rows(int M, const int* row_ptr, const int* col, const float* v
 // d: width of q, k and v rows (32, 64 or 128).  probs: NULL or nnz floats.
 template <typename T>
 hipError_t attention_launch(int M, int d, const int* row_ptr, const int* col, const float* val, const T* q, const T* k,
-                            const T* v, float scale, float* out, float* probs, hipStream_t stream)
+                            const T* v, float scale, float* out, float* probs, PlanRef plan, hipStream_t stream)
 {
     if (M <= 0) return hipSuccess;
     switch (d) {
-    case 32: return launch_rows<T, 32>(M, row_ptr, col, val, q, k, v, scale, out, probs, stream);
-    case 64: return launch_rows<T, 64>(M, row_ptr, col, val, q, k, v, scale, out, probs, stream);
-    case 128: return launch_rows<T, 128>(M, row_ptr, col, val, q, k, v, scale, out, probs, stream);
+    case 32: return launch_rows<T, 32>(M, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
+    case 64: return launch_rows<T, 64>(M, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
+    case 128: return launch_rows<T, 128>(M, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
 template hipError_t attention_launch<float>(int, int, const int*, const int*, const float*, const float*, const float*,
-                                            const float*, float, float*, float*, hipStream_t);
+                                            const float*, float, float*, float*, PlanRef, hipStream_t);
 template hipError_t attention_launch<__half>(int, int, const int*, const int*, const float*, const __half*, const __half*,
-                                             const __half*, float, float*, float*, hipStream_t);
+                                             const __half*, float, float*, float*, PlanRef, hipStream_t);
 
 } // namespace rode

@@ -353,20 +353,28 @@ int rode_hip_csr_softmax_backward_f32(int M, const int* d_row_offsets, const flo
 
 int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
                                const float* d_values, const void* d_q, const void* d_k, const void* d_v,
-                               float scale, float* d_out, float* d_probs, void* stream)
+                               float scale, float* d_out, float* d_probs, const rode_hip_plans* plans, void* stream)
 {
     if (M < 0 || !d_row_offsets) return hipErrorInvalidValue;
+    rode::PlanRef plan;
+    if (plans && plans->groups) { // only a group plan means anything to this kernel
+        rode_hip_plans only_groups = {};
+        only_groups.groups = plans->groups;
+        only_groups.group_counts = plans->group_counts;
+        if (!plan_ref(&only_groups, 0, plan) || plan.group_counts[0] != rode::row_groups(M)) return hipErrorInvalidValue;
+    }
     if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
     if (M > 0 && (!d_column_indices || !d_values || !d_q || !d_k || !d_v || !d_out)) return hipErrorInvalidValue;
     if (!aligned16(d_q) || !aligned16(d_k) || !aligned16(d_v) || !aligned16(d_out)) return hipErrorInvalidValue;
     if (dtype == RODE_DENSE_F32)
         return rode::attention_launch<float>(M, d, d_row_offsets, d_column_indices, d_values, static_cast<const float*>(d_q),
                                              static_cast<const float*>(d_k), static_cast<const float*>(d_v), scale, d_out,
-                                             d_probs, as_stream(stream));
+                                             d_probs, plan, as_stream(stream));
     if (dtype == RODE_DENSE_F16)
         return rode::attention_launch<__half>(M, d, d_row_offsets, d_column_indices, d_values,
                                               static_cast<const __half*>(d_q), static_cast<const __half*>(d_k),
-                                              static_cast<const __half*>(d_v), scale, d_out, d_probs, as_stream(stream));
+                                              static_cast<const __half*>(d_v), scale, d_out, d_probs, plan,
+                                              as_stream(stream));
     return hipErrorInvalidValue;
 }
 

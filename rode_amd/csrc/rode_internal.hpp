@@ -47,6 +47,11 @@ struct PlanRef {
 
 hipError_t group_plan_launch(int M, const int* row_ptr, const int* col, int* plan, hipStream_t stream);
 
+// (plan: only a group plan is used)
+template <typename T>
+hipError_t attention_launch(int M, int d, const int* row_ptr, const int* col, const float* val, const T* q, const T* k,
+                            const T* v, float scale, float* out, float* probs, PlanRef plan, hipStream_t stream);
+
 hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, const int* col, int* plan,
                            hipStream_t stream);
 
@@ -79,9 +84,6 @@ template <typename T>
 hipError_t sddmm_window_launch(int m2, int k, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
                                const int* plan, const void* plan_rows, hipStream_t stream);
 
-template <typename T>
-hipError_t attention_launch(int M, int d, const int* row_ptr, const int* col, const float* val, const T* q, const T* k,
-                            const T* v, float scale, float* out, float* probs, hipStream_t stream);
 size_t csr_transpose_workspace_bytes(int nnz);
 hipError_t csr_transpose_launch(int M, int N, int nnz, const int* row_ptr, const int* col, int* t_row_ptr, int* t_col,
                                 int* perm, void* workspace, hipStream_t stream);

@@ -180,3 +180,48 @@ def test_every_nonzero_has_one_owner_and_what_is_refused():
     assert code == 0 and all(c == 0 for c, _ in parts)
     assert (sum(p for _, p in parts) - plain_c).abs().max().item() <= 2e-5 * plain_c.abs().max().item()
     assert spmm(0, plans())[0] != 0  # a group plan without the whole-lists promise
+
+
+@pytest.mark.parametrize("d,half", [(64, False), (64, True), (128, False), (32, True)])
+def test_fused_attention_of_groups(d, half):
+    """rode_hip_attention_forward with a group plan of at least 2048 groups with a run (one
+    wave per group: scores of the run for four rows at once, then their softmax, then P.V
+    over the run) against fp64 on the host and against the same entry point without a plan;
+    rows in no kept group, rows with holes, empty rows and short rows are all in the matrix."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import rode_sddmm_hip
+    from rode_amd.autograd import _attention_call
+    rng = np.random.default_rng(40 + d)
+    m, n = 12002, 12500
+    rp, col, val = _window_matrix(rng, m, n, 96, 6)
+    val = rng.uniform(0.5, 1.5, len(col)).astype(np.float32)
+    mask = make_csr(rp, col, val, m, n, d, locality=True)
+    assert isinstance(mask.plan, rode_sddmm_hip.GroupPlan) and mask.plan.counts[1] >= 2048
+    plain = make_csr(rp, col, val, m, n, d, locality=False)
+    assert plain.plan is None
+    dt = torch.float16 if half else torch.float32
+    mk = lambda r, s: torch.from_numpy((s * rng.standard_normal((r, d))).astype(np.float32)).to(DEV, dt)
+    q, k, v = mk(m, 1.2), mk(n, 1.2), mk(n, 1.0)
+    scale = 0.4
+    out, probs = _attention_call(mask, mask.values, q, k, v, scale, True)
+    out_only, none = _attention_call(mask, mask.values, q, k, v, scale, False)
+    assert none is None and torch.equal(out, out_only)
+    q64, k64, v64 = (t.double().cpu().numpy() for t in (q, k, v))
+    lens = np.diff(rp)
+    rows = np.repeat(np.arange(m), lens)
+    sc = scale * val.astype(np.float64) * np.einsum("ij,ij->i", q64[rows], k64[col])
+    top = np.full(m, -np.inf)
+    np.maximum.at(top, rows, sc)
+    e = np.exp(sc - top[rows])
+    den = np.zeros(m)
+    np.add.at(den, rows, e)
+    ref_p = e / den[rows]
+    ref_out = np.zeros((m, d))
+    np.add.at(ref_out, rows, ref_p[:, None] * v64[col])
+    tol = 2e-3 if half else 5e-5
+    assert np.abs(probs.cpu().numpy() - ref_p).max() <= tol
+    assert np.abs(out.cpu().numpy() - ref_out).max() <= tol * max(1.0, np.abs(ref_out).max())
+    assert not out[torch.from_numpy(lens == 0).to(DEV)].any()
+    out2, probs2 = _attention_call(plain, plain.values, q, k, v, scale, True)
+    assert (out - out2).abs().max().item() <= tol * max(1.0, out2.abs().max().item())
+    assert (probs - probs2).abs().max().item() <= tol
