@@ -72,17 +72,20 @@ def parse_args():
     return p.parse_args()
 
 
-def work_split(row_ptr, col, ncols, owned_slots=0, hub_min_len=0):
+def work_split(row_ptr, col, ncols, owned_slots=0, hub_min_len=0, group_rows=None):
     """Which nonzeros the residue kernels own (tail rule of RoDeSpmm.cu:71-82) and how
     many distinct dense rows each kernel family touches.  ``owned_slots``: rows of
     32..owned_slots aligned slots are summed, tail included, by the SpMM block kernel.
     ``hub_min_len`` > 0: rows of at least that many aligned slots belong, whole, to the
-    hub kernels."""
+    hub kernels.  ``group_rows``: mask of the rows that belong, whole, to the group kernels
+    (counted under the same "hub" keys: a plan is one or the other)."""
     rp = row_ptr.astype(np.int64)
     s, e = rp[:-1], rp[1:]
     pad = s % 4
     N = e - s + pad
     hub_row = (N >= hub_min_len) if hub_min_len > 0 else np.zeros(len(N), dtype=bool)
+    if group_rows is not None:
+        hub_row = group_rows
     tail_first = np.where(N >= 32, s - pad + N // 32 * 32, s)
     tail_first = np.where((N >= 32) & (N <= owned_slots), e, tail_first)
     in_hub = np.repeat(hub_row, e - s)
@@ -101,7 +104,7 @@ def algorithmic_bytes(kernel, split, m1, m2, k, elem):
     """Compulsory traffic of one launch: every array element it needs, once."""
     if kernel.endswith("block"):
         nnz, rows, distinct, meta = split["nnz_blk"], split["rows_blk"], split["distinct_blk"], m1 * 12 + 4
-    elif kernel.endswith("hub"):
+    elif kernel.endswith("hub") or kernel.endswith("group"):  # (a group: 32 bytes of plan for four rows)
         nnz, rows, distinct, meta = split["nnz_hub"], split["rows_hub"], split["distinct_hub"], split["rows_hub"] * 12
     else:
         nnz, rows, distinct, meta = split["nnz_res"], m2, split["distinct_res"], m2 * 12
@@ -147,6 +150,8 @@ def main():
     stream = torch.cuda.current_stream().cuda_stream
     import ctypes
     hub = csr.plan if isinstance(csr.plan, rode_sddmm_hip.HubPlan) else None
+    grp = csr.plan if isinstance(csr.plan, rode_sddmm_hip.GroupPlan) else None
+    lists_run = grp is None or grp.counts[2] > 0  # (with every row in a group the list kernels are not launched)
     spmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan, k, 4))
     sddmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan))
 
@@ -287,15 +292,18 @@ def main():
     preprocess_ms = event_time(preprocess, reps)
     del p_blk, p_st, p_res, p_ws
     kernels = {}
-    if csr.m1 > 0:
+    if csr.m1 > 0 and lists_run:
         kernels["spmm_block"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_BLOCK), reps)  # incl. rows summed whole
         kernels["sddmm_block"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_BLOCK), reps)
-    if csr.m2 > 0:
+    if csr.m2 > 0 and lists_run:
         kernels["spmm_residue"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_RESIDUE), reps)
         kernels["sddmm_residue"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_RESIDUE), reps)
     if hub is not None:  # the rows of the hub plan: piece kernel (+ the sum of the partial rows of C for SpMM)
         kernels["spmm_hub"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_HUB), reps)
         kernels["sddmm_hub"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_HUB), reps)
+    if grp is not None:  # the rows of the group plan's groups (the same flag selects them)
+        kernels["spmm_group"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_HUB), reps)
+        kernels["sddmm_group"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_HUB), reps)
     spmm_ms = event_time(lambda: (clear_c(), spmm(csr.m1, csr.m2)), reps)
     sddmm_ms = event_time(lambda: sddmm(csr.m1, csr.m2), reps)
     spmm_contract_ms = event_time(spmm_reference_contract, reps)
@@ -309,8 +317,12 @@ def main():
 
     # the SpMM block kernel sums rows of 32..1024 slots whole when there are >= 16384 segments
     hub_min_len = hub.counts[2] if hub is not None else 0
-    split_sddmm = work_split(row_ptr, col, n, 0, hub_min_len)
-    split_spmm = work_split(row_ptr, col, n, 1024 if csr.m1 >= 16384 else 0, hub_min_len)
+    group_rows = None
+    if grp is not None:
+        group_rows = np.zeros(m, dtype=bool)
+        group_rows[: 4 * grp.counts[0]] = np.repeat(grp.groups()[:, 1] > 0, 4)
+    split_sddmm = work_split(row_ptr, col, n, 0, hub_min_len, group_rows)
+    split_spmm = work_split(row_ptr, col, n, 1024 if csr.m1 >= 16384 else 0, hub_min_len, group_rows)
     per_kernel = {}
     for name, ms in kernels.items():
         split = split_spmm if name.startswith("spmm") else split_sddmm
@@ -318,7 +330,7 @@ def main():
         if name == "spmm_residue":
             m2_eff = split["rows_res"]
         ab = algorithmic_bytes(name, split, csr.m1, m2_eff, k, elem)
-        knnz = split["nnz_" + {"block": "blk", "residue": "res", "hub": "hub"}[name.split("_")[1]]]
+        knnz = split["nnz_" + {"block": "blk", "residue": "res", "hub": "hub", "group": "hub"}[name.split("_")[1]]]
         per_kernel[name] = {"ms": round(ms, 4), "algorithmic_bytes": ab,
                             "algorithmic_GBs": round(ab / ms / 1e6, 1),
                             "gather_model_GBs": round((knnz * (8 + k * elem)) / ms / 1e6, 1),
@@ -330,7 +342,7 @@ def main():
         table = json.load(open(tpath))
         prefix = f"{args.workload}/k{k}/{args.dtype}/seg{csr.config['seg_length']}/"
         # with a locality plan the residue rows are the window kernel's
-        windowed = csr.plan is not None and hub is None and dominant.endswith("residue") and k * elem > 128
+        windowed = csr.plan is not None and hub is None and grp is None and dominant.endswith("residue") and k * elem > 128
         entry = table.get(prefix + dominant + "_window") if windowed else None
         entry = entry or table.get(prefix + dominant)
         if entry is not None and entry.get("sources") == kernel_sources_fingerprint():
@@ -462,11 +474,14 @@ def main():
                                   else "step = clear C rows + SpMM + SDDMM"),
                    "rows": m, "cols": n, "nnz": nnz, "K": k, "seg_length": csr.config["seg_length"],
                    "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale,
-                   "locality_plan": None if csr.plan is None or hub is not None else
+                   "locality_plan": None if csr.plan is None or hub is not None or grp is not None else
                    {"residue_chunks": csr.plan.counts[0], "chunks_with_lds_window": csr.plan.counts[1]},
                    "hub_plan": None if hub is None else
                    {"hub_rows": hub.counts[0], "shortest": hub.counts[2], "nnz_share": round(split_sddmm["nnz_hub"] / nnz, 3),
-                    "column_slabs": hub.counts[1], "slab_rows": 2048}},
+                    "column_slabs": hub.counts[1], "slab_rows": 2048},
+                   "group_plan": None if grp is None else
+                   {"groups_of_four_rows": grp.counts[0], "groups_with_a_shared_run": grp.counts[1],
+                    "rows_left_to_the_list_kernels": grp.counts[2], "nnz_share": round(split_sddmm["nnz_hub"] / nnz, 3)}},
         "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C",
                  "reference_contract_ms": round(spmm_contract_ms, 4),
                  "reference_contract": "memset of all of C + the typed entry point without the whole-lists promise "

@@ -73,7 +73,7 @@ attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restr
         return;
     }
 
-    float a[1][VEC];
+    typename DotVec<T>::Reg a[1][DotVec<T>::kRegs];
     load_lhs_slice<T, D, 1, false>(q, row, D, lane, a);
     const T* k_lane = k + ls * VEC;
     const T* v_lane = v + ls * VEC;
@@ -156,7 +156,7 @@ __device__ __forceinline__ float softmax_step(float sc, bool live, float& m_run,
 // takes the nonzeros outside the run, row by row, the way attention_rows_kernel does.
 // Raw scores wait in the probs array itself; the lanes that wrote them normalise them.
 template <typename T, int D, bool WRITE_P>
-__global__ void __launch_bounds__(kWgThreads)
+__global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
                        const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ q,
                        const T* __restrict__ k, const T* __restrict__ v, float scale, float* __restrict__ out,
@@ -174,7 +174,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     if (d.len <= 0) return; // not a group: attention_rows_kernel has its rows
     const int ls = lane % LPR, group = lane / LPR;
     const int row0 = g * R;
-    float a[R][1][VEC];
+    typename DotVec<T>::Reg a[R][1][DotVec<T>::kRegs];
     int first[R]; // where the run starts in column_indices / values, per row
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -209,15 +209,9 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
                 const int room = d.len - 1 - (j0 + group_first + 4 * qd); // (rows past the run repeat its last row)
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    float b[VEC];
-                    DenseVec<T>::load(k_quad + (ptrdiff_t)min(t, room) * D, b);
+                    const uint4 b = *reinterpret_cast<const uint4*>(k_quad + (ptrdiff_t)min(t, room) * D);
 #pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        float sum = 0.f;
-#pragma unroll
-                        for (int x = 0; x < VEC; ++x) sum = fmaf(a[r][0][x], b[x], sum);
-                        p4[r][t] = sum;
-                    }
+                    for (int r = 0; r < R; ++r) p4[r][t] = DotVec<T>::dot_raw(a[r][0], b, 0.f);
                 }
                 const bool hi2 = ls & 2, hi1 = ls & 1;
 #pragma unroll

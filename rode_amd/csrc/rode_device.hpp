@@ -133,6 +133,64 @@ struct DenseVec<__half> {
     }
 };
 
+// The left operand of a dot product as a lane keeps it (DenseVec<T>::kElems elements), and
+// its dot product with as many consecutive elements of the right operand, accumulated in
+// fp32.  fp32: one fused multiply-add per element.  fp16: the pairs stay packed as loaded
+// and go through v_dot2c_f32_f16 (two products, exact in fp32, and the sum per
+// instruction; no conversion instructions).
+template <typename T>
+struct DotVec {
+    using Reg = float;
+    static constexpr int kRegs = DenseVec<T>::kElems;
+    __device__ __forceinline__ static void zero(Reg (&a)[kRegs])
+    {
+#pragma unroll
+        for (int x = 0; x < kRegs; ++x) a[x] = 0.f;
+    }
+    __device__ __forceinline__ static void load(const T* p, Reg (&a)[kRegs]) { DenseVec<T>::load(p, a); }
+    __device__ __forceinline__ static float dot_raw(const Reg (&a)[kRegs], const uint4& raw, float acc)
+    {
+        float b[kRegs];
+        DenseVec<T>::unpack(raw, b);
+#pragma unroll
+        for (int x = 0; x < kRegs; ++x) acc = fmaf(a[x], b[x], acc);
+        return acc;
+    }
+    __device__ __forceinline__ static float dot(const Reg (&a)[kRegs], const T* p, float acc)
+    {
+        return dot_raw(a, *reinterpret_cast<const uint4*>(p), acc);
+    }
+};
+
+template <>
+struct DotVec<__half> {
+    using Reg = uint32_t; // two fp16 elements
+    static constexpr int kRegs = 4;
+    typedef _Float16 Pair __attribute__((ext_vector_type(2)));
+    __device__ __forceinline__ static void zero(Reg (&a)[kRegs])
+    {
+#pragma unroll
+        for (int x = 0; x < kRegs; ++x) a[x] = 0u;
+    }
+    __device__ __forceinline__ static void load(const __half* p, Reg (&a)[kRegs])
+    {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        a[0] = raw.x; a[1] = raw.y; a[2] = raw.z; a[3] = raw.w;
+    }
+    __device__ __forceinline__ static float dot_raw(const Reg (&a)[kRegs], const uint4& raw, float acc)
+    {
+        const uint32_t b[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int x = 0; x < kRegs; ++x)
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(Pair, a[x]), __builtin_bit_cast(Pair, b[x]), acc, false);
+        return acc;
+    }
+    __device__ __forceinline__ static float dot(const Reg (&a)[kRegs], const __half* p, float acc)
+    {
+        return dot_raw(a, *reinterpret_cast<const uint4*>(p), acc);
+    }
+};
+
 // Make LDS writes of this wave visible to its other lanes.  A wave executes its
 // LDS instructions in order, so only the compiler has to be kept from moving
 // accesses across this point.

@@ -39,7 +39,7 @@ __device__ __forceinline__ void sddmm_row_slots(int row, int base, int mask, int
                                                 float* __restrict__ out)
 {
     using S = SddmmShape<T, KT>;
-    float a[NS][S::kVec];
+    typename S::Reg a[NS][S::kRegs];
     load_lhs_slice<T, KT, NS, EDGE>(lhs, row, k, lane, a);
     const T* rhs_lane = rhs + (lane % S::kLpr) * S::kVec;
 
@@ -133,7 +133,7 @@ sddmm_residue_body(int bid, int nblocks, int m2, int k, RowOwners owners, const 
             v[i] = val[idx];
         }
     }
-    float a[NS][VEC];
+    typename S::Reg a[NS][S::kRegs];
     load_lhs_slice<T, KT, NS, EDGE>(lhs, row, k, lane, a);
     const T* rhs_lane = rhs + ls * VEC;
     wave_lds_sync();
@@ -228,7 +228,7 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     const int w = wave % WPG; // this wave among the waves of its group
     const int ls = lane % LPR;
     const int row0 = g * R;
-    float a[R][1][VEC];
+    typename S::Reg a[R][1][S::kRegs];
     int first[R]; // where the run starts in column_indices / values, per row
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -252,20 +252,10 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const int c = d.lo + min(j0 + group_first + 4 * q + t, d.len - 1);
-                    float b[VEC];
-                    if (!EDGE || ls * VEC < k) {
-                        DenseVec<T>::load(rhs_lane + (size_t)c * k, b);
-                    } else {
+                    uint4 b = make_uint4(0u, 0u, 0u, 0u);
+                    if (!EDGE || ls * VEC < k) b = *reinterpret_cast<const uint4*>(rhs_lane + (size_t)c * k);
 #pragma unroll
-                        for (int x = 0; x < VEC; ++x) b[x] = 0.f;
-                    }
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        float sum = 0.f;
-#pragma unroll
-                        for (int x = 0; x < VEC; ++x) sum = fmaf(a[r][0][x], b[x], sum);
-                        p[r][t] = sum;
-                    }
+                    for (int r = 0; r < R; ++r) p[r][t] = DotVec<T>::dot_raw(a[r][0], b, 0.f);
                 }
                 // transpose-reduce per row: afterwards lane (ls & 3) == t holds column t of the quad
                 const bool hi2 = ls & 2, hi1 = ls & 1;

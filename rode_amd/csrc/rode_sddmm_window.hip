@@ -121,8 +121,11 @@ sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ col, const fl
         const int col_off = tile * TW + ls * VEC;
         const bool col_ok = !EDGE || col_off < k;
         const T* rhs_lane = rhs + (col_ok ? col_off : 0);
-        float a[VEC];
-        DenseVec<T>::unpack(a_raw, a); // zeros past the last column: those lanes add nothing
+        typename DotVec<T>::Reg a[DotVec<T>::kRegs]; // zeros past the last column: those lanes add nothing
+        {
+            const uint32_t w[4] = {a_raw.x, a_raw.y, a_raw.z, a_raw.w};
+            DotVec<T>::load(reinterpret_cast<const T*>(w), a);
+        }
         const bool more = tile + 1 < tiles;
         if constexpr (!PER_TILE) {
             if (tile > 0) __syncthreads(); // every wave is done with the previous tile's window
@@ -158,14 +161,7 @@ sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ col, const fl
                         window_quad<T, EDGE, PER_TILE>(rr, pc, local, 2 * i + h, win_bytes, wave_all_hit, miss_t, first_t,
                                                        col, rhs_lane, k, col_ok, raw);
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            float b[VEC];
-                            DenseVec<T>::unpack(raw[j], b);
-                            float sum = 0.f;
-#pragma unroll
-                            for (int x = 0; x < VEC; ++x) sum = fmaf(a[x], b[x], sum);
-                            part8[4 * h + j] = sum;
-                        }
+                        for (int j = 0; j < 4; ++j) part8[4 * h + j] = DotVec<T>::dot_raw(a, raw[j], 0.f);
                     }
                     acc[i] += transpose_reduce8(part8, ls);
                 }
@@ -178,12 +174,7 @@ sddmm_residue_window_kernel(int m2, int k, const int* __restrict__ col, const fl
                     window_quad<T, EDGE, PER_TILE>(rr, pc, local, q, win_bytes, wave_all_hit, miss_t, first_t, col,
                                                    rhs_lane, k, col_ok, raw);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        float b[VEC];
-                        DenseVec<T>::unpack(raw[j], b);
-#pragma unroll
-                        for (int x = 0; x < VEC; ++x) acc[4 * q + j] = fmaf(a[x], b[x], acc[4 * q + j]);
-                    }
+                    for (int j = 0; j < 4; ++j) acc[4 * q + j] = DotVec<T>::dot_raw(a, raw[j], acc[4 * q + j]);
                 }
             }
         }

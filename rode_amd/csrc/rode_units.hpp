@@ -13,6 +13,8 @@ namespace rode {
 template <typename T, int KT>
 struct SddmmShape {
     static constexpr int kVec = DenseVec<T>::kElems;
+    static constexpr int kRegs = DotVec<T>::kRegs; // registers of a lane's part of the lhs row
+    using Reg = typename DotVec<T>::Reg;
     static constexpr int kLpr = KT / kVec;     // lanes that cover one slab of a dense row
     static constexpr int kQuads = kLpr / 4;    // slot quads per lane group per unit
     static_assert(KT % kVec == 0 && kLpr >= 4 && kLpr <= 32 && (kLpr & (kLpr - 1)) == 0,
@@ -21,28 +23,22 @@ struct SddmmShape {
 
 // <lhs row, rhs row> restricted to this lane's elements.
 template <typename T, int KT, int NS, bool EDGE>
-__device__ __forceinline__ float lane_dot(const float (&a)[NS][SddmmShape<T, KT>::kVec], const T* __restrict__ row_lane,
-                                          int k, int lane_elem)
+__device__ __forceinline__ float lane_dot(const typename DotVec<T>::Reg (&a)[NS][DotVec<T>::kRegs],
+                                          const T* __restrict__ row_lane, int k, int lane_elem)
 {
-    constexpr int VEC = SddmmShape<T, KT>::kVec;
     float d = 0.f;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        if (!EDGE || lane_elem + s * KT < k) {
-            float b[VEC];
-            DenseVec<T>::load(row_lane + s * KT, b);
-#pragma unroll
-            for (int x = 0; x < VEC; ++x) d = fmaf(a[s][x], b[x], d);
-        }
-    }
+    for (int s = 0; s < NS; ++s)
+        if (!EDGE || lane_elem + s * KT < k) d = DotVec<T>::dot(a[s], row_lane + s * KT, d);
     return d;
 }
 
 // Dot products of one 32-slot unit of a block segment.  `my_col` is the column of this
 // lane's slot.  Returns the dot product for this lane's slot.
 template <typename T, int KT, int NS, bool EDGE>
-__device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane, const float (&a)[NS][SddmmShape<T, KT>::kVec],
-                                            int my_col, int k, int* lds_cols, int lane)
+__device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane,
+                                            const typename DotVec<T>::Reg (&a)[NS][DotVec<T>::kRegs], int my_col, int k,
+                                            int* lds_cols, int lane)
 {
     using S = SddmmShape<T, KT>;
     constexpr int LPR = S::kLpr;
@@ -78,15 +74,14 @@ __device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane, cons
 
 template <typename T, int KT, int NS, bool EDGE>
 __device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int row, int k, int lane,
-                                               float (&a)[NS][SddmmShape<T, KT>::kVec])
+                                               typename DotVec<T>::Reg (&a)[NS][DotVec<T>::kRegs])
 {
     using S = SddmmShape<T, KT>;
     const int e0 = (lane % S::kLpr) * S::kVec;
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-#pragma unroll
-        for (int x = 0; x < S::kVec; ++x) a[s][x] = 0.f;
-        if (!EDGE || e0 + s * KT < k) DenseVec<T>::load(lhs + (size_t)row * k + e0 + s * KT, a[s]);
+        DotVec<T>::zero(a[s]);
+        if (!EDGE || e0 + s * KT < k) DotVec<T>::load(lhs + (size_t)row * k + e0 + s * KT, a[s]);
     }
 }
 
