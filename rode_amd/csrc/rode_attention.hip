@@ -154,7 +154,10 @@ __device__ __forceinline__ float softmax_step(float sc, bool live, float& m_run,
 // loaded once for the four rows (the score part is the SDDMM group kernel's, the output
 // part the SpMM group kernel's, with a running softmax per row in between); then the wave
 // takes the nonzeros outside the run, row by row, the way attention_rows_kernel does.
-// Raw scores wait in the probs array itself; the lanes that wrote them normalise them.
+// With WRITE_P the raw scores of the first kGroupScoresKept columns of the run wait in LDS,
+// the others in the probs array itself; the lanes that wrote them normalise them.
+constexpr int kGroupScoresKept = 512;
+
 template <typename T, int D, bool WRITE_P>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
@@ -167,7 +170,9 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     constexpr int QUADS = LPR / 4; // slot quads per lane group per 32-slot unit (SddmmShape::kQuads)
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) float lds_p[kWavesPerWg][R][kWave];
+    __shared__ float lds_s[WRITE_P ? kWavesPerWg * R * kGroupScoresKept : 1];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    float* my_s = lds_s + (WRITE_P ? wave * R * kGroupScoresKept : 0);
     const int g = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (g >= n_groups) return;
     const RowGroup d = groups[g];
@@ -228,7 +233,9 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
         for (int r = 0; r < R; ++r) {
             const float sc = live ? scale * (val[first[r] + j] * dot[r]) : -INFINITY;
             lds_p[wave][r][lane] = softmax_step<VEC>(sc, live, m_run[r], l_lane[r], acc[r]);
-            if (WRITE_P && live) probs[first[r] + j] = sc;
+            if (WRITE_P && live) {
+                if (j < kGroupScoresKept) my_s[r * kGroupScoresKept + j] = sc; else probs[first[r] + j] = sc;
+            }
         }
         wave_lds_sync();
         const int nq = min(kWave / 4, (d.len - j0 + 3) / 4);
@@ -299,7 +306,10 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
         if (WRITE_P) {
             // every lane normalises the scores it wrote itself: same walk over the run and over the rest
             const float m_safe = m_run[r] == -INFINITY ? 0.f : m_run[r];
-            for (int j = lane; j < d.len; j += kWave) probs[first[r] + j] = __expf(probs[first[r] + j] - m_safe) * inv;
+            for (int j = lane; j < d.len; j += kWave) {
+                const float sc = j < kGroupScoresKept ? my_s[r * kGroupScoresKept + j] : probs[first[r] + j];
+                probs[first[r] + j] = __expf(sc - m_safe) * inv;
+            }
             const int s = row_ptr[row0 + r], e = row_ptr[row0 + r + 1];
             const int split = d.pos[r], cnt = split + (e - (s + split + d.len));
             for (int slot = lane; slot < cnt; slot += kWave) {

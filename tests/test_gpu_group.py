@@ -182,18 +182,21 @@ def test_every_nonzero_has_one_owner_and_what_is_refused():
     assert spmm(0, plans())[0] != 0  # a group plan without the whole-lists promise
 
 
-@pytest.mark.parametrize("d,half", [(64, False), (64, True), (128, False), (32, True)])
-def test_fused_attention_of_groups(d, half):
+@pytest.mark.parametrize("d,half,m,window", [(64, False, 12002, 96), (64, True, 12002, 96), (128, False, 12002, 96),
+                                             (32, True, 12002, 96), (32, False, 10000, 600)])
+def test_fused_attention_of_groups(d, half, m, window):
     """rode_hip_attention_forward with a group plan of at least 2048 groups with a run (one
     wave per group: scores of the run for four rows at once, then their softmax, then P.V
     over the run) against fp64 on the host and against the same entry point without a plan;
-    rows in no kept group, rows with holes, empty rows and short rows are all in the matrix."""
+    rows in no kept group, rows with holes, empty rows and short rows are all in the matrix.
+    The last case has runs of more than 512 columns: the raw scores past the first 512 wait
+    in the output array instead of LDS."""
     from gpu_common import DEV, make_csr
     from rode_amd import rode_sddmm_hip
     from rode_amd.autograd import _attention_call
     rng = np.random.default_rng(40 + d)
-    m, n = 12002, 12500
-    rp, col, val = _window_matrix(rng, m, n, 96, 6)
+    n = m + 498
+    rp, col, val = _window_matrix(rng, m, n, window, 6)
     val = rng.uniform(0.5, 1.5, len(col)).astype(np.float32)
     mask = make_csr(rp, col, val, m, n, d, locality=True)
     assert isinstance(mask.plan, rode_sddmm_hip.GroupPlan) and mask.plan.counts[1] >= 2048

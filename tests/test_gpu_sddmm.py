@@ -141,6 +141,19 @@ def test_fp16_operands(k):
         _check(make_csr(rp, col, val, m, n, k, seg), rp, col, val, lhs, rhs, half=True)
 
 
+def test_fp16_subnormal_operands():
+    """fp16 operands below the smallest normal number (2^-14) count with their value: the
+    packed dot-product instruction of the fp16 kernels does not flush them."""
+    from gpu_common import make_csr, run_sddmm
+    rng = np.random.default_rng(3)
+    m, n, k = 64, 64, 64
+    rp = np.arange(0, m * 8 + 1, 8, dtype=np.int32)
+    col = np.concatenate([np.sort(rng.choice(n, 8, replace=False)) for _ in range(m)]).astype(np.int32)
+    csr = make_csr(rp, col, np.ones(len(col), dtype=np.float32), m, n, k)
+    out = run_sddmm(csr, np.full((m, k), 2.0 ** -20, dtype=np.float32), np.full((n, k), 2.0 ** 10, dtype=np.float32), True)
+    assert (out == k * 2.0 ** -10).all()   # every product and every partial sum is exact in fp32
+
+
 def test_special_cases_and_edges():
     from gpu_common import DEV, make_csr, run_sddmm
     from helpers import random_csr
