@@ -219,6 +219,11 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     using S = SddmmShape<T, KT>;
     constexpr int LPR = S::kLpr, VEC = S::kVec, R = kGroupRows;
     static_assert(WPG == 1 || WPG == kWavesPerWg, "a group has one wave, or one workgroup");
+    // (when the lhs rows of the group, as the lanes of a quad hold them, fit 32 registers: with
+    // 64, fp32 rows of 64 elements, the kernel needs 164 registers, a wave less per SIMD, and
+    // config 5 takes 0.075 ms instead of 0.059; reading them from an LDS copy instead does not
+    // help, the compiler then keeps as many registers for loads in flight)
+    constexpr bool kQuadLanes = R * (LPR / 4) * S::kRegs <= 32;
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int g = xcd_logical_block(blockIdx.x, gridDim.x) * (kWavesPerWg / WPG) + wave / WPG;
@@ -228,50 +233,95 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     const int w = wave % WPG; // this wave among the waves of its group
     const int ls = lane % LPR;
     const int row0 = g * R;
-    typename S::Reg a[R][1][S::kRegs];
     int first[R]; // where the run starts in column_indices / values, per row
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
-        first[r] = row_ptr[row0 + r] + d.pos[r];
-    }
-    const T* rhs_lane = rhs + ls * VEC;
+    for (int r = 0; r < R; ++r) first[r] = row_ptr[row0 + r] + d.pos[r];
     // this wave's share of the run, in quads of columns; lane e of a step has column j0 + e
     const int quads = (d.len + 3) / 4;
     const int q_begin = quads * w / WPG, q_end = quads * (w + 1) / WPG;
     const int j_end = min(d.len, 4 * q_end);
-    const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
-    for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
-        if (j0 + (lane & 32) < j_end) { // the upper half sits out a step that has nothing for it
-            float result[R];
+    if constexpr (kQuadLanes) {
+        // Four lanes per rhs row: lane t of the four has the 16-byte vectors t, t + 4, ... of
+        // every row, so a dot product is summed over four lanes only (two exchanges per row of
+        // the group and quad of columns instead of two per level of log2(LPR)).
+        constexpr int E = LPR / 4;
+        const int t4 = lane & 3;
+        typename S::Reg a[R][E][S::kRegs];
 #pragma unroll
-            for (int r = 0; r < R; ++r) result[r] = 0.f;
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int q = 0; q < S::kQuads; ++q) {
+            for (int i = 0; i < E; ++i) {
+                DotVec<T>::zero(a[r][i]);
+                if (!EDGE || (t4 + 4 * i) * VEC < k) DotVec<T>::load(lhs + (size_t)(row0 + r) * k + (t4 + 4 * i) * VEC, a[r][i]);
+            }
+        const T* rhs_lane = rhs + t4 * VEC;
+        for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
+            const int cq = j0 + (lane & ~3); // first column of this lane quad
+            if (cq < j_end) {
                 float p[R][4];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    const int c = d.lo + min(j0 + group_first + 4 * q + t, d.len - 1);
-                    uint4 b = make_uint4(0u, 0u, 0u, 0u);
-                    if (!EDGE || ls * VEC < k) b = *reinterpret_cast<const uint4*>(rhs_lane + (size_t)c * k);
+                    const T* row = rhs_lane + (size_t)(d.lo + min(cq + t, d.len - 1)) * k;
 #pragma unroll
-                    for (int r = 0; r < R; ++r) p[r][t] = DotVec<T>::dot_raw(a[r][0], b, 0.f);
+                    for (int r = 0; r < R; ++r) p[r][t] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < E; ++i) {
+                        uint4 b = make_uint4(0u, 0u, 0u, 0u);
+                        if (!EDGE || (t4 + 4 * i) * VEC < k) b = *reinterpret_cast<const uint4*>(row + 4 * i * VEC);
+#pragma unroll
+                        for (int r = 0; r < R; ++r) p[r][t] = DotVec<T>::dot_raw(a[r][i], b, p[r][t]);
+                    }
                 }
-                // transpose-reduce per row: afterwards lane (ls & 3) == t holds column t of the quad
-                const bool hi2 = ls & 2, hi1 = ls & 1;
+                // transpose-reduce per row: afterwards lane t4 holds column cq + t4 = j0 + lane
+                const bool hi2 = t4 & 2, hi1 = t4 & 1;
+                const int j = j0 + lane;
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const float q0 = (hi2 ? p[r][2] : p[r][0]) + lane_xor2(hi2 ? p[r][0] : p[r][2]);
                     const float q1 = (hi2 ? p[r][3] : p[r][1]) + lane_xor2(hi2 ? p[r][1] : p[r][3]);
-                    float v = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
-                    v = butterfly_sum<4, LPR>(v);
-                    if ((ls >> 2) == q) result[r] = v;
+                    const float v = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
+                    if (j < j_end) out[first[r] + j] = val[first[r] + j] * v;
                 }
             }
-            const int j = j0 + lane;
-            if (j < j_end) {
+        }
+    } else {
+        typename S::Reg a[R][1][S::kRegs];
 #pragma unroll
-                for (int r = 0; r < R; ++r) out[first[r] + j] = val[first[r] + j] * result[r];
+        for (int r = 0; r < R; ++r) load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
+        const T* rhs_lane = rhs + ls * VEC;
+        const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
+        for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
+            if (j0 + (lane & 32) < j_end) { // the upper half sits out a step that has nothing for it
+                float result[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) result[r] = 0.f;
+#pragma unroll
+                for (int q = 0; q < S::kQuads; ++q) {
+                    float p[R][4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int c = d.lo + min(j0 + group_first + 4 * q + t, d.len - 1);
+                        uint4 b = make_uint4(0u, 0u, 0u, 0u);
+                        if (!EDGE || ls * VEC < k) b = *reinterpret_cast<const uint4*>(rhs_lane + (size_t)c * k);
+#pragma unroll
+                        for (int r = 0; r < R; ++r) p[r][t] = DotVec<T>::dot_raw(a[r][0], b, 0.f);
+                    }
+                    // transpose-reduce per row: afterwards lane (ls & 3) == t holds column t of the quad
+                    const bool hi2 = ls & 2, hi1 = ls & 1;
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const float q0 = (hi2 ? p[r][2] : p[r][0]) + lane_xor2(hi2 ? p[r][0] : p[r][2]);
+                        const float q1 = (hi2 ? p[r][3] : p[r][1]) + lane_xor2(hi2 ? p[r][1] : p[r][3]);
+                        float v = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
+                        v = butterfly_sum<4, LPR>(v);
+                        if ((ls >> 2) == q) result[r] = v;
+                    }
+                }
+                const int j = j0 + lane;
+                if (j < j_end) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) out[first[r] + j] = val[first[r] + j] * result[r];
+                }
             }
         }
     }
