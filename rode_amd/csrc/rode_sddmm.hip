@@ -225,7 +225,9 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     // help, the compiler then keeps as many registers for loads in flight)
     constexpr bool kQuadLanes = R * (LPR / 4) * S::kRegs <= 32;
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    // (the wave's number is the same in all its lanes; saying so keeps the group's description,
+    // the position in the run and the base address of its rhs rows in scalar registers)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
     const int g = xcd_logical_block(blockIdx.x, gridDim.x) * (kWavesPerWg / WPG) + wave / WPG;
     if (g >= n_groups) return;
     const RowGroup d = groups[g];
@@ -240,6 +242,10 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     const int quads = (d.len + 3) / 4;
     const int q_begin = quads * w / WPG, q_end = quads * (w + 1) / WPG;
     const int j_end = min(d.len, 4 * q_end);
+    // an rhs row of the run = a scalar address (the run's first row at this step) + this lane's
+    // 32-bit offset (row within the step, the lane's elements)
+    const unsigned row_bytes = (unsigned)k * (unsigned)sizeof(T);
+    const T* rhs_run = rhs + (size_t)d.lo * k;
     if constexpr (kQuadLanes) {
         // Four lanes per rhs row: lane t of the four has the 16-byte vectors t, t + 4, ... of
         // every row, so a dot product is summed over four lanes only (two exchanges per row of
@@ -254,20 +260,21 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
                 DotVec<T>::zero(a[r][i]);
                 if (!EDGE || (t4 + 4 * i) * VEC < k) DotVec<T>::load(lhs + (size_t)(row0 + r) * k + (t4 + 4 * i) * VEC, a[r][i]);
             }
-        const T* rhs_lane = rhs + t4 * VEC;
         for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
             const int cq = j0 + (lane & ~3); // first column of this lane quad
             if (cq < j_end) {
+                const char* step_rows = reinterpret_cast<const char*>(rhs_run + (size_t)j0 * k);
                 float p[R][4];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    const T* row = rhs_lane + (size_t)(d.lo + min(cq + t, d.len - 1)) * k;
+                    const unsigned at = __umul24(min((lane & ~3) + t, d.len - 1 - j0), row_bytes) + t4 * VEC * (unsigned)sizeof(T);
 #pragma unroll
                     for (int r = 0; r < R; ++r) p[r][t] = 0.f;
 #pragma unroll
                     for (int i = 0; i < E; ++i) {
                         uint4 b = make_uint4(0u, 0u, 0u, 0u);
-                        if (!EDGE || (t4 + 4 * i) * VEC < k) b = *reinterpret_cast<const uint4*>(row + 4 * i * VEC);
+                        if (!EDGE || (t4 + 4 * i) * VEC < k)
+                            b = *reinterpret_cast<const uint4*>(step_rows + (at + 4 * i * VEC * (unsigned)sizeof(T)));
 #pragma unroll
                         for (int r = 0; r < R; ++r) p[r][t] = DotVec<T>::dot_raw(a[r][i], b, p[r][t]);
                     }
@@ -288,10 +295,10 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
         typename S::Reg a[R][1][S::kRegs];
 #pragma unroll
         for (int r = 0; r < R; ++r) load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
-        const T* rhs_lane = rhs + ls * VEC;
         const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
         for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
             if (j0 + (lane & 32) < j_end) { // the upper half sits out a step that has nothing for it
+                const char* step_rows = reinterpret_cast<const char*>(rhs_run + (size_t)j0 * k);
                 float result[R];
 #pragma unroll
                 for (int r = 0; r < R; ++r) result[r] = 0.f;
@@ -300,9 +307,9 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
                     float p[R][4];
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
-                        const int c = d.lo + min(j0 + group_first + 4 * q + t, d.len - 1);
+                        const unsigned at = __umul24(min(group_first + 4 * q + t, d.len - 1 - j0), row_bytes) + ls * VEC * (unsigned)sizeof(T);
                         uint4 b = make_uint4(0u, 0u, 0u, 0u);
-                        if (!EDGE || ls * VEC < k) b = *reinterpret_cast<const uint4*>(rhs_lane + (size_t)c * k);
+                        if (!EDGE || ls * VEC < k) b = *reinterpret_cast<const uint4*>(step_rows + at);
 #pragma unroll
                         for (int r = 0; r < R; ++r) p[r][t] = DotVec<T>::dot_raw(a[r][0], b, 0.f);
                     }
@@ -424,6 +431,7 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
     if constexpr (NS == 1) {
         if (e == hipSuccess && grouped) {
             // one wave per group when there are groups enough to fill the GPU that way, else a workgroup
+            // (two waves per group, 8192 waves on config 5: 0.052 ms instead of 0.038)
             if (plan.group_counts[1] >= kGroupWaveEach) {
                 const int wgs = (owners.n_groups + kWavesPerWg - 1) / kWavesPerWg;
                 sddmm_group_kernel<T, KT, EDGE, 1><<<(wgs + kXcds - 1) / kXcds * kXcds, kWgThreads, 0, s1>>>(

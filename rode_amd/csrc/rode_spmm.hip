@@ -302,7 +302,7 @@ spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, RowOwners owner
 // run, the waves' sums meet in LDS, and wave w adds the total of row w to C (the row is in
 // no other work item: no atomics).
 template <typename T, int TN, bool EDGE, int WPG>
-__global__ void __launch_bounds__(kWgThreads)
+__global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
                   const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
                   const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C)
@@ -315,7 +315,9 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg][R][kWave];
     __shared__ __attribute__((aligned(16))) A sums[WPG > 1 ? kWavesPerWg : 1][R][TN];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    // (the wave's number is the same in all its lanes; saying so keeps the group's description,
+    // the position in the run and the addresses of its dense rows in scalar registers)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
     const int g = xcd_logical_block(blockIdx.x, gridDim.x) * GPW + wave / WPG;
     if (g >= n_groups) return;
     const RowGroup d = groups[g];
@@ -339,11 +341,23 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int x = 0; x < VEC; ++x) acc[r][x] = A(0);
-    for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
-        const int j = j0 + lane;
+    // a dense row of the run = a scalar address (start of the run, step, quad) + this lane's
+    // 32-bit offset (its lane group's quad, its elements of the tile, the row in the quad)
+    const T* b_run = B + tile + (size_t)d.lo * n;
+    const unsigned row_bytes = (unsigned)n * (unsigned)sizeof(T);
+    const unsigned lane_off = 4u * group * row_bytes + (col_ok ? ls * VEC * (unsigned)sizeof(T) : 0u); // in bytes
+    A v_next[R]; // the values of the next step are loaded while this one is computed
 #pragma unroll
-        for (int r = 0; r < R; ++r) lds_v[wave][r][lane] = j < j_end ? val[first[r] + j] : A(0);
+    for (int r = 0; r < R; ++r) v_next[r] = 4 * q_begin + lane < j_end ? val[first[r] + 4 * q_begin + lane] : A(0);
+    for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) lds_v[wave][r][lane] = v_next[r];
         wave_lds_sync();
+        {
+            const int j = j0 + kWave + lane;
+#pragma unroll
+            for (int r = 0; r < R; ++r) v_next[r] = j < j_end ? val[first[r] + j] : A(0);
+        }
         const int nq = min(kWave / 4, (j_end - j0 + 3) / 4);
 #pragma unroll
         for (int i = 0; i < kWave / 4 / G; ++i) {
@@ -351,11 +365,15 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
             if (q < nq) {
                 // four consecutive rows of B (the last quad of a run may be cut short: its rows
                 // past the run repeat the run's last row, their values are zero)
-                const T* b_quad = b_lane + (size_t)(d.lo + j0 + 4 * q) * n;
+                const char* b_quad = reinterpret_cast<const char*>(b_run + (size_t)(j0 + 4 * i * G) * n);
                 const int room = d.len - 1 - (j0 + 4 * q);
+                const unsigned o1 = room >= 1 ? row_bytes : 0u;
+                const unsigned o2 = room >= 2 ? 2u * row_bytes : o1;
+                const unsigned o3 = room >= 3 ? 3u * row_bytes : o2;
+                const unsigned off[4] = {lane_off, lane_off + o1, lane_off + o2, lane_off + o3};
                 A b[4][VEC];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) DenseVec<T>::load(b_quad + (size_t)min(t, room) * n, b[t]);
+                for (int t = 0; t < 4; ++t) DenseVec<T>::load(reinterpret_cast<const T*>(b_quad + off[t]), b[t]);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     A v[4];
