@@ -54,7 +54,7 @@ attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restr
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) float lds_p[kWavesPerWg * kWave];
     __shared__ float lds_s[WRITE_P ? kWavesPerWg * kScoresKept : 1];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
     const int row = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (row >= M) return;
     if (owned_elsewhere(owners, row, 0)) return; // a row of a group: attention_group_kernel has it
@@ -171,7 +171,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) float lds_p[kWavesPerWg][R][kWave];
     __shared__ float lds_s[WRITE_P ? kWavesPerWg * R * kGroupScoresKept : 1];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
     float* my_s = lds_s + (WRITE_P ? wave * R * kGroupScoresKept : 0);
     const int g = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (g >= n_groups) return;

@@ -74,7 +74,7 @@ sddmm_block_body(int bid, int nblocks, int m1, int k, RowOwners owners, const in
                  const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
 {
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
     const int seg = xcd_logical_block(bid, nblocks) * kWavesPerWg + wave;
     if (seg >= m1) return;
 
@@ -108,7 +108,7 @@ sddmm_residue_body(int bid, int nblocks, int m2, int k, RowOwners owners, const 
     constexpr int OWN = kBlockItems / LPR;    // slots owned by one lane
     constexpr int LQ = LPR / 4;               // lane quads per group
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * RPW * kBlockItems];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
     const int group = lane / LPR, ls = lane % LPR;
     const int item = (xcd_logical_block(bid, nblocks) * kWavesPerWg + wave) * RPW + group;
     if (item >= m2) return;
@@ -352,7 +352,7 @@ sddmm_hub_kernel(int k, int merge, const int* __restrict__ hub, const int* __res
                  const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
 {
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
     const HubPlan hp = hub_plan_view(hub);
     const long long item = (long long)xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (item >= (long long)hp.n_hub * hub_groups(hp.slabs, merge)) return;

@@ -126,7 +126,7 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, RowOwners 
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
     const int seg0 = xcd_logical_block(bid, nblocks) * kWavesPerWg;
     const int seg = seg0 + wave;
     BlockItem it{-1, 0, 0, 0};
@@ -206,7 +206,7 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, RowOwner
     constexpr int OWN = kBlockItems / LPR;  // slots staged by one lane
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * RPW * kBlockItems];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * RPW * kBlockItems];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
     const int group = lane / LPR, ls = lane % LPR;
     const int item = (xcd_logical_block(bid, nblocks) * kWavesPerWg + wave) * RPW + group;
     if (item >= m2) return;
@@ -439,7 +439,7 @@ spmm_hub_kernel(int n, int merge, const int* __restrict__ hub, const int* __rest
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
     const HubPlan hp = hub_plan_view(hub);
     const long long item = (long long)xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (item >= (long long)hp.n_hub * hub_groups(hp.slabs, merge)) return;
