@@ -222,7 +222,8 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     // (when the lhs rows of the group, as the lanes of a quad hold them, fit 32 registers: with
     // 64, fp32 rows of 64 elements, the kernel needs 164 registers, a wave less per SIMD, and
     // config 5 takes 0.075 ms instead of 0.059; reading them from an LDS copy instead does not
-    // help, the compiler then keeps as many registers for loads in flight)
+    // help, the compiler then keeps as many registers for loads in flight; two passes over the
+    // run with two rows each load every rhs row twice: 0.078 ms)
     constexpr bool kQuadLanes = R * (LPR / 4) * S::kRegs <= 32;
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
     // (the wave's number is the same in all its lanes; saying so keeps the group's description,
