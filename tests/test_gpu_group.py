@@ -181,6 +181,17 @@ def test_every_nonzero_has_one_owner_and_what_is_refused():
     assert (sum(p for _, p in parts) - plain_c).abs().max().item() <= 2e-5 * plain_c.abs().max().item()
     assert spmm(0, plans())[0] != 0  # a group plan without the whole-lists promise
 
+    # the attention entry point refuses a group plan made for another number of rows
+    q = torch.zeros(m + 8, k, device=DEV)
+    o = torch.zeros(m + 8, k, device=DEV)
+    rp8 = torch.cat([csr.row_offsets, csr.row_offsets[-1:].repeat(8)])
+    p = plans()
+    args = (0, None, k, rp8.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(), q.data_ptr(), B.data_ptr(),
+            B.data_ptr(), ctypes.c_float(1.0), o.data_ptr(), None, ctypes.byref(p), None)
+    assert lib.rode_hip_attention_forward(args[0], m + 8, *args[2:]) != 0
+    assert lib.rode_hip_attention_forward(args[0], m, *args[2:]) == 0
+    torch.cuda.synchronize()
+
 
 @pytest.mark.parametrize("d,half,m,window", [(64, False, 12002, 96), (64, True, 12002, 96), (128, False, 12002, 96),
                                              (32, True, 12002, 96), (32, False, 10000, 600)])
