@@ -9,7 +9,7 @@
 // RoDe_SDDMM/RoDeSddmm.cu:96-140).  The plan changes no result.
 //
 //   group_runs_kernel   per row: its longest run of consecutive columns (first column,
-//                       length, position in the row); one thread per row.
+//                       length, position in the row); one wave per row.
 //   group_desc_kernel   per group: the intersection of its rows' runs; the group is kept
 //                       if that run has at least kGroupMinRun columns and holds at least
 //                       three quarters of the group's nonzeros.
@@ -22,33 +22,49 @@ namespace {
 
 constexpr int kGroupMinRun = 64;
 
+// One wave per row, 64 nonzeros per step: lane e flags its nonzero when a run starts there
+// (its column is not its predecessor's plus one); the ballot of the flags is walked bit by
+// bit - the same in every lane, on the scalar unit - closing a run at every flag.  Of runs
+// of equal length the first counts.
 __global__ void __launch_bounds__(kWgThreads)
 group_runs_kernel(int M, const int* __restrict__ row_ptr, const int* __restrict__ col, int* __restrict__ runs)
 {
-    const int row = blockIdx.x * kWgThreads + threadIdx.x;
-    if (row >= M) return;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+    const long long row_ll = (long long)blockIdx.x * kWavesPerWg + wave;
+    if (row_ll >= M) return;
+    const int row = (int)row_ll;
     const int s = row_ptr[row], e = row_ptr[row + 1];
     int best_first = 0, best_len = 0, best_pos = 0;
-    int first = 0, len = 0, pos = 0, prev = -2;
-    for (int i = s; i < e; ++i) {
-        const int c = col[i];
-        if (c == prev + 1) {
-            ++len;
-        } else {
-            first = c;
-            len = 1;
-            pos = i - s;
+    int run_first = 0, run_pos = 0; // the run that is open: its first column, its position in the row
+    for (int base = s; base < e; base += kWave) {
+        const int i = base + lane;
+        const bool live = i < e;
+        const int c = live ? col[i] : 0;
+        const bool starts = live && (i == s || col[i - 1] + 1 != c);
+        unsigned long long flags = __ballot(starts);
+        while (flags) {
+            const int f = __builtin_ctzll(flags);
+            flags &= flags - 1;
+            const int pos = base - s + f;
+            if (pos - run_pos > best_len) {
+                best_first = run_first;
+                best_len = pos - run_pos;
+                best_pos = run_pos;
+            }
+            run_first = __builtin_amdgcn_readlane(c, f);
+            run_pos = pos;
         }
-        if (len > best_len) {
-            best_first = first;
-            best_len = len;
-            best_pos = pos;
-        }
-        prev = c;
     }
-    runs[3 * row] = best_first;
-    runs[3 * row + 1] = best_len;
-    runs[3 * row + 2] = best_pos;
+    if (e - s - run_pos > best_len) {
+        best_first = run_first;
+        best_len = e - s - run_pos;
+        best_pos = run_pos;
+    }
+    if (lane == 0) {
+        runs[3 * row] = best_first;
+        runs[3 * row + 1] = best_len;
+        runs[3 * row + 2] = best_pos;
+    }
 }
 
 __global__ void __launch_bounds__(kWgThreads)
@@ -101,7 +117,7 @@ hipError_t group_plan_launch(int M, const int* row_ptr, const int* col, int* pla
     group_header_kernel<<<1, kWave, 0, stream>>>(M, groups, plan);
     if (groups > 0) {
         int* runs = plan + kGroupHeaderInts + (size_t)groups * (sizeof(RowGroup) / sizeof(int)); // scratch behind the table
-        group_runs_kernel<<<(M + kWgThreads - 1) / kWgThreads, kWgThreads, 0, stream>>>(M, row_ptr, col, runs);
+        group_runs_kernel<<<(M + kWavesPerWg - 1) / kWavesPerWg, kWgThreads, 0, stream>>>(M, row_ptr, col, runs);
         group_desc_kernel<<<(groups + kWgThreads - 1) / kWgThreads, kWgThreads, 0, stream>>>(groups, row_ptr, runs, plan);
     }
     return hipGetLastError();

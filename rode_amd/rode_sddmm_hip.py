@@ -209,7 +209,7 @@ def hub_plan(row_offsets, column_indices, m, n, min_len):
 
 class GroupPlan:
     """Group plan of one pattern (``rode_hip_group_plan``): the device array and a host copy
-    of its header ``[groups, groups with a shared run, 0, 0]``."""
+    of its header ``[groups, groups with a shared run, rows outside those groups, 0]``."""
 
     def __init__(self, data, counts):
         self.data = data
