@@ -312,7 +312,7 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
     constexpr int GPW = kWavesPerWg / WPG; // groups per workgroup
     static_assert(WPG == 1 || WPG == kWavesPerWg, "a group has one wave, or one workgroup");
-    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
+    __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg][WPG == 1 ? R : 1][kWave];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg][R][kWave];
     __shared__ __attribute__((aligned(16))) A sums[WPG > 1 ? kWavesPerWg : 1][R][TN];
     // (the wave's number is the same in all its lanes; saying so keeps the group's description,
@@ -387,36 +387,85 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
         }
         wave_lds_sync();
     }
+    if constexpr (WPG == 1) {
+        // the nonzeros outside the run, of the four rows at once: their columns and values are
+        // loaded together and their gathers follow each other without a wait in between (row
+        // after row, a wave would sit through two memory round trips per row and step)
+        int row_first[R], split[R], cnt[R], max_cnt = 0;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-#pragma unroll
-        for (int x = 0; x < VEC; ++x) acc[r][x] = butterfly_sum<LPR, kWave>(acc[r][x]);
-        if (WPG > 1 && group == 0) {
-#pragma unroll
-            for (int x = 0; x < VEC; ++x) sums[wave][r][ls * VEC + x] = acc[r][x];
+        for (int r = 0; r < R; ++r) {
+            row_first[r] = first[r] - d.pos[r];
+            split[r] = d.pos[r];
+            cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (first[r] + d.len)); // the slots before the run + those after it
+            max_cnt = max(max_cnt, cnt[r]);
         }
-    }
-    if (WPG > 1) __syncthreads();
-    // the rows this wave finishes: their nonzeros before and after the run, then the update of C
+        for (int off = 0; off < max_cnt; off += kWave) {
+            const int slot = off + lane;
 #pragma unroll
-    for (int r = w; r < R; r += WPG) {
-        const int row = row0 + r, s = row_ptr[row], e = row_ptr[row + 1];
-        const int run_first = s + d.pos[r], run_end = run_first + d.len;
-        A outside[VEC]; // the slots before the run and, in the same pass, those after it
-        spmm_sum_slots<T, TN>(s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, lane, lds_c + wave * kWave,
-                              &lds_v[wave][0][0], b_lane, n, col, val, outside);
-        if (group == 0 && col_ok) {
-            A* c_lane = C + (size_t)row * n + tile + ls * VEC;
+            for (int r = 0; r < R; ++r) {
+                const int live = min(cnt[r] - off, kWave); // this row's slots in this step (may be <= 0)
+                int c = 0;
+                A v = A(0);
+                if (lane < ((live + 3) & ~3)) { // (slots past the end of the last quad: value 0, column of a real slot)
+                    const bool past = slot >= cnt[r];
+                    const int at = past ? cnt[r] - 1 : slot;
+                    const int idx = row_first[r] + at + (at >= split[r] ? d.len : 0);
+                    c = col[idx];
+                    v = past ? A(0) : val[idx];
+                }
+                lds_c[wave][r][lane] = c;
+                lds_v[wave][r][lane] = v;
+            }
+            wave_lds_sync();
 #pragma unroll
-            for (int x = 0; x < VEC; ++x) {
-                A total = outside[x];
-                if (WPG > 1) {
+            for (int r = 0; r < R; ++r) {
+                const int live = min(cnt[r] - off, kWave);
+                if (live >= kWave)
+                    spmm_gather<T, TN, 16 / G, true>(b_lane, (size_t)n, acc[r], lds_c[wave][r], lds_v[wave][r], group, G, 16);
+                else if (live > 0)
+                    spmm_gather<T, TN, 16 / G, false>(b_lane, (size_t)n, acc[r], lds_c[wave][r], lds_v[wave][r], group, G,
+                                                      (live + 3) / 4);
+            }
+            wave_lds_sync();
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int x = 0; x < VEC; ++x) acc[r][x] = butterfly_sum<LPR, kWave>(acc[r][x]);
+            if (group == 0 && col_ok) {
+                A* c_lane = C + (size_t)(row0 + r) * n + tile + ls * VEC;
+#pragma unroll
+                for (int x = 0; x < VEC; ++x) c_lane[x] += acc[r][x]; // (long rows are accumulated into C by contract)
+            }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int x = 0; x < VEC; ++x) acc[r][x] = butterfly_sum<LPR, kWave>(acc[r][x]);
+            if (group == 0) {
+#pragma unroll
+                for (int x = 0; x < VEC; ++x) sums[wave][r][ls * VEC + x] = acc[r][x];
+            }
+        }
+        __syncthreads();
+        // the row this wave finishes: its nonzeros before and after the run, then the update of C
+#pragma unroll
+        for (int r = w; r < R; r += WPG) {
+            const int row = row0 + r, s = row_ptr[row], e = row_ptr[row + 1];
+            const int run_first = s + d.pos[r], run_end = run_first + d.len;
+            A outside[VEC]; // the slots before the run and, in the same pass, those after it
+            spmm_sum_slots<T, TN>(s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, lane, lds_c[wave][0],
+                                  &lds_v[wave][0][0], b_lane, n, col, val, outside);
+            if (group == 0 && col_ok) {
+                A* c_lane = C + (size_t)row * n + tile + ls * VEC;
+#pragma unroll
+                for (int x = 0; x < VEC; ++x) {
+                    A total = outside[x];
 #pragma unroll
                     for (int v = 0; v < WPG; ++v) total += sums[v][r][ls * VEC + x];
-                } else {
-                    total += acc[r][x];
+                    c_lane[x] += total; // (long rows are accumulated into C by contract)
                 }
-                c_lane[x] += total; // (long rows are accumulated into C by contract)
             }
         }
     }
