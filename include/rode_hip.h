@@ -386,6 +386,14 @@ int rode_hip_csr_transpose(int M, int N, int nnz, const int* d_row_offsets, cons
                            int* d_t_row_offsets, int* d_t_column_indices, int* d_perm, void* d_workspace,
                            size_t workspace_bytes, void* stream);
 
+/*
+ * d_dst[i] = d_src[d_index[i]] for i < n: the values of the transposed pattern,
+ * values_t = values[perm], with perm from rode_hip_csr_transpose.  d_index and d_dst
+ * 16-byte aligned, d_dst must not be d_src, every index in range of d_src.  No counterpart in
+ * the reference (see rode_hip_csr_transpose).
+ */
+int rode_hip_permute_f32(int n, const float* d_src, const int* d_index, float* d_dst, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,7 @@ SIGNATURES = {
     "rode_hip_csr_softmax_backward_f32": (c_int, [c_int] + [c_void_p] * 4 + [ctypes.c_float, c_void_p]),
     "rode_hip_csr_transpose_workspace_bytes": (c_size_t, [c_int]),
     "rode_hip_csr_transpose": (c_int, [c_int] * 3 + [c_void_p] * 6 + [c_size_t, c_void_p]),
+    "rode_hip_permute_f32": (c_int, [c_int] + [c_void_p] * 4),
     "rode_hip_attention_forward": (c_int, [c_int] * 3 + [c_void_p] * 6 + [ctypes.c_float] + [c_void_p] * 4),
 }
 

@@ -44,8 +44,8 @@ class SddmmFunction(torch.autograd.Function):
         if ctx.needs_input_grad[2]:
             d_lhs = _spmm(csr, gv, rhs.float()).to(lhs.dtype)
         if ctx.needs_input_grad[3]:
-            csr_t, perm = csr.transpose()
-            d_rhs = _spmm(csr_t, gv[perm], lhs.float()).to(rhs.dtype)
+            csr_t, perm = csr.transpose(with_values=False)
+            d_rhs = _spmm(csr_t, rode_sddmm_hip.permute(gv, perm), lhs.float()).to(rhs.dtype)
         if ctx.needs_input_grad[1]:
             d_values = _sddmm(csr, g, lhs, rhs).to(values.dtype)
         return None, d_values, d_lhs, d_rhs
@@ -65,8 +65,8 @@ class SpmmFunction(torch.autograd.Function):
         g = g.contiguous().float()
         d_values = d_dense = None
         if ctx.needs_input_grad[2]:
-            csr_t, perm = csr.transpose()
-            d_dense = _spmm(csr_t, values.float()[perm], g).to(dense.dtype)
+            csr_t, perm = csr.transpose(with_values=False)
+            d_dense = _spmm(csr_t, rode_sddmm_hip.permute(values.float().contiguous(), perm), g).to(dense.dtype)
         if ctx.needs_input_grad[1]:
             if g.shape[1] % 4 != 0 or g.shape[1] > 512:
                 raise NotImplementedError("the gradient with respect to the sparse values is an SDDMM over the dense "
@@ -166,17 +166,17 @@ class FusedAttentionFunction(torch.autograd.Function):
         dq = dk = dv = None
         csr_t = perm = None
         if ctx.needs_input_grad[2] or ctx.needs_input_grad[3]:
-            csr_t, perm = csr.transpose()
+            csr_t, perm = csr.transpose(with_values=False)
         if ctx.needs_input_grad[3]:
-            dv = _spmm(csr_t, probs[perm], g).to(v.dtype)
+            dv = _spmm(csr_t, rode_sddmm_hip.permute(probs, perm), g).to(v.dtype)
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            dp = _sddmm(csr, torch.ones_like(probs), g, v.float())
+            dp = _sddmm(csr, csr.ones(), g, v.float())
             ds = _softmax_call("rode_hip_csr_softmax_backward_f32", csr.row_offsets, probs, dp, scale)
             ds.mul_(csr.values)  # scores are values (.) (q k^T)
             if ctx.needs_input_grad[1]:
                 dq = _spmm(csr, ds, k.float()).to(q.dtype)
             if ctx.needs_input_grad[2]:
-                dk = _spmm(csr_t, ds[perm], q.float()).to(k.dtype)
+                dk = _spmm(csr_t, rode_sddmm_hip.permute(ds, perm), q.float()).to(k.dtype)
         return None, dq, dk, dv, None
 
 

@@ -380,6 +380,13 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
 
 size_t rode_hip_csr_transpose_workspace_bytes(int nnz) { return rode::csr_transpose_workspace_bytes(nnz); }
 
+int rode_hip_permute_f32(int n, const float* d_src, const int* d_index, float* d_dst, void* stream)
+{
+    if (n < 0 || (n > 0 && (!d_src || !d_index || !d_dst || !aligned16(d_index) || !aligned16(d_dst) || d_src == d_dst)))
+        return hipErrorInvalidValue;
+    return rode::permute_launch(n, d_src, d_index, d_dst, as_stream(stream));
+}
+
 int rode_hip_csr_transpose(int M, int N, int nnz, const int* d_row_offsets, const int* d_column_indices,
                            int* d_t_row_offsets, int* d_t_column_indices, int* d_perm, void* d_workspace,
                            size_t workspace_bytes, void* stream)

@@ -84,6 +84,7 @@ template <typename T>
 hipError_t sddmm_window_launch(int m2, int k, const int* col, const float* val, const T* lhs, const T* rhs, float* out,
                                const int* plan, const void* plan_rows, hipStream_t stream);
 
+hipError_t permute_launch(int n, const float* src, const int* index, float* dst, hipStream_t stream);
 size_t csr_transpose_workspace_bytes(int nnz);
 hipError_t csr_transpose_launch(int M, int N, int nnz, const int* row_ptr, const int* col, int* t_row_ptr, int* t_col,
                                 int* perm, void* workspace, hipStream_t stream);

@@ -177,6 +177,33 @@ size_t csr_transpose_workspace_bytes(int nnz)
     return 3 * round16((size_t)max(nnz, 1) * 4) + round16((size_t)kRadix * max(sort_blocks(nnz), 1) * 4);
 }
 
+namespace {
+
+// dst[i] = src[index[i]]: four outputs per thread, the indices and the results as 128-bit
+// accesses, the four reads wherever the indices point.
+__global__ void __launch_bounds__(kWgThreads)
+permute_kernel(int n, const float* __restrict__ src, const int* __restrict__ index, float* __restrict__ dst)
+{
+    const long long i0 = ((long long)blockIdx.x * kWgThreads + threadIdx.x) * 4;
+    if (i0 + 3 < n) {
+        const int4 at = *reinterpret_cast<const int4*>(index + i0);
+        *reinterpret_cast<float4*>(dst + i0) = make_float4(src[at.x], src[at.y], src[at.z], src[at.w]);
+    } else {
+        for (long long i = i0; i < n; ++i) dst[i] = src[index[i]];
+    }
+}
+
+} // namespace
+
+// The values of a transposed pattern: values_t = values[perm] (perm from csr_transpose_launch).
+hipError_t permute_launch(int n, const float* src, const int* index, float* dst, hipStream_t stream)
+{
+    if (n <= 0) return hipSuccess;
+    const long long threads = ((long long)n + 3) / 4;
+    permute_kernel<<<(int)((threads + kWgThreads - 1) / kWgThreads), kWgThreads, 0, stream>>>(n, src, index, dst);
+    return hipGetLastError();
+}
+
 hipError_t csr_transpose_launch(int M, int N, int nnz, const int* row_ptr, const int* col, int* t_row_ptr, int* t_col,
                                 int* perm, void* workspace, hipStream_t stream)
 {

@@ -169,21 +169,38 @@ class RoDeCSR:
         other.values = other.values.to(self.device).contiguous()
         return other
 
-    def transpose(self):
-        """``(csr_t, perm)``: the decomposed pattern of the transposed matrix and the
-        permutation with ``csr_t.values == self.values[perm]`` (built on the GPU once,
-        then cached).  Needed by the gradients with respect to the column-side operands."""
+    def transpose(self, with_values=True):
+        """``(csr_t, perm)``: the decomposed pattern of the transposed matrix and the int32
+        permutation with ``csr_t.values == self.values[perm]`` (built on the GPU once, then
+        cached).  Needed by the gradients with respect to the column-side operands; a caller
+        that brings its own values for ``csr_t`` passes ``with_values=False`` and gets the
+        cached pattern as it is, without the gather of this instance's values."""
         cached = self._shared.get("transpose")
         if cached is None:
             row_offsets_t, rows_t, perm = rode_sddmm_hip.csr_transpose(self.row_offsets, self.column_indices,
                                                                        self.m, self.n)
-            perm = perm.to(torch.int64)
-            csr_t = RoDeCSR(row_offsets_t, rows_t, self.values.float()[perm], self.device, self.n, self.m, self.k,
-                            config=self.config, locality=self.locality)
+            csr_t = RoDeCSR(row_offsets_t, rows_t, self._permuted_values(perm).float(), self.device, self.n, self.m,
+                            self.k, config=self.config, locality=self.locality)
             cached = (csr_t, perm)
             self._shared["transpose"] = cached
         csr_t, perm = cached
-        return csr_t.with_values(self.values[perm]), perm
+        if not with_values:
+            return csr_t, perm
+        return csr_t.with_values(self._permuted_values(perm)), perm
+
+    def ones(self):
+        """A float32 vector of ones over the nonzeros (made once per pattern): the values of an
+        SDDMM that samples without weighting."""
+        cached = self._shared.get("ones")
+        if cached is None:
+            cached = torch.ones(self.nnz, dtype=torch.float32, device=self.device)
+            self._shared["ones"] = cached
+        return cached
+
+    def _permuted_values(self, perm):
+        if self.values.dtype == torch.float32:
+            return rode_sddmm_hip.permute(self.values.contiguous(), perm)
+        return self.values[perm]
 
     @classmethod
     def from_random(cls, m, n, nnz_per_row, device, k=128):

@@ -153,6 +153,20 @@ def csr_transpose(row_offsets, column_indices, m, n):
     return row_offsets_t, column_indices_t, perm
 
 
+def permute(values, perm):
+    """``values[perm]`` for a float32 vector and the int32 ``perm`` of ``csr_transpose``: the
+    values of the transposed pattern (``rode_hip_permute_f32``)."""
+    _check_input(values, "values")
+    _check_input(perm, "perm")
+    _check(values.dtype == torch.float32 and perm.dtype == torch.int32, "values must be float32 and perm int32")
+    _check(values.dim() == 1 and perm.dim() == 1 and values.device == perm.device, "values and perm must be vectors on one device")
+    out = torch.empty(perm.numel(), dtype=torch.float32, device=values.device)
+    with torch.cuda.device(values.device):
+        _lib.check(_lib.load().rode_hip_permute_f32(perm.numel(), values.data_ptr(), perm.data_ptr(), out.data_ptr(),
+                                                     _stream_handle(values.device)), "rode_hip_permute_f32")
+    return out
+
+
 class HubPlan:
     """Hub plan of one pattern (``rode_hip_hub_plan``): the device array and a host copy
     of its header ``[hub rows, slabs, min_len, usable, room, 0, 0, 0]``."""

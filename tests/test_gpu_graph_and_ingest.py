@@ -135,3 +135,24 @@ def test_csr_transpose_edges_and_full_size():
     want = _transpose_reference(rp, col, m, n)
     for g, w, name in zip(got, want, ("row_offsets_t", "column_indices_t", "perm")):
         assert np.array_equal(g.cpu().numpy().astype(np.int64), w), name
+
+
+@pytest.mark.gpu
+def test_permute_values():
+    """rode_hip_permute_f32: values[perm] for lengths that are and are not multiples of four,
+    and what it refuses."""
+    from rode_amd import _lib, rode_sddmm_hip
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(3)
+    for n in (0, 1, 5, 64, 1003, 200001):
+        src = torch.randn(max(n, 1), generator=g).to(dev)
+        perm = torch.randperm(max(n, 1), generator=g)[:n].to(torch.int32).to(dev)
+        out = rode_sddmm_hip.permute(src, perm)
+        assert out.shape == (n,) and torch.equal(out, src[perm.long()])
+    lib = _lib.load()
+    src = torch.randn(16, device=dev)
+    idx = torch.arange(16, dtype=torch.int32, device=dev)
+    assert lib.rode_hip_permute_f32(16, src.data_ptr(), idx.data_ptr(), src.data_ptr(), None) != 0   # in place
+    assert lib.rode_hip_permute_f32(-1, src.data_ptr(), idx.data_ptr(), src.data_ptr(), None) != 0
+    with pytest.raises(RuntimeError):
+        rode_sddmm_hip.permute(src, idx.long())
