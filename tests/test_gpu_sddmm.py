@@ -230,6 +230,30 @@ def test_torch_oracle_and_compare_results():
         assert "RoDeCSR(m=511" in repr(csr)
 
 
+# the configuration list of the reference's Python driver (test_pytorch.py:66-91): small,
+# irregular, medium, rectangular, sparsity sweep, prime dimensions, large irregular
+PYTHON_DRIVER_CONFIGS = [(64, 64, 8), (128, 128, 16), (256, 256, 32), (63, 67, 10), (127, 131, 20), (511, 517, 33),
+                         (512, 512, 32), (1024, 1024, 64), (2048, 2048, 128), (2048, 256, 32), (256, 2048, 32),
+                         (1999, 257, 45), (1024, 1024, 4), (1024, 1024, 64), (1024, 1024, 256), (127, 131, 23),
+                         (509, 521, 67), (4093, 4099, 128)]
+
+
+@pytest.mark.parametrize("k", [128, 32])
+def test_python_driver_configurations(k):
+    """Every configuration of the reference's Python driver through its own flow
+    (test_pytorch.py:163-222): from_random, rode_sddmm, torch.sparse.sampled_addmm,
+    compare_results; K=128 is the driver's default, K=32 the other supported width."""
+    from gpu_common import DEV
+    from rode_amd import RoDeCSR, compare_results, rode_sddmm, torch_sddmm_reference
+    for i, (m, n, per_row) in enumerate(PYTHON_DRIVER_CONFIGS):
+        torch.manual_seed(1000 + i)
+        csr = RoDeCSR.from_random(m, n, per_row, DEV, k)
+        torch.manual_seed(123); lhs = torch.randn(m, k, device=DEV)
+        torch.manual_seed(456); rhs = torch.randn(n, k, device=DEV)
+        stats = compare_results(rode_sddmm(csr, lhs, rhs), torch_sddmm_reference(csr.to_torch_sparse_csr(), lhs, rhs), csr)
+        assert stats["passed"] and stats["total_count"] == csr.nnz, (m, n, per_row, stats)
+
+
 @pytest.mark.parametrize("name,k", [("c1_uniform", 32), ("c2_lognormal", 32), ("c2_lognormal", 128)])
 def test_benchmark_configs_against_oracle(name, k):
     from gpu_common import make_csr
