@@ -240,8 +240,13 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, RowOwner
             }
         }
         wave_lds_sync();
-        spmm_gather<T, TN, kBlockItems / 4, false>(B + tile + (col_ok ? ls * VEC : 0), (size_t)n, acc, my_c, my_v, 0, 1,
-                                                   padded / 4);
+        // (two quads in flight where their dense rows fit 32 registers: config 4 K=64 0.550 -> 0.535 ms, K=32
+        // 0.305 -> 0.292; with fp16's eight elements per load it costs waves per SIMD instead: 0.66 -> 0.76 ms)
+        if constexpr (VEC <= 4)
+            spmm_gather_pairs<T, TN, kBlockItems / 4>(B + tile + (col_ok ? ls * VEC : 0), (size_t)n, acc, my_c, my_v, padded / 4);
+        else
+            spmm_gather<T, TN, kBlockItems / 4, false>(B + tile + (col_ok ? ls * VEC : 0), (size_t)n, acc, my_c, my_v, 0, 1,
+                                                       padded / 4);
     }
 
     A* c_lane = C + (size_t)row * n + tile + ls * VEC;

@@ -136,4 +136,46 @@ __device__ __forceinline__ void spmm_gather(const T* __restrict__ b_lane, size_t
     }
 }
 
+// The same sum over the quads 0 .. nquads - 1, two quads per step: the loads of both are
+// issued before either is used (eight dense rows in flight per lane instead of four), and a
+// quad that does not exist loads nothing and adds zeros.  For work items of a few quads
+// whose kernels are bound by memory latency (residue rows).
+template <typename T, int TN, int QUADS_MAX>
+__device__ __forceinline__ void spmm_gather_pairs(const T* __restrict__ b_lane, size_t ldb,
+                                                  typename DenseVec<T>::Acc (&acc)[SpmmShape<T, TN>::kVec],
+                                                  const int* lds_col, const typename DenseVec<T>::Acc* lds_val, int nquads)
+{
+    using A = typename DenseVec<T>::Acc;
+    constexpr int VEC = SpmmShape<T, TN>::kVec;
+    static_assert(QUADS_MAX % 2 == 0, "two quads per step");
+#pragma unroll
+    for (int q = 0; q < QUADS_MAX; q += 2) {
+        if (q < nquads) {
+            A v[2][4], b[2][4][VEC];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    v[h][j] = A(0);
+#pragma unroll
+                    for (int x = 0; x < VEC; ++x) b[h][j][x] = A(0);
+                }
+                if (q + h < nquads) {
+                    const int4 c4 = *reinterpret_cast<const int4*>(lds_col + 4 * (q + h));
+                    const int c[4] = {c4.x, c4.y, c4.z, c4.w};
+                    load_quad(lds_val + 4 * (q + h), v[h]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) DenseVec<T>::load(b_lane + (size_t)c[j] * ldb, b[h][j]);
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int x = 0; x < VEC; ++x) acc[x] = fma(v[h][j], b[h][j][x], acc[x]);
+        }
+    }
+}
+
 } // namespace rode
