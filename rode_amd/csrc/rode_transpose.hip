@@ -184,7 +184,9 @@ namespace {
 __global__ void __launch_bounds__(kWgThreads)
 permute_kernel(int n, const float* __restrict__ src, const int* __restrict__ index, float* __restrict__ dst)
 {
-    const long long i0 = ((long long)blockIdx.x * kWgThreads + threadIdx.x) * 4;
+    // (neighbouring outputs read neighbouring places of src when the pattern has any locality:
+    // a contiguous range of workgroups per XCD keeps those re-reads in one L2)
+    const long long i0 = ((long long)xcd_logical_block(blockIdx.x, gridDim.x) * kWgThreads + threadIdx.x) * 4;
     if (i0 + 3 < n) {
         const int4 at = *reinterpret_cast<const int4*>(index + i0);
         *reinterpret_cast<float4*>(dst + i0) = make_float4(src[at.x], src[at.y], src[at.z], src[at.w]);
@@ -200,7 +202,8 @@ hipError_t permute_launch(int n, const float* src, const int* index, float* dst,
 {
     if (n <= 0) return hipSuccess;
     const long long threads = ((long long)n + 3) / 4;
-    permute_kernel<<<(int)((threads + kWgThreads - 1) / kWgThreads), kWgThreads, 0, stream>>>(n, src, index, dst);
+    const long long wgs = ((threads + kWgThreads - 1) / kWgThreads + kXcds - 1) / kXcds * kXcds;
+    permute_kernel<<<(int)wgs, kWgThreads, 0, stream>>>(n, src, index, dst);
     return hipGetLastError();
 }
 
