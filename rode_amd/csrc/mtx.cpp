@@ -48,6 +48,7 @@ const char* skip_blank(const char* p, const char* end)
 
 const char* line_end(const char* p, const char* end)
 {
+    if (p >= end) return end; // (an empty text has no address to search from)
     const void* nl = std::memchr(p, '\n', end - p);
     return nl ? static_cast<const char*>(nl) : end;
 }
@@ -71,16 +72,23 @@ bool parse_value(const char*& p, const char* end, double& out)
 {
     p = skip_blank(p, end);
     if (p >= end || *p == '\n') return false;
-    char buf[64];
     size_t len = 0;
-    while (p + len < end && len + 1 < sizeof(buf) && !std::isspace(static_cast<unsigned char>(p[len]))) {
-        buf[len] = p[len];
-        ++len;
+    while (p + len < end && !std::isspace(static_cast<unsigned char>(p[len]))) ++len;
+    // strtod wants a terminated string and the text has none: the token is copied (to the
+    // stack, unless it is longer than any sensible number)
+    char buf[64];
+    std::string big;
+    const char* token = buf;
+    if (len < sizeof(buf)) {
+        std::memcpy(buf, p, len);
+        buf[len] = 0;
+    } else {
+        big.assign(p, len);
+        token = big.c_str();
     }
-    buf[len] = 0;
     char* stop = nullptr;
-    out = std::strtod(buf, &stop);
-    if (stop == buf) return false;
+    out = std::strtod(token, &stop);
+    if (stop != token + len) return false; // (not a number, or a number followed by something else)
     p += len;
     return true;
 }

@@ -87,6 +87,21 @@ def test_rejects_bad_files(tmp_path):
     bad.write_text("hello\n")
     with pytest.raises(ValueError, match="not a Matrix Market"):
         rio.read_matrix_market(bad)
+    bad.write_text("")
+    with pytest.raises(ValueError):
+        rio.read_matrix_market(bad)
+    bad.write_text("%%MatrixMarket matrix coordinate real general\n2 2 1\n1 1 1.5abc\n")
+    with pytest.raises(ValueError):
+        rio.read_matrix_market(bad)
+
+
+def test_a_number_of_any_length(tmp_path):
+    """A value written with more digits than any buffer guess (80 here) is read whole."""
+    f = tmp_path / "long.mtx"
+    f.write_text("%%MatrixMarket matrix coordinate real general\n2 2 2\n1 1 0." + "3" * 80 + "\n2 2 " + "1" + "0" * 79 + "e-70\n")
+    m, n, rp, col, val = rio.read_matrix_market(f)
+    assert (m, n) == (2, 2) and rp.tolist() == [0, 1, 2] and col.tolist() == [0, 1]
+    np.testing.assert_allclose(val, np.array([1 / 3, 1e9], dtype=np.float32), rtol=1e-6)
 
 
 def test_pad_rows_matches_the_reference_generators():
