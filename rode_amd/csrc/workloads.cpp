@@ -188,6 +188,7 @@ void rode_wl_fill(int config, int M, int ncols, double p0, double p1, uint64_t s
 #pragma omp for schedule(dynamic, 256)
         for (int r = 0; r < M; ++r) {
             gen_row(config, M, ncols, p0, p1, seed, r, sc, cols, &vals);
+            if (cols.empty()) continue; // (an empty row has nothing to copy, and its vectors may have no storage)
             std::memcpy(cols_out + row_ptr[r], cols.data(), cols.size() * sizeof(int));
             std::memcpy(vals_out + row_ptr[r], vals.data(), vals.size() * sizeof(float));
         }
