@@ -219,13 +219,13 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     using S = SddmmShape<T, KT>;
     constexpr int LPR = S::kLpr, VEC = S::kVec, R = kGroupRows;
     static_assert(WPG == 1 || WPG == kWavesPerWg, "a group has one wave, or one workgroup");
+    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * (WPG == 1 ? R : 1) * kWave];
     // (when the lhs rows of the group, as the lanes of a quad hold them, fit 32 registers: with
     // 64, fp32 rows of 64 elements, the kernel needs 164 registers, a wave less per SIMD, and
     // config 5 takes 0.075 ms instead of 0.059; reading them from an LDS copy instead does not
     // help, the compiler then keeps as many registers for loads in flight; two passes over the
     // run with two rows each load every rhs row twice: 0.078 ms)
     constexpr bool kQuadLanes = R * (LPR / 4) * S::kRegs <= 32;
-    __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
     // (the wave's number is the same in all its lanes; saying so keeps the group's description,
     // the position in the run and the base address of its rhs rows in scalar registers)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
@@ -333,14 +333,63 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
             }
         }
     }
-    // the rows this wave finishes: their nonzeros before and after the run
+    if constexpr (WPG == 1) {
+        // the nonzeros outside the run, of the four rows at once: 64 slots per row and step,
+        // their columns and values loaded together, their dot products one row after the other
+        // without a wait in between (row after row, a wave sits through the memory round trips
+        // of every row)
+        typename S::Reg a[R][1][S::kRegs];
+        int row_first[R], split[R], cnt[R], max_cnt = 0;
 #pragma unroll
-    for (int r = w; r < R; r += WPG) {
-        const int row = row0 + r, s = row_ptr[row], e = row_ptr[row + 1];
-        const int run_first = s + d.pos[r], run_end = run_first + d.len;
-        // (the slots before the run and, in the same pass, those after it)
-        sddmm_row_slots<T, KT, 1, EDGE>(row, s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, k, lane,
-                                        lds + wave * kWave, col, val, lhs, rhs, out);
+        for (int r = 0; r < R; ++r) {
+            load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
+            row_first[r] = first[r] - d.pos[r];
+            split[r] = d.pos[r];
+            cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (first[r] + d.len)); // the slots before the run + those after it
+            max_cnt = max(max_cnt, cnt[r]);
+        }
+        const T* rhs_lane = rhs + ls * VEC;
+        for (int off = 0; off < max_cnt; off += kWave) {
+            const int slot = off + lane;
+            int idx[R];
+            float v[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                idx[r] = -1;
+                v[r] = 0.f;
+                int c = 0;
+                if (off + (lane & 32) < cnt[r]) { // (a row without slots in this half of the step reads nothing)
+                    const bool live = slot < cnt[r];
+                    const int at = live ? slot : cnt[r] - 1; // (lanes past the end repeat the last slot and store nothing)
+                    const int i = row_first[r] + at + (at >= split[r] ? d.len : 0);
+                    c = col[i];
+                    if (live) {
+                        idx[r] = i;
+                        v[r] = val[i];
+                    }
+                }
+                lds[(wave * R + r) * kWave + lane] = c;
+            }
+            wave_lds_sync();
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (off + (lane & 32) < cnt[r]) {
+                    const float dot = sddmm_unit_staged<T, KT, 1, EDGE>(rhs_lane, a[r], k, lds + (wave * R + r) * kWave, lane);
+                    if (idx[r] >= 0) out[idx[r]] = v[r] * dot;
+                }
+            }
+            wave_lds_sync();
+        }
+    } else {
+        // the rows this wave finishes: their nonzeros before and after the run
+#pragma unroll
+        for (int r = w; r < R; r += WPG) {
+            const int row = row0 + r, s = row_ptr[row], e = row_ptr[row + 1];
+            const int run_first = s + d.pos[r], run_end = run_first + d.len;
+            // (the slots before the run and, in the same pass, those after it)
+            sddmm_row_slots<T, KT, 1, EDGE>(row, s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, k, lane,
+                                            lds + wave * kWave, col, val, lhs, rhs, out);
+        }
     }
 }
 

@@ -33,19 +33,15 @@ __device__ __forceinline__ float lane_dot(const typename DotVec<T>::Reg (&a)[NS]
     return d;
 }
 
-// Dot products of one 32-slot unit of a block segment.  `my_col` is the column of this
-// lane's slot.  Returns the dot product for this lane's slot.
+// Dot products of the 32-slot units of one step, the slots' columns already in lds_cols
+// (lds_cols[e] = column of lane e's slot).  Returns the dot product for this lane's slot.
 template <typename T, int KT, int NS, bool EDGE>
-__device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane,
-                                            const typename DotVec<T>::Reg (&a)[NS][DotVec<T>::kRegs], int my_col, int k,
-                                            int* lds_cols, int lane)
+__device__ __forceinline__ float sddmm_unit_staged(const T* __restrict__ rhs_lane,
+                                                   const typename DotVec<T>::Reg (&a)[NS][DotVec<T>::kRegs], int k,
+                                                   const int* lds_cols, int lane)
 {
     using S = SddmmShape<T, KT>;
     constexpr int LPR = S::kLpr;
-
-    lds_cols[lane] = my_col;
-    wave_lds_sync();
-
     const int ls = lane % LPR;                    // lane inside its group
     const int group_first = (lane & 31) - ls;     // first slot (within the half) of this group
     const int* group_cols = lds_cols + (lane & 32) + group_first;
@@ -70,6 +66,18 @@ __device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane,
         if ((ls >> 2) == q) result = r;
     }
     return result;
+}
+
+// Dot products of one 32-slot unit of a block segment.  `my_col` is the column of this
+// lane's slot.  Returns the dot product for this lane's slot.
+template <typename T, int KT, int NS, bool EDGE>
+__device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane,
+                                            const typename DotVec<T>::Reg (&a)[NS][DotVec<T>::kRegs], int my_col, int k,
+                                            int* lds_cols, int lane)
+{
+    lds_cols[lane] = my_col;
+    wave_lds_sync();
+    return sddmm_unit_staged<T, KT, NS, EDGE>(rhs_lane, a, k, lds_cols, lane);
 }
 
 template <typename T, int KT, int NS, bool EDGE>
