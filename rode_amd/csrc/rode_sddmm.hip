@@ -204,12 +204,72 @@ sddmm_pair_kernel(int g1, int m1, int m2, int k, RowOwners owners, const int* __
                                             rhs, out, plan);
 }
 
+// The nonzeros of a kept group outside its run, of the four rows at once: 64 slots per row
+// and step, their columns and values loaded together, their dot products one row after the
+// other without a wait in between (row after row, a wave sits through the memory round trips
+// of every row).  lds_cols: kGroupRows * 64 ints of this wave.
+template <typename T, int KT, bool EDGE>
+__device__ __forceinline__ void sddmm_group_leftovers(const RowGroup& d, int row0, const int (&first)[kGroupRows], int k, int lane,
+                                                      int* lds_cols, const int* __restrict__ row_ptr,
+                                                      const int* __restrict__ col, const float* __restrict__ val,
+                                                      const T* __restrict__ lhs, const T* __restrict__ rhs,
+                                                      float* __restrict__ out)
+{
+    using S = SddmmShape<T, KT>;
+    constexpr int R = kGroupRows;
+    typename S::Reg a[R][1][S::kRegs];
+    int row_first[R], split[R], cnt[R], max_cnt = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
+        row_first[r] = first[r] - d.pos[r];
+        split[r] = d.pos[r];
+        cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (first[r] + d.len)); // the slots before the run + those after it
+        max_cnt = max(max_cnt, cnt[r]);
+    }
+    const T* rhs_lane = rhs + (lane % S::kLpr) * S::kVec;
+    for (int off = 0; off < max_cnt; off += kWave) {
+        const int slot = off + lane;
+        int idx[R];
+        float v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            idx[r] = -1;
+            v[r] = 0.f;
+            int c = 0;
+            if (off + (lane & 32) < cnt[r]) { // (a row without slots in this half of the step reads nothing)
+                const bool live = slot < cnt[r];
+                const int at = live ? slot : cnt[r] - 1; // (lanes past the end repeat the last slot and store nothing)
+                const int i = row_first[r] + at + (at >= split[r] ? d.len : 0);
+                c = col[i];
+                if (live) {
+                    idx[r] = i;
+                    v[r] = val[i];
+                }
+            }
+            lds_cols[r * kWave + lane] = c;
+        }
+        wave_lds_sync();
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (off + (lane & 32) < cnt[r]) {
+                const float dot = sddmm_unit_staged<T, KT, 1, EDGE>(rhs_lane, a[r], k, lds_cols + r * kWave, lane);
+                if (idx[r] >= 0) out[idx[r]] = v[r] * dot;
+            }
+        }
+        wave_lds_sync();
+    }
+}
+
 // The groups of a group plan (rode_group.hip): one workgroup per group of four adjacent
 // rows that share a run of consecutive columns.  The waves split the run; every rhs row of
 // it is loaded once (its address follows from the run, no column index is read) and
 // multiplied with the lhs rows of all four rows of the group, which stay in registers.
 // Wave w then computes row w's nonzeros outside the run as usual.  Single-slab rows only
 // (k <= 128 elements per lane tile): four lhs slices of more slabs would not fit.
+// (A variant in which the four waves of a workgroup took four consecutive groups and read
+// the union of their runs through LDS tiles, loaded once per workgroup, ran in the same
+// time on config 5 - 0.049 ms fp32, 0.035 against 0.033 ms fp16 - and was taken out.)
 template <typename T, int KT, bool EDGE, int WPG>
 __global__ void __launch_bounds__(kWgThreads)
 sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
@@ -220,12 +280,6 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     constexpr int LPR = S::kLpr, VEC = S::kVec, R = kGroupRows;
     static_assert(WPG == 1 || WPG == kWavesPerWg, "a group has one wave, or one workgroup");
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * (WPG == 1 ? R : 1) * kWave];
-    // (when the lhs rows of the group, as the lanes of a quad hold them, fit 32 registers: with
-    // 64, fp32 rows of 64 elements, the kernel needs 164 registers, a wave less per SIMD, and
-    // config 5 takes 0.075 ms instead of 0.059; reading them from an LDS copy instead does not
-    // help, the compiler then keeps as many registers for loads in flight; two passes over the
-    // run with two rows each load every rhs row twice: 0.078 ms)
-    constexpr bool kQuadLanes = R * (LPR / 4) * S::kRegs <= 32;
     // (the wave's number is the same in all its lanes; saying so keeps the group's description,
     // the position in the run and the base address of its rhs rows in scalar registers)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
@@ -234,7 +288,6 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     const RowGroup d = groups[g];
     if (d.len <= 0) return; // not a group: its rows are in the lists
     const int w = wave % WPG; // this wave among the waves of its group
-    const int ls = lane % LPR;
     const int row0 = g * R;
     int first[R]; // where the run starts in column_indices / values, per row
 #pragma unroll
@@ -247,139 +300,67 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     // 32-bit offset (row within the step, the lane's elements)
     const unsigned row_bytes = (unsigned)k * (unsigned)sizeof(T);
     const T* rhs_run = rhs + (size_t)d.lo * k;
-    if constexpr (kQuadLanes) {
-        // Four lanes per rhs row: lane t of the four has the 16-byte vectors t, t + 4, ... of
-        // every row, so a dot product is summed over four lanes only (two exchanges per row of
-        // the group and quad of columns instead of two per level of log2(LPR)).
-        constexpr int E = LPR / 4;
-        const int t4 = lane & 3;
-        typename S::Reg a[R][E][S::kRegs];
+    // LP lanes per rhs row, each with E of its 16-byte vectors (LP lanes apart): half as many lanes
+    // as a row has vectors, so that a dot product crosses half as many lanes as in the list
+    // kernels, and the lhs rows of the group still fit 32 registers.  (With four lanes per row
+    // at fp32 rows of 64 - 64 registers of lhs rows, 164 in all, a wave less per SIMD - config 5
+    // took 0.075 ms instead of 0.059; from an LDS copy of the lhs rows the compiler spends the
+    // registers on loads in flight instead; two passes of two rows each: 0.078 ms.)
+    constexpr int LP = LPR >= 8 ? LPR / 2 : LPR, E = LPR / LP;
+    const int lp = lane % LP; // this lane among the lanes of its rhs row
+    typename S::Reg a[R][E][S::kRegs];
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int i = 0; i < E; ++i) {
-                DotVec<T>::zero(a[r][i]);
-                if (!EDGE || (t4 + 4 * i) * VEC < k) DotVec<T>::load(lhs + (size_t)(row0 + r) * k + (t4 + 4 * i) * VEC, a[r][i]);
-            }
-        for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
-            const int cq = j0 + (lane & ~3); // first column of this lane quad
-            if (cq < j_end) {
-                const char* step_rows = reinterpret_cast<const char*>(rhs_run + (size_t)j0 * k);
+        for (int i = 0; i < E; ++i) {
+            DotVec<T>::zero(a[r][i]);
+            if (!EDGE || (lp + LP * i) * VEC < k) DotVec<T>::load(lhs + (size_t)(row0 + r) * k + (lp + LP * i) * VEC, a[r][i]);
+        }
+    const int group_first = lane - lp; // first column (within the step) of this lane group
+    for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
+        if (j0 + (lane & 32) < j_end) { // the upper half sits out a step that has nothing for it
+            const char* step_rows = reinterpret_cast<const char*>(rhs_run + (size_t)j0 * k);
+            float result[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) result[r] = 0.f;
+#pragma unroll
+            for (int q = 0; q < LP / 4; ++q) {
                 float p[R][4];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    const unsigned at = __umul24(min((lane & ~3) + t, d.len - 1 - j0), row_bytes) + t4 * VEC * (unsigned)sizeof(T);
+                    const unsigned at = __umul24(min(group_first + 4 * q + t, d.len - 1 - j0), row_bytes) + lp * VEC * (unsigned)sizeof(T);
 #pragma unroll
                     for (int r = 0; r < R; ++r) p[r][t] = 0.f;
 #pragma unroll
                     for (int i = 0; i < E; ++i) {
                         uint4 b = make_uint4(0u, 0u, 0u, 0u);
-                        if (!EDGE || (t4 + 4 * i) * VEC < k)
-                            b = *reinterpret_cast<const uint4*>(step_rows + (at + 4 * i * VEC * (unsigned)sizeof(T)));
+                        if (!EDGE || (lp + LP * i) * VEC < k)
+                            b = *reinterpret_cast<const uint4*>(step_rows + (at + LP * i * VEC * (unsigned)sizeof(T)));
 #pragma unroll
                         for (int r = 0; r < R; ++r) p[r][t] = DotVec<T>::dot_raw(a[r][i], b, p[r][t]);
                     }
                 }
-                // transpose-reduce per row: afterwards lane t4 holds column cq + t4 = j0 + lane
-                const bool hi2 = t4 & 2, hi1 = t4 & 1;
-                const int j = j0 + lane;
+                // transpose-reduce per row: afterwards lane (lp & 3) == t holds column t of the quad
+                const bool hi2 = lp & 2, hi1 = lp & 1;
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const float q0 = (hi2 ? p[r][2] : p[r][0]) + lane_xor2(hi2 ? p[r][0] : p[r][2]);
                     const float q1 = (hi2 ? p[r][3] : p[r][1]) + lane_xor2(hi2 ? p[r][1] : p[r][3]);
-                    const float v = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
-                    if (j < j_end) out[first[r] + j] = val[first[r] + j] * v;
+                    float v = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
+                    v = butterfly_sum<4, LP>(v);
+                    if ((lp >> 2) == q) result[r] = v;
                 }
             }
-        }
-    } else {
-        typename S::Reg a[R][1][S::kRegs];
+            const int j = j0 + lane;
+            if (j < j_end) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
-        const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
-        for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
-            if (j0 + (lane & 32) < j_end) { // the upper half sits out a step that has nothing for it
-                const char* step_rows = reinterpret_cast<const char*>(rhs_run + (size_t)j0 * k);
-                float result[R];
-#pragma unroll
-                for (int r = 0; r < R; ++r) result[r] = 0.f;
-#pragma unroll
-                for (int q = 0; q < S::kQuads; ++q) {
-                    float p[R][4];
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const unsigned at = __umul24(min(group_first + 4 * q + t, d.len - 1 - j0), row_bytes) + ls * VEC * (unsigned)sizeof(T);
-                        uint4 b = make_uint4(0u, 0u, 0u, 0u);
-                        if (!EDGE || ls * VEC < k) b = *reinterpret_cast<const uint4*>(step_rows + at);
-#pragma unroll
-                        for (int r = 0; r < R; ++r) p[r][t] = DotVec<T>::dot_raw(a[r][0], b, 0.f);
-                    }
-                    // transpose-reduce per row: afterwards lane (ls & 3) == t holds column t of the quad
-                    const bool hi2 = ls & 2, hi1 = ls & 1;
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        const float q0 = (hi2 ? p[r][2] : p[r][0]) + lane_xor2(hi2 ? p[r][0] : p[r][2]);
-                        const float q1 = (hi2 ? p[r][3] : p[r][1]) + lane_xor2(hi2 ? p[r][1] : p[r][3]);
-                        float v = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
-                        v = butterfly_sum<4, LPR>(v);
-                        if ((ls >> 2) == q) result[r] = v;
-                    }
-                }
-                const int j = j0 + lane;
-                if (j < j_end) {
-#pragma unroll
-                    for (int r = 0; r < R; ++r) out[first[r] + j] = val[first[r] + j] * result[r];
-                }
+                for (int r = 0; r < R; ++r) out[first[r] + j] = val[first[r] + j] * result[r];
             }
         }
     }
     if constexpr (WPG == 1) {
-        // the nonzeros outside the run, of the four rows at once: 64 slots per row and step,
-        // their columns and values loaded together, their dot products one row after the other
-        // without a wait in between (row after row, a wave sits through the memory round trips
-        // of every row)
-        typename S::Reg a[R][1][S::kRegs];
-        int row_first[R], split[R], cnt[R], max_cnt = 0;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
-            row_first[r] = first[r] - d.pos[r];
-            split[r] = d.pos[r];
-            cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (first[r] + d.len)); // the slots before the run + those after it
-            max_cnt = max(max_cnt, cnt[r]);
-        }
-        const T* rhs_lane = rhs + ls * VEC;
-        for (int off = 0; off < max_cnt; off += kWave) {
-            const int slot = off + lane;
-            int idx[R];
-            float v[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                idx[r] = -1;
-                v[r] = 0.f;
-                int c = 0;
-                if (off + (lane & 32) < cnt[r]) { // (a row without slots in this half of the step reads nothing)
-                    const bool live = slot < cnt[r];
-                    const int at = live ? slot : cnt[r] - 1; // (lanes past the end repeat the last slot and store nothing)
-                    const int i = row_first[r] + at + (at >= split[r] ? d.len : 0);
-                    c = col[i];
-                    if (live) {
-                        idx[r] = i;
-                        v[r] = val[i];
-                    }
-                }
-                lds[(wave * R + r) * kWave + lane] = c;
-            }
-            wave_lds_sync();
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (off + (lane & 32) < cnt[r]) {
-                    const float dot = sddmm_unit_staged<T, KT, 1, EDGE>(rhs_lane, a[r], k, lds + (wave * R + r) * kWave, lane);
-                    if (idx[r] >= 0) out[idx[r]] = v[r] * dot;
-                }
-            }
-            wave_lds_sync();
-        }
+        sddmm_group_leftovers<T, KT, EDGE>(d, row0, first, k, lane, lds + wave * kGroupRows * kWave, row_ptr, col, val, lhs, rhs,
+                                           out);
     } else {
         // the rows this wave finishes: their nonzeros before and after the run
 #pragma unroll

@@ -103,16 +103,17 @@ def test_grouped_rows_against_oracle(k, half):
         assert np.abs(C.cpu().numpy() - want).max() <= 1e-12 * max(1.0, np.abs(want).max())
 
 
-@pytest.mark.parametrize("half", [False, True])
-def test_one_wave_per_group(half):
+@pytest.mark.parametrize("k,half", [(64, False), (64, True), (48, False), (72, True), (32, False), (128, False)])
+def test_one_wave_per_group(k, half):
     """From 2048 groups with a run on, a group is the work of one wave instead of one
-    workgroup (no sums through LDS): the same checks on a matrix with about 2250 such groups."""
+    workgroup (no sums through LDS): the same checks on a matrix with about 2250 such groups,
+    at widths that fill a lane tile and at widths that do not (48, 72)."""
     import oracle
     from gpu_common import TOL_F16, TOL_F32, make_csr, round_half, run_sddmm, run_spmm
     from helpers import spmm_row_l1_error, sddmm_row_l1_errors
     from rode_amd import rode_sddmm_hip
     rng = np.random.default_rng(11)
-    m, n, k = 12002, 12500, 64
+    m, n = 12002, 12500
     rp, col, val = _window_matrix(rng, m, n, 96, 6)
     csr = make_csr(rp, col, val, m, n, k, locality=True)
     assert isinstance(csr.plan, rode_sddmm_hip.GroupPlan) and csr.plan.counts[1] >= 2048
