@@ -213,11 +213,13 @@ int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_
 /*
  * Group plan (no counterpart in the reference either).  For matrices whose adjacent rows
  * share long runs of consecutive column indices (sliding-window attention masks, dense
- * bands, block structure): groups of RODE_HIP_GROUP_ROWS adjacent rows whose common run
- * has at least 64 columns and holds at least three quarters of their nonzeros are
- * processed by kernels of their own, which load every dense row of the run once for all
- * rows of the group (and compute its address instead of reading column indices).  The
- * other kernels leave those rows out.  Same results up to the order of the fp32 additions.
+ * bands, block structure): groups of RODE_HIP_GROUP_ROWS adjacent rows whose longest runs
+ * have at least 64 columns in common, holding at least three quarters of their nonzeros,
+ * and start and end within 255 columns of each other, are processed by kernels of their
+ * own.  Those walk the columns the runs cover between them once, load every dense row of
+ * that range once for all rows of the group (its address follows from the range, no column
+ * index is read), and leave a row out at the columns outside its own run.  The other
+ * kernels leave those rows out.  Same results up to the order of the fp32 additions.
  *   d_plan       rode_hip_group_plan_bytes(M) bytes, 16-byte aligned, out
  *   h_counts     HOST int[4], out (the call waits for its kernels): [0] groups (M / 4,
  *                whole groups only), [1] groups with a run, [2] rows outside those groups

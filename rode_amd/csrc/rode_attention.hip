@@ -180,11 +180,14 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     const int ls = lane % LPR, group = lane / LPR;
     const int row0 = g * R;
     typename DotVec<T>::Reg a[R][1][DotVec<T>::kRegs];
-    int first[R]; // where the run starts in column_indices / values, per row
+    // per row: the slot of column j of the range is first[r] + j, for the columns j of the row's own run, from[r] <= j < to[r]
+    int first[R], from[R], to[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         load_lhs_slice<T, D, 1, false>(q, row0 + r, D, lane, a[r]);
-        first[r] = row_ptr[row0 + r] + d.pos[r];
+        from[r] = d.head(r);
+        to[r] = d.len - d.tail(r);
+        first[r] = row_ptr[row0 + r] + d.pos[r] - from[r];
     }
     const T* k_lane = k + ls * VEC;
     const T* v_lane = v + ls * VEC;
@@ -202,7 +205,6 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
     for (int j0 = 0; j0 < d.len; j0 += kWave) {
         const int j = j0 + lane;
-        const bool live = j < d.len;
         float dot[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) dot[r] = 0.f;
@@ -231,6 +233,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
+            const bool live = j >= from[r] && j < to[r];
             const float sc = live ? scale * (val[first[r] + j] * dot[r]) : -INFINITY;
             lds_p[wave][r][lane] = softmax_step<VEC>(sc, live, m_run[r], l_lane[r], acc[r]);
             if (WRITE_P && live) {
@@ -267,12 +270,12 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int s = row_ptr[row0 + r], e = row_ptr[row0 + r + 1];
-        const int split = d.pos[r], cnt = split + (e - (s + split + d.len));
+        const int split = d.pos[r], jump = to[r] - from[r], cnt = e - s - jump;
         for (int off = 0; off < cnt; off += kWave) {
             const int slot = off + lane;
             const bool live = slot < cnt;
             const int at = live ? slot : cnt - 1;
-            const int idx = s + at + (at >= split ? d.len : 0);
+            const int idx = s + at + (at >= split ? jump : 0);
             const int c = col[idx];
             const float w = val[idx];
             float sc = -INFINITY;
@@ -306,14 +309,16 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
         if (WRITE_P) {
             // every lane normalises the scores it wrote itself: same walk over the run and over the rest
             const float m_safe = m_run[r] == -INFINITY ? 0.f : m_run[r];
-            for (int j = lane; j < d.len; j += kWave) {
-                const float sc = j < kGroupScoresKept ? my_s[r * kGroupScoresKept + j] : probs[first[r] + j];
-                probs[first[r] + j] = __expf(sc - m_safe) * inv;
+            for (int j = lane; j < to[r]; j += kWave) {
+                if (j >= from[r]) {
+                    const float sc = j < kGroupScoresKept ? my_s[r * kGroupScoresKept + j] : probs[first[r] + j];
+                    probs[first[r] + j] = __expf(sc - m_safe) * inv;
+                }
             }
             const int s = row_ptr[row0 + r], e = row_ptr[row0 + r + 1];
-            const int split = d.pos[r], cnt = split + (e - (s + split + d.len));
+            const int split = d.pos[r], jump = to[r] - from[r], cnt = e - s - jump;
             for (int slot = lane; slot < cnt; slot += kWave) {
-                const int idx = s + slot + (slot >= split ? d.len : 0);
+                const int idx = s + slot + (slot >= split ? jump : 0);
                 probs[idx] = __expf(probs[idx] - m_safe) * inv;
             }
         }

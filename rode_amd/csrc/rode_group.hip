@@ -10,9 +10,11 @@
 //
 //   group_runs_kernel   per row: its longest run of consecutive columns (first column,
 //                       length, position in the row); one wave per row.
-//   group_desc_kernel   per group: the intersection of its rows' runs; the group is kept
-//                       if that run has at least kGroupMinRun columns and holds at least
-//                       three quarters of the group's nonzeros.
+//   group_desc_kernel   per group: the columns its rows' runs have in common and the range
+//                       they cover between them; the group is kept if the common part has
+//                       at least kGroupMinRun columns and holds at least three quarters of
+//                       the group's nonzeros, and the runs start and end within 255 columns
+//                       of each other.
 #include "rode_items.hpp"
 #include "rode_internal.hpp"
 
@@ -73,25 +75,36 @@ group_desc_kernel(int groups, const int* __restrict__ row_ptr, const int* __rest
     const int g = blockIdx.x * kWgThreads + threadIdx.x;
     if (g >= groups) return;
     RowGroup d;
-    int lo = 0, hi = 0x7fffffff;
+    int lo = 0, hi = 0x7fffffff;           // the columns all four runs hold
+    int first = 0x7fffffff, last = 0;      // the columns any of them holds
     long long slots = 0;
 #pragma unroll
     for (int r = 0; r < kGroupRows; ++r) {
         const int row = g * kGroupRows + r;
-        lo = max(lo, runs[3 * row]);
-        hi = min(hi, runs[3 * row] + runs[3 * row + 1]);
+        const int a = runs[3 * row], b = a + runs[3 * row + 1];
+        lo = max(lo, a);
+        hi = min(hi, b);
+        first = min(first, a);
+        last = max(last, b);
         slots += row_ptr[row + 1] - row_ptr[row];
     }
-    const int len = hi - lo;
-    const bool keep = len >= kGroupMinRun && 4ll * kGroupRows * len >= 3 * slots;
-    d.lo = keep ? lo : 0;
-    d.len = keep ? len : 0;
+    const int common = hi - lo;
+    // kept: a long common part that holds most of the group's nonzeros, and runs that start and
+    // end within 255 columns of each other (what a byte per row can say)
+    const bool keep = common >= kGroupMinRun && 4ll * kGroupRows * common >= 3 * slots && lo - first <= 255 && last - hi <= 255;
+    d.lo = keep ? first : 0;
+    d.len = keep ? last - first : 0;
+    d.heads = d.tails = 0u;
 #pragma unroll
     for (int r = 0; r < kGroupRows; ++r) {
         const int row = g * kGroupRows + r;
-        d.pos[r] = keep ? runs[3 * row + 2] + (lo - runs[3 * row]) : 0;
+        const int a = runs[3 * row], b = a + runs[3 * row + 1];
+        d.pos[r] = keep ? runs[3 * row + 2] : 0;
+        if (keep) {
+            d.heads |= (unsigned)(a - first) << (8 * r);
+            d.tails |= (unsigned)(last - b) << (8 * r);
+        }
     }
-    d.reserved[0] = d.reserved[1] = 0;
     reinterpret_cast<RowGroup*>(plan + kGroupHeaderInts)[g] = d;
     if (keep) {
         atomicAdd(plan + 1, 1);

@@ -11,11 +11,21 @@ namespace rode {
 // Rows that the kernels of a plan have taken out of the two lists (see the hub plan and the
 // group plan below): the standard kernels ask before they touch a row.
 constexpr int kGroupRows = 4; // rows of one group of the group plan
+// A kept group: every row has a run of consecutive columns, and the runs cover [lo, lo + len)
+// between them - row r's own run is [lo + head(r), lo + len - tail(r)), with head and tail
+// below 256 (the runs of a sliding window start and end a column apart from row to row).
+// The group kernels walk the whole range for all rows; a row takes no part at the columns
+// outside its own run.
 struct RowGroup {
-    int lo, len;          // the run of consecutive columns [lo, lo + len) that all rows of the group hold; len 0: no group
-    int pos[kGroupRows];  // where the run starts in each row (slots from the row's first nonzero)
-    int reserved[2];
+    int lo, len;          // the columns [lo, lo + len) that the runs of the group's rows cover; len 0: no group
+    int pos[kGroupRows];  // where its own run starts in each row (slots from the row's first nonzero)
+    unsigned heads;       // byte r: columns of the range before row r's run
+    unsigned tails;       // byte r: columns of the range after row r's run
+    __host__ __device__ int head(int r) const { return (int)((heads >> (8 * r)) & 255u); }
+    __host__ __device__ int tail(int r) const { return (int)((tails >> (8 * r)) & 255u); }
+    __host__ __device__ int run(int r) const { return len - head(r) - tail(r); } // length of row r's own run
 };
+static_assert(sizeof(RowGroup) == 32, "the group plan holds 32 bytes per group");
 struct RowOwners {
     int hub_min_len = 0;              // > 0: rows of that aligned length or more belong to the hub kernels
     const RowGroup* groups = nullptr; // the groups of a group plan, or null

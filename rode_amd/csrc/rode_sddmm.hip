@@ -209,7 +209,7 @@ sddmm_pair_kernel(int g1, int m1, int m2, int k, RowOwners owners, const int* __
 // other without a wait in between (row after row, a wave sits through the memory round trips
 // of every row).  lds_cols: kGroupRows * 64 ints of this wave.
 template <typename T, int KT, bool EDGE>
-__device__ __forceinline__ void sddmm_group_leftovers(const RowGroup& d, int row0, const int (&first)[kGroupRows], int k, int lane,
+__device__ __forceinline__ void sddmm_group_leftovers(const RowGroup& d, int row0, int k, int lane,
                                                       int* lds_cols, const int* __restrict__ row_ptr,
                                                       const int* __restrict__ col, const float* __restrict__ val,
                                                       const T* __restrict__ lhs, const T* __restrict__ rhs,
@@ -218,13 +218,14 @@ __device__ __forceinline__ void sddmm_group_leftovers(const RowGroup& d, int row
     using S = SddmmShape<T, KT>;
     constexpr int R = kGroupRows;
     typename S::Reg a[R][1][S::kRegs];
-    int row_first[R], split[R], cnt[R], max_cnt = 0;
+    int row_first[R], split[R], jump[R], cnt[R], max_cnt = 0;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         load_lhs_slice<T, KT, 1, EDGE>(lhs, row0 + r, k, lane, a[r]);
-        row_first[r] = first[r] - d.pos[r];
+        row_first[r] = row_ptr[row0 + r];
         split[r] = d.pos[r];
-        cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (first[r] + d.len)); // the slots before the run + those after it
+        jump[r] = d.run(r);
+        cnt[r] = row_ptr[row0 + r + 1] - row_first[r] - jump[r]; // the slots before the run + those after it
         max_cnt = max(max_cnt, cnt[r]);
     }
     const T* rhs_lane = rhs + (lane % S::kLpr) * S::kVec;
@@ -240,7 +241,7 @@ __device__ __forceinline__ void sddmm_group_leftovers(const RowGroup& d, int row
             if (off + (lane & 32) < cnt[r]) { // (a row without slots in this half of the step reads nothing)
                 const bool live = slot < cnt[r];
                 const int at = live ? slot : cnt[r] - 1; // (lanes past the end repeat the last slot and store nothing)
-                const int i = row_first[r] + at + (at >= split[r] ? d.len : 0);
+                const int i = row_first[r] + at + (at >= split[r] ? jump[r] : 0);
                 c = col[i];
                 if (live) {
                     idx[r] = i;
@@ -289,9 +290,14 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     if (d.len <= 0) return; // not a group: its rows are in the lists
     const int w = wave % WPG; // this wave among the waves of its group
     const int row0 = g * R;
-    int first[R]; // where the run starts in column_indices / values, per row
+    // per row: the slot of column j of the range is at[r] + j, for the columns j of the row's own run, from[r] <= j < to[r]
+    int at[R], from[R], to[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) first[r] = row_ptr[row0 + r] + d.pos[r];
+    for (int r = 0; r < R; ++r) {
+        from[r] = d.head(r);
+        to[r] = d.len - d.tail(r);
+        at[r] = row_ptr[row0 + r] + d.pos[r] - from[r];
+    }
     // this wave's share of the run, in quads of columns; lane e of a step has column j0 + e
     const int quads = (d.len + 3) / 4;
     const int q_begin = quads * w / WPG, q_end = quads * (w + 1) / WPG;
@@ -352,23 +358,21 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
                 }
             }
             const int j = j0 + lane;
-            if (j < j_end) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) out[first[r] + j] = val[first[r] + j] * result[r];
-            }
+            for (int r = 0; r < R; ++r)
+                if (j >= from[r] && j < min(to[r], j_end)) out[at[r] + j] = val[at[r] + j] * result[r];
         }
     }
     if constexpr (WPG == 1) {
-        sddmm_group_leftovers<T, KT, EDGE>(d, row0, first, k, lane, lds + wave * kGroupRows * kWave, row_ptr, col, val, lhs, rhs,
-                                           out);
+        sddmm_group_leftovers<T, KT, EDGE>(d, row0, k, lane, lds + wave * kGroupRows * kWave, row_ptr, col, val, lhs, rhs, out);
     } else {
         // the rows this wave finishes: their nonzeros before and after the run
 #pragma unroll
         for (int r = w; r < R; r += WPG) {
             const int row = row0 + r, s = row_ptr[row], e = row_ptr[row + 1];
-            const int run_first = s + d.pos[r], run_end = run_first + d.len;
+            const int run_first = s + d.pos[r], run_end = run_first + d.run(r);
             // (the slots before the run and, in the same pass, those after it)
-            sddmm_row_slots<T, KT, 1, EDGE>(row, s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, k, lane,
+            sddmm_row_slots<T, KT, 1, EDGE>(row, s, 0, (run_first - s) + (e - run_end), run_first - s, d.run(r), k, lane,
                                             lds + wave * kWave, col, val, lhs, rhs, out);
         }
     }

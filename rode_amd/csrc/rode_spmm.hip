@@ -333,9 +333,14 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     const bool col_ok = !EDGE || tile + ls * VEC < n;
     const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
     const int row0 = g * R;
-    int first[R]; // where the run starts in column_indices / values, per row
+    // per row: the slot of column j of the range is at[r] + j, for the columns j of the row's own run, from[r] <= j < to[r]
+    int at[R], from[R], to[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) first[r] = row_ptr[row0 + r] + d.pos[r];
+    for (int r = 0; r < R; ++r) {
+        from[r] = d.head(r);
+        to[r] = d.len - d.tail(r);
+        at[r] = row_ptr[row0 + r] + d.pos[r] - from[r];
+    }
 
     // this wave's share of the run, in quads of columns
     const int quads = (d.len + 3) / 4;
@@ -353,7 +358,10 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     const unsigned lane_off = 4u * group * row_bytes + (col_ok ? ls * VEC * (unsigned)sizeof(T) : 0u); // in bytes
     A v_next[R]; // the values of the next step are loaded while this one is computed
 #pragma unroll
-    for (int r = 0; r < R; ++r) v_next[r] = 4 * q_begin + lane < j_end ? val[first[r] + 4 * q_begin + lane] : A(0);
+    for (int r = 0; r < R; ++r) {
+        const int j = 4 * q_begin + lane;
+        v_next[r] = j >= from[r] && j < min(to[r], j_end) ? val[at[r] + j] : A(0);
+    }
     for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
 #pragma unroll
         for (int r = 0; r < R; ++r) lds_v[wave][r][lane] = v_next[r];
@@ -361,7 +369,7 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
         {
             const int j = j0 + kWave + lane;
 #pragma unroll
-            for (int r = 0; r < R; ++r) v_next[r] = j < j_end ? val[first[r] + j] : A(0);
+            for (int r = 0; r < R; ++r) v_next[r] = j >= from[r] && j < min(to[r], j_end) ? val[at[r] + j] : A(0);
         }
         const int nq = min(kWave / 4, (j_end - j0 + 3) / 4);
 #pragma unroll
@@ -396,12 +404,13 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
         // the nonzeros outside the run, of the four rows at once: their columns and values are
         // loaded together and their gathers follow each other without a wait in between (row
         // after row, a wave would sit through two memory round trips per row and step)
-        int row_first[R], split[R], cnt[R], max_cnt = 0;
+        int row_first[R], split[R], jump[R], cnt[R], max_cnt = 0;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            row_first[r] = first[r] - d.pos[r];
+            row_first[r] = at[r] + from[r] - d.pos[r];
             split[r] = d.pos[r];
-            cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (first[r] + d.len)); // the slots before the run + those after it
+            jump[r] = to[r] - from[r];
+            cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (at[r] + to[r])); // the slots before the run + those after it
             max_cnt = max(max_cnt, cnt[r]);
         }
         for (int off = 0; off < max_cnt; off += kWave) {
@@ -413,8 +422,8 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
                 A v = A(0);
                 if (lane < ((live + 3) & ~3)) { // (slots past the end of the last quad: value 0, column of a real slot)
                     const bool past = slot >= cnt[r];
-                    const int at = past ? cnt[r] - 1 : slot;
-                    const int idx = row_first[r] + at + (at >= split[r] ? d.len : 0);
+                    const int slot_at = past ? cnt[r] - 1 : slot;
+                    const int idx = row_first[r] + slot_at + (slot_at >= split[r] ? jump[r] : 0);
                     c = col[idx];
                     v = past ? A(0) : val[idx];
                 }
@@ -458,9 +467,9 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
 #pragma unroll
         for (int r = w; r < R; r += WPG) {
             const int row = row0 + r, s = row_ptr[row], e = row_ptr[row + 1];
-            const int run_first = s + d.pos[r], run_end = run_first + d.len;
+            const int run_first = s + d.pos[r], run_end = run_first + d.run(r);
             A outside[VEC]; // the slots before the run and, in the same pass, those after it
-            spmm_sum_slots<T, TN>(s, 0, (run_first - s) + (e - run_end), run_first - s, d.len, lane, lds_c[wave][0],
+            spmm_sum_slots<T, TN>(s, 0, (run_first - s) + (e - run_end), run_first - s, d.run(r), lane, lds_c[wave][0],
                                   &lds_v[wave][0][0], b_lane, n, col, val, outside);
             if (group == 0 && col_ok) {
                 A* c_lane = C + (size_t)row * n + tile + ls * VEC;

@@ -236,8 +236,9 @@ class GroupPlan:
         return self.counts[1] > 0
 
     def groups(self):
-        """int32 array (groups, 8): first column and length of the shared run (0: none), its
-        position in each of the four rows, two unused."""
+        """int32 array (groups, 8): first column and length of the range the four rows' runs
+        cover (0: group not kept), the position of its own run in each row, and per row, a byte
+        each, how many columns of the range lie before and after its run."""
         return self.data[4:4 + 8 * self.counts[0]].cpu().numpy().reshape(-1, 8)
 
 

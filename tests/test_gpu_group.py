@@ -55,13 +55,17 @@ def test_plan_contents():
                     best = (int(c[i]), j - i + 1, i)
                 i = j + 1
             runs.append(best)
-        lo, hi = max(a for a, _, _ in runs), min(a + l for a, l, _ in runs)
+        lo, hi = max(a for a, _, _ in runs), min(a + l for a, l, _ in runs)       # what the four runs have in common
+        first, last = min(a for a, _, _ in runs), max(a + l for a, l, _ in runs)  # what they cover between them
         slots = rp[4 * g + 4] - rp[4 * g]
-        keep = hi - lo >= 64 and 16 * (hi - lo) >= 3 * slots
+        keep = hi - lo >= 64 and 16 * (hi - lo) >= 3 * slots and lo - first <= 255 and last - hi <= 255
         if keep:
             kept += 1
-            assert desc[g, 0] == lo and desc[g, 1] == hi - lo
-            assert desc[g, 2:6].tolist() == [p + lo - a for a, _, p in runs]
+            assert desc[g, 0] == first and desc[g, 1] == last - first
+            assert desc[g, 2:6].tolist() == [p for _, _, p in runs]
+            heads, tails = int(desc[g, 6]) & 0xffffffff, int(desc[g, 7]) & 0xffffffff
+            assert [(heads >> (8 * r)) & 255 for r in range(4)] == [a - first for a, _, _ in runs]
+            assert [(tails >> (8 * r)) & 255 for r in range(4)] == [last - a - l for a, l, _ in runs]
         else:
             assert desc[g, 1] == 0
     assert plan.counts[1] == kept and 0 < kept < m // 4   # the ragged rows break some groups
