@@ -107,6 +107,51 @@ def test_grouped_rows_against_oracle(k, half):
         assert np.abs(C.cpu().numpy() - want).max() <= 1e-12 * max(1.0, np.abs(want).max())
 
 
+@pytest.mark.parametrize("m,half", [(600, False), (9000, True)])
+def test_runs_that_shift_from_row_to_row(m, half):
+    """A window that moves eight columns per row: the four runs of a group start 0, 8, 16 and
+    24 columns into the range they cover, and every row is left out of the kernels' walk at
+    the columns it does not have.  600 rows: a workgroup per group; 9000 rows: a wave per group."""
+    import oracle
+    from gpu_common import TOL_F16, TOL_F32, make_csr, round_half, run_sddmm, run_spmm
+    from helpers import spmm_row_l1_error, sddmm_row_l1_errors
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(m)
+    k, window = 64, 200
+    n = 8 * m + window
+    rows = [np.array(sorted(set(range(8 * r, 8 * r + window)) | set(rng.choice(n, 10, replace=False).tolist())), dtype=np.int32)
+            for r in range(m)]
+    rp = np.zeros(m + 1, dtype=np.int32)
+    rp[1:] = np.cumsum([len(c) for c in rows])
+    col = np.concatenate(rows)
+    val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
+    csr = make_csr(rp, col, val, m, n, k, locality=True)
+    assert isinstance(csr.plan, rode_sddmm_hip.GroupPlan) and csr.plan.counts[1] >= (2048 if m > 8192 else 100)
+    desc = csr.plan.groups()
+    g = np.nonzero(desc[:, 1] > 0)[0][0]
+    heads = int(desc[g, 6]) & 0xffffffff
+    assert sorted((heads >> (8 * r)) & 255 for r in range(4))[-1] >= 24 and desc[g, 1] >= window + 24
+    B = rng.standard_normal((n, k)).astype(np.float32)
+    L = rng.standard_normal((m, k)).astype(np.float32)
+    Bq, Lq = (round_half(B), round_half(L)) if half else (B, L)
+    tol = TOL_F16 if half else TOL_F32
+    assert spmm_row_l1_error(run_spmm(csr, B, half), oracle.spmm_f64(rp, col, val, Bq)) <= tol
+    ref64, scale = oracle.sddmm_f64(rp, col, val, Lq, Bq, with_abs=True)
+    err, cond = sddmm_row_l1_errors(run_sddmm(csr, L, B, half), ref64, scale, rp)
+    assert float(err[cond <= 100].max(initial=0.0)) <= tol
+    if m > 8192:  # the fused attention forward on the same pattern, against the three kernels without a plan
+        from rode_amd import sparse_attention
+        plain = make_csr(rp, col, val, m, n, k, locality=False)
+        dev = csr.device
+        dt = torch.float16 if half else torch.float32
+        q = torch.from_numpy(L).to(dev, dt)
+        kk = torch.from_numpy(B).to(dev, dt)
+        vv = torch.from_numpy(rng.standard_normal((n, k)).astype(np.float32)).to(dev, dt)
+        a = sparse_attention(csr, q, kk, vv, scale=0.3, fused=True)
+        b = sparse_attention(plain, q, kk, vv, scale=0.3, fused=False)
+        assert (a - b).abs().max().item() <= 2e-3 * max(1.0, b.abs().max().item())
+
+
 @pytest.mark.parametrize("k,half", [(64, False), (64, True), (48, False), (72, True), (32, False), (128, False)])
 def test_one_wave_per_group(k, half):
     """From 2048 groups with a run on, a group is the work of one wave instead of one
