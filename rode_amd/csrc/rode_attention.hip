@@ -167,7 +167,6 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
 {
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
-    constexpr int QUADS = LPR / 4; // slot quads per lane group per 32-slot unit (SddmmShape::kQuads)
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) float lds_p[kWavesPerWg][R][kWave];
     __shared__ float lds_s[WRITE_P ? kWavesPerWg * R * kGroupScoresKept : 1];
@@ -179,12 +178,17 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     if (d.len <= 0) return; // not a group: attention_rows_kernel has its rows
     const int ls = lane % LPR, group = lane / LPR;
     const int row0 = g * R;
-    typename DotVec<T>::Reg a[R][1][DotVec<T>::kRegs];
+    // the scores of the run: LP lanes per k row, each with E of its 16-byte vectors (LP lanes apart), as in
+    // sddmm_group_kernel: a dot product crosses half as many lanes
+    constexpr int LP = LPR >= 8 ? LPR / 2 : LPR, E = LPR / LP;
+    const int lp = lane % LP;
+    typename DotVec<T>::Reg a[R][E][DotVec<T>::kRegs];
     // per row: the slot of column j of the range is first[r] + j, for the columns j of the row's own run, from[r] <= j < to[r]
     int first[R], from[R], to[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        load_lhs_slice<T, D, 1, false>(q, row0 + r, D, lane, a[r]);
+#pragma unroll
+        for (int i = 0; i < E; ++i) DotVec<T>::load(q + (size_t)(row0 + r) * D + (lp + LP * i) * VEC, a[r][i]);
         from[r] = d.head(r);
         to[r] = d.len - d.tail(r);
         first[r] = row_ptr[row0 + r] + d.pos[r] - from[r];
@@ -202,7 +206,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     }
 
     // the run: lane e of a step has column j0 + e
-    const int group_first = (lane & 31) - ls + (lane & 32); // first column (within the step) of this lane group
+    const int group_first = lane - lp; // first column (within the step) of this lane group
     for (int j0 = 0; j0 < d.len; j0 += kWave) {
         const int j = j0 + lane;
         float dot[R];
@@ -210,24 +214,29 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
         for (int r = 0; r < R; ++r) dot[r] = 0.f;
         if (j0 + (lane & 32) < d.len) { // the upper half sits out a step that has nothing for it
 #pragma unroll
-            for (int qd = 0; qd < QUADS; ++qd) {
+            for (int qd = 0; qd < LP / 4; ++qd) {
                 float p4[R][4];
-                const T* k_quad = k_lane + (size_t)(d.lo + j0 + group_first + 4 * qd) * D;
-                const int room = d.len - 1 - (j0 + group_first + 4 * qd); // (rows past the run repeat its last row)
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    const uint4 b = *reinterpret_cast<const uint4*>(k_quad + (ptrdiff_t)min(t, room) * D);
+                    // (rows past the range repeat its last row)
+                    const T* k_row = k + (size_t)(d.lo + min(j0 + group_first + 4 * qd + t, d.len - 1)) * D + lp * VEC;
 #pragma unroll
-                    for (int r = 0; r < R; ++r) p4[r][t] = DotVec<T>::dot_raw(a[r][0], b, 0.f);
+                    for (int r = 0; r < R; ++r) p4[r][t] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < E; ++i) {
+                        const uint4 b = *reinterpret_cast<const uint4*>(k_row + LP * i * VEC);
+#pragma unroll
+                        for (int r = 0; r < R; ++r) p4[r][t] = DotVec<T>::dot_raw(a[r][i], b, p4[r][t]);
+                    }
                 }
-                const bool hi2 = ls & 2, hi1 = ls & 1;
+                const bool hi2 = lp & 2, hi1 = lp & 1;
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const float q0 = (hi2 ? p4[r][2] : p4[r][0]) + lane_xor2(hi2 ? p4[r][0] : p4[r][2]);
                     const float q1 = (hi2 ? p4[r][3] : p4[r][1]) + lane_xor2(hi2 ? p4[r][1] : p4[r][3]);
                     float sum = (hi1 ? q1 : q0) + lane_xor1(hi1 ? q0 : q1);
-                    sum = butterfly_sum<4, LPR>(sum);
-                    if ((ls >> 2) == qd) dot[r] = sum;
+                    sum = butterfly_sum<4, LP>(sum);
+                    if ((lp >> 2) == qd) dot[r] = sum;
                 }
             }
         }
@@ -271,6 +280,8 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     for (int r = 0; r < R; ++r) {
         const int s = row_ptr[row0 + r], e = row_ptr[row0 + r + 1];
         const int split = d.pos[r], jump = to[r] - from[r], cnt = e - s - jump;
+        typename DotVec<T>::Reg a_row[1][DotVec<T>::kRegs]; // this row of q as the lanes of sddmm_unit hold it
+        load_lhs_slice<T, D, 1, false>(q, row0 + r, D, lane, a_row);
         for (int off = 0; off < cnt; off += kWave) {
             const int slot = off + lane;
             const bool live = slot < cnt;
@@ -280,7 +291,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
             const float w = val[idx];
             float sc = -INFINITY;
             if (off + (lane & 32) < cnt) {
-                const float dd = sddmm_unit<T, D, 1, false>(k_lane, a[r], c, D, my_c, lane);
+                const float dd = sddmm_unit<T, D, 1, false>(k_lane, a_row, c, D, my_c, lane);
                 if (live) sc = scale * (w * dd);
             }
             my_p[lane] = softmax_step<VEC>(sc, live, m_run[r], l_lane[r], acc[r]);
