@@ -49,19 +49,30 @@ constexpr int kOwnedMinSegments = 16384;
 // own: it needs a quarter of the block kernel's registers and keeps twice the waves per CU.
 constexpr int kPairMaxWorkgroups = 16384;
 
+// A row of C that is written once and not read again by the kernel that writes it: stored
+// with the non-temporal hint, so that it does not push the gathered rows of B out of the
+// caches on its way (config 4, K=128: residue kernel 1.19 -> 1.09 ms; the same hint on the
+// loads of B, on SDDMM's loads of rhs or on its stores of `out` made those kernels slower).
 template <int VEC>
 __device__ __forceinline__ void store_row(float* dst, const float (&acc)[VEC])
 {
+    typedef float Quad __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int x = 0; x < VEC; x += 4)
-        *reinterpret_cast<float4*>(dst + x) = make_float4(acc[x], acc[x + 1], acc[x + 2], acc[x + 3]);
+    for (int x = 0; x < VEC; x += 4) {
+        const Quad v = {acc[x], acc[x + 1], acc[x + 2], acc[x + 3]};
+        __builtin_nontemporal_store(v, reinterpret_cast<Quad*>(dst + x));
+    }
 }
 
 template <int VEC>
 __device__ __forceinline__ void store_row(double* dst, const double (&acc)[VEC])
 {
+    typedef double Pair __attribute__((ext_vector_type(2)));
 #pragma unroll
-    for (int x = 0; x < VEC; x += 2) *reinterpret_cast<double2*>(dst + x) = make_double2(acc[x], acc[x + 1]);
+    for (int x = 0; x < VEC; x += 2) {
+        const Pair v = {acc[x], acc[x + 1]};
+        __builtin_nontemporal_store(v, reinterpret_cast<Pair*>(dst + x));
+    }
 }
 
 // Sum over the aligned slots [base, base + cnt) of values * B rows, for this lane's columns
