@@ -148,6 +148,13 @@ struct DotVec {
         for (int x = 0; x < kRegs; ++x) a[x] = 0.f;
     }
     __device__ __forceinline__ static void load(const T* p, Reg (&a)[kRegs]) { DenseVec<T>::load(p, a); }
+    // the same for a row that nobody reads again soon: loaded with the non-temporal hint
+    __device__ __forceinline__ static void load_once(const T* p, Reg (&a)[kRegs])
+    {
+        typedef unsigned Quad __attribute__((ext_vector_type(4)));
+        const Quad v = __builtin_nontemporal_load(reinterpret_cast<const Quad*>(p));
+        DenseVec<T>::unpack(make_uint4(v[0], v[1], v[2], v[3]), a);
+    }
     __device__ __forceinline__ static float dot_raw(const Reg (&a)[kRegs], const uint4& raw, float acc)
     {
         float b[kRegs];
@@ -176,6 +183,12 @@ struct DotVec<__half> {
     {
         const uint4 raw = *reinterpret_cast<const uint4*>(p);
         a[0] = raw.x; a[1] = raw.y; a[2] = raw.z; a[3] = raw.w;
+    }
+    __device__ __forceinline__ static void load_once(const __half* p, Reg (&a)[kRegs])
+    {
+        typedef unsigned Quad __attribute__((ext_vector_type(4)));
+        const Quad v = __builtin_nontemporal_load(reinterpret_cast<const Quad*>(p));
+        a[0] = v[0]; a[1] = v[1]; a[2] = v[2]; a[3] = v[3];
     }
     __device__ __forceinline__ static float dot_raw(const Reg (&a)[kRegs], const uint4& raw, float acc)
     {

@@ -134,7 +134,7 @@ sddmm_residue_body(int bid, int nblocks, int m2, int k, RowOwners owners, const 
         }
     }
     typename S::Reg a[NS][S::kRegs];
-    load_lhs_slice<T, KT, NS, EDGE>(lhs, row, k, lane, a);
+    load_lhs_slice<T, KT, NS, EDGE, true>(lhs, row, k, lane, a);
     const T* rhs_lane = rhs + ls * VEC;
     wave_lds_sync();
 

@@ -80,7 +80,11 @@ __device__ __forceinline__ float sddmm_unit(const T* __restrict__ rhs_lane,
     return sddmm_unit_staged<T, KT, NS, EDGE>(rhs_lane, a, k, lds_cols, lane);
 }
 
-template <typename T, int KT, int NS, bool EDGE>
+// ONCE: the row is used by this work item only (a residue row): loaded with the non-temporal
+// hint, so that the stream of lhs rows does not displace gathered rhs rows (config 4: residue
+// kernel 1.375 -> 1.334 ms at K=128, 0.656 -> 0.626 at K=64; for the group kernels, which
+// read their lhs rows twice, the hint costs 8 %).
+template <typename T, int KT, int NS, bool EDGE, bool ONCE = false>
 __device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int row, int k, int lane,
                                                typename DotVec<T>::Reg (&a)[NS][DotVec<T>::kRegs])
 {
@@ -89,7 +93,12 @@ __device__ __forceinline__ void load_lhs_slice(const T* __restrict__ lhs, int ro
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
         DotVec<T>::zero(a[s]);
-        if (!EDGE || e0 + s * KT < k) DotVec<T>::load(lhs + (size_t)row * k + e0 + s * KT, a[s]);
+        if (!EDGE || e0 + s * KT < k) {
+            if constexpr (ONCE)
+                DotVec<T>::load_once(lhs + (size_t)row * k + e0 + s * KT, a[s]);
+            else
+                DotVec<T>::load(lhs + (size_t)row * k + e0 + s * KT, a[s]);
+        }
     }
 }
 
