@@ -150,8 +150,9 @@ __device__ __forceinline__ float softmax_step(float sc, bool live, float& m_run,
 }
 
 // The groups of a group plan (rode_group.hip): one wave per group of four adjacent rows
-// that share a run of consecutive columns.  Along the run every k row and every v row is
-// loaded once for the four rows (the score part is the SDDMM group kernel's, the output
+// whose runs of consecutive columns cover a range between them.  Along the range every k row
+// and every v row is loaded once for the four rows (a row's score is -inf, its probability
+// zero, at the columns outside its own run) (the score part is the SDDMM group kernel's, the output
 // part the SpMM group kernel's, with a running softmax per row in between); then the wave
 // takes the nonzeros outside the run, row by row, the way attention_rows_kernel does.
 // With WRITE_P the raw scores of the first kGroupScoresKept columns of the run wait in LDS,

@@ -1,9 +1,10 @@
-// Group plan: groups of kGroupRows adjacent rows that share a long run of consecutive
-// column indices (sliding-window attention masks, dense bands, block structure).  The
-// group kernels (spmm_group_kernel, sddmm_group_kernel) walk the shared run once for all
-// rows of a group: one gather of a dense row serves every row of the group, and the dense
-// rows of a run are consecutive in memory, so no column index is read for them.  The
-// nonzeros of a row outside the run are processed as usual, by the same workgroup; the
+// Group plan: groups of kGroupRows adjacent rows whose longest runs of consecutive column
+// indices overlap for the most part (sliding-window attention masks, dense bands, block
+// structure).  The group kernels (spmm_group_kernel, sddmm_group_kernel,
+// attention_group_kernel) walk the range of columns the runs cover between them once for
+// all rows of a group: one load of a dense row serves every row of the group, and the dense
+// rows of the range are consecutive in memory, so no column index is read for them.  The
+// nonzeros of a row outside its run are processed as usual, by the same workgroup; the
 // standard kernels leave grouped rows out.  No counterpart in the reference, whose kernels
 // gather the dense row of every nonzero of every row (RoDe_SpMM/RoDeSpmm.cu:140-160,
 // RoDe_SDDMM/RoDeSddmm.cu:96-140).  The plan changes no result.

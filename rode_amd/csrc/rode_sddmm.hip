@@ -262,12 +262,15 @@ __device__ __forceinline__ void sddmm_group_leftovers(const RowGroup& d, int row
     }
 }
 
-// The groups of a group plan (rode_group.hip): one workgroup per group of four adjacent
-// rows that share a run of consecutive columns.  The waves split the run; every rhs row of
-// it is loaded once (its address follows from the run, no column index is read) and
-// multiplied with the lhs rows of all four rows of the group, which stay in registers.
-// Wave w then computes row w's nonzeros outside the run as usual.  Single-slab rows only
-// (k <= 128 elements per lane tile): four lhs slices of more slabs would not fit.
+// The groups of a group plan (rode_group.hip): four adjacent rows whose runs of consecutive
+// columns cover the range [lo, lo + len) between them.  One wave per group (WPG = 1), or a
+// workgroup whose four waves split the range.  Every rhs row of the range is loaded once
+// (its address follows from the range, no column index is read) and multiplied with the lhs
+// rows of all four rows of the group, which stay in registers; a row gets no output at the
+// columns outside its own run.  Then the rows' nonzeros outside their runs: with one wave per
+// group, of the four rows together (sddmm_group_leftovers); with a workgroup, wave w takes
+// row w's.  Single-slab rows only (k <= 128 elements per lane tile): four lhs slices of more
+// slabs would not fit.
 // (A variant in which the four waves of a workgroup took four consecutive groups and read
 // the union of their runs through LDS tiles, loaded once per workgroup, ran in the same
 // time on config 5 - 0.049 ms fp32, 0.035 against 0.033 ms fp16 - and was taken out.)

@@ -311,12 +311,14 @@ spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, RowOwners owner
                                        B, C, plan);
 }
 
-// The groups of a group plan (rode_group.hip): one workgroup per group of four adjacent
-// rows that share a run of consecutive columns.  The waves split the run; every dense row
-// of it is loaded once and multiplied into the sums of all four rows (its address follows
-// from the run, no column index is read).  Wave w then adds row w's nonzeros outside the
-// run, the waves' sums meet in LDS, and wave w adds the total of row w to C (the row is in
-// no other work item: no atomics).
+// The groups of a group plan (rode_group.hip): four adjacent rows whose runs of consecutive
+// columns cover the range [lo, lo + len) between them.  One wave per group (WPG = 1), or a
+// workgroup whose four waves split the range.  Every dense row of the range is loaded once
+// and multiplied into the sums of all four rows (its address follows from the range, no
+// column index is read; a row's value is zero at the columns outside its own run).  Then the
+// rows' nonzeros outside their runs: with one wave per group, of the four rows together;
+// with a workgroup, wave w adds row w's, the waves' sums meet in LDS, and wave w adds the
+// total of row w to C.  A row is in no other work item: no atomics.
 template <typename T, int TN, bool EDGE, int WPG>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
