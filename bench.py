@@ -29,15 +29,20 @@ TOL = {"f32": 1e-4, "f16": 2e-3}  # max over rows of |err|_inf / |ref row|_1
 
 
 def kernel_sources_fingerprint():
-    """Hash of the SpMM / SDDMM kernel sources.  Every entry of profiles/traffic.json
-    carries the fingerprint of the sources it was measured on; an entry measured on other
-    sources is not reported."""
+    """Hash of the code of the SpMM / SDDMM kernel sources (comments and blank lines left
+    out, so that rewording a comment does not disown a measurement).  Every entry of
+    profiles/traffic.json carries the fingerprint of the sources it was measured on; an
+    entry measured on other sources is not reported."""
     import hashlib
+    import re
     h = hashlib.sha256()
     for name in ("rode_device.hpp", "rode_items.hpp", "rode_units.hpp", "rode_window.hpp", "rode_spmm.hip", "rode_sddmm.hip",
                  "rode_spmm_window.hip", "rode_sddmm_window.hip"):
-        with open(os.path.join(ROOT, "rode_amd", "csrc", name), "rb") as f:
-            h.update(f.read())
+        with open(os.path.join(ROOT, "rode_amd", "csrc", name), "r", encoding="utf-8") as f:
+            for line in f:
+                code = re.sub(r"//.*$", "", line).strip()
+                if code:
+                    h.update(code.encode("utf-8") + b"\n")
     return h.hexdigest()[:16]
 
 
