@@ -10,6 +10,8 @@ gradient is again one of the two kernels on the same pattern or on its transpose
     C   = A B                   :  dB = A^T dC               (SpMM, transposed pattern)
                                    dv = (dC B^T)|pattern      (SDDMM with unit values)
 """
+import ctypes
+
 import torch
 
 from . import _lib, rode_sddmm_hip
@@ -130,7 +132,6 @@ def _attention_call(csr, values, q, k, v, scale, want_probs):
     if values.numel() == 0:  # no nonzeros: nothing attends to anything
         return torch.zeros((m, d), dtype=torch.float32, device=q.device), probs
     out = torch.empty((m, d), dtype=torch.float32, device=q.device)
-    import ctypes
     plans = rode_sddmm_hip.plans_struct(csr.plan if isinstance(csr.plan, rode_sddmm_hip.GroupPlan) else None)
     with torch.cuda.device(q.device):
         code = lib.rode_hip_attention_forward(
