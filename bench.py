@@ -361,6 +361,9 @@ def main():
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": dom["algorithmic_GBs"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(dom["algorithmic_GBs"] / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "traffic_source": traffic_note,
+                # the same kernel's measured HBM bytes over its time: how busy the memory system was
+                "traffic_GBs": None if traffic is None else round(traffic / kernels[dominant] / 1e6, 1),
+                "traffic_frac": None if traffic is None else round(traffic / kernels[dominant] / 1e6 / HBM_PEAK_GBS, 4),
                 "gather_model_frac": round(dom["gather_model_GBs"] / HBM_PEAK_GBS, 4)}
 
     # ---- CPU baseline: the oracle on a bounded sample of the same matrix --------
