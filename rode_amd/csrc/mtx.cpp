@@ -14,6 +14,8 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -105,7 +107,7 @@ extern "C" {
 
 // Parses the text of a Matrix Market file.  Returns a handle (rode_mtx_free it) and the
 // shape and nonzero count of the CSR matrix, or NULL with a message in err.
-void* rode_mtx_parse(const char* data, size_t len, int* m_out, int* n_out, long long* nnz_out, char* err, int errlen)
+static void* parse_text(const char* data, size_t len, int* m_out, int* n_out, long long* nnz_out, char* err, int errlen)
 {
     const char* p = data;
     const char* end = data + len;
@@ -154,6 +156,11 @@ void* rode_mtx_parse(const char* data, size_t len, int* m_out, int* n_out, long 
     }
     if (m > INT32_MAX || n > INT32_MAX || entries > (1ll << 40)) {
         fail(err, errlen, "matrix too large for 32-bit indices");
+        return nullptr;
+    }
+    // the mirrored entry (c, r) of a symmetric file must be a valid position as well
+    if (symmetry != "general" && m != n) {
+        fail(err, errlen, "a " + symmetry + " matrix must be square, got " + std::to_string(m) + " x " + std::to_string(n));
         return nullptr;
     }
 
@@ -263,6 +270,20 @@ void* rode_mtx_parse(const char* data, size_t len, int* m_out, int* n_out, long 
     *n_out = mat->n;
     *nnz_out = kept[m];
     return mat;
+}
+
+// No exception leaves the library: a size line that asks for more memory than there is
+// (std::bad_alloc from the tables sized by it) is reported like any other bad file.
+void* rode_mtx_parse(const char* data, size_t len, int* m_out, int* n_out, long long* nnz_out, char* err, int errlen)
+{
+    try {
+        return parse_text(data, len, m_out, n_out, nnz_out, err, errlen);
+    } catch (const std::bad_alloc&) {
+        fail(err, errlen, "out of memory: the size line describes a matrix that does not fit");
+    } catch (const std::exception& e) {
+        fail(err, errlen, std::string("parser error: ") + e.what());
+    }
+    return nullptr;
 }
 
 void rode_mtx_copy(void* handle, int* row_ptr, int* col, float* val)

@@ -79,6 +79,8 @@ def read_matrix_market(path, native=None):
         while line.startswith("%") or not line.strip():
             line = f.readline()
         m, n, entries = (int(t) for t in line.split()[:3])
+        if symmetry != "general" and m != n:
+            raise ValueError(f"{path}: a {symmetry} matrix must be square, got {m} x {n}")
         data = np.loadtxt(f, dtype=np.float64, ndmin=2, comments="%") if entries else np.zeros((0, 3))
     if data.shape[0] != entries:
         raise ValueError(f"{path}: header promises {entries} entries, file has {data.shape[0]}")

@@ -73,6 +73,42 @@ def test_large_file_in_parallel_pieces(tmp_path, parser):
     assert rp.tolist() == [0, 1, 2] and col.tolist() == [1, 0] and val.tolist() == [15.0, -0.25]
 
 
+@pytest.mark.parametrize("native", [True, False])
+def test_rejects_symmetric_files_that_are_not_square_and_sizes_beyond_memory(tmp_path, native):
+    """The mirrored entry of a symmetric file lands in row `column`: a non-square one is
+    refused before anything is counted.  A size line that no machine can hold comes back as
+    an error as well (nothing is thrown through the C boundary)."""
+    bad = tmp_path / "s.mtx"
+    for kind in ("symmetric", "skew-symmetric"):
+        bad.write_text(f"%%MatrixMarket matrix coordinate real {kind}\n2 100000 2\n1 99999 1.0\n2 100000 2.0\n")
+        with pytest.raises(ValueError, match="must be square"):
+            rio.read_matrix_market(bad, native=native)
+
+
+def test_a_size_line_beyond_memory_is_an_error_not_an_abort(tmp_path):
+    """A size line whose tables cannot be allocated comes back as ValueError: nothing is
+    thrown through the C boundary.  Run in a child process with its address space capped at
+    4 GiB, so that the 16 GB table of row starts fails at once instead of being allocated."""
+    import subprocess
+    import sys
+    bad = tmp_path / "huge.mtx"
+    bad.write_text("%%MatrixMarket matrix coordinate real general\n2000000000 2000000000 0\n")
+    code = (
+        "import resource, sys\n"
+        "sys.path.insert(0, %r)\n"
+        "from rode_amd import io as rio\n"
+        "rio._load_native()\n"
+        "resource.setrlimit(resource.RLIMIT_AS, (4 << 30, 4 << 30))\n"
+        "try:\n"
+        "    rio.read_matrix_market(%r, native=True)\n"
+        "except ValueError as e:\n"
+        "    print('ValueError:', e)\n"
+    ) % (str(__import__("pathlib").Path(__file__).resolve().parents[1]), str(bad))
+    done = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert "ValueError" in done.stdout and "memory" in done.stdout
+
+
 def test_rejects_bad_files(tmp_path):
     bad = tmp_path / "b.mtx"
     bad.write_text("%%MatrixMarket matrix array real general\n2 2\n1\n2\n3\n4\n")
