@@ -150,9 +150,8 @@ __device__ __forceinline__ float softmax_step(float sc, bool live, float& m_run,
 }
 
 // The groups of a group plan (rode_group.hip): one wave per group of four adjacent rows
-// whose runs of consecutive columns cover a range between them.  Along the range every k row
-// and every v row is loaded once for the four rows (a row's score is -inf, its probability
-// zero, at the columns outside its own run) (the score part is the SDDMM group kernel's, the output
+// whose runs of consecutive columns overlap in a long shared run (shared_run).  Along it every
+// k row and every v row is loaded once for the four rows (the score part is the SDDMM group kernel's, the output
 // part the SpMM group kernel's, with a running softmax per row in between); then the wave
 // takes the nonzeros outside the run, row by row, the way attention_rows_kernel does.
 // With WRITE_P the raw scores of the first kGroupScoresKept columns of the run wait in LDS,
@@ -175,8 +174,8 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     float* my_s = lds_s + (WRITE_P ? wave * R * kGroupScoresKept : 0);
     const int g = xcd_logical_block(blockIdx.x, gridDim.x) * kWavesPerWg + wave;
     if (g >= n_groups) return;
-    const RowGroup d = groups[g];
-    if (d.len <= 0) return; // not a group: attention_rows_kernel has its rows
+    if (groups[g].len <= 0) return; // not a group: attention_rows_kernel has its rows
+    const RowGroup d = shared_run(groups[g]); // the columns [lo, lo + len) that all four runs hold
     const int ls = lane % LPR, group = lane / LPR;
     const int row0 = g * R;
     // the scores of the run: LP lanes per k row, each with E of its 16-byte vectors (LP lanes apart), as in
@@ -184,15 +183,13 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
     constexpr int LP = LPR >= 8 ? LPR / 2 : LPR, E = LPR / LP;
     const int lp = lane % LP;
     typename DotVec<T>::Reg a[R][E][DotVec<T>::kRegs];
-    // per row: the slot of column j of the range is first[r] + j, for the columns j of the row's own run, from[r] <= j < to[r]
-    int first[R], from[R], to[R];
+    // per row: the slot of column j of the shared run is first[r] + j
+    int first[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
         for (int i = 0; i < E; ++i) DotVec<T>::load(q + (size_t)(row0 + r) * D + (lp + LP * i) * VEC, a[r][i]);
-        from[r] = d.head(r);
-        to[r] = d.len - d.tail(r);
-        first[r] = row_ptr[row0 + r] + d.pos[r] - from[r];
+        first[r] = row_ptr[row0 + r] + d.pos[r];
     }
     const T* k_lane = k + ls * VEC;
     const T* v_lane = v + ls * VEC;
@@ -243,7 +240,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const bool live = j >= from[r] && j < to[r];
+            const bool live = j < d.len;
             const float sc = live ? scale * (val[first[r] + j] * dot[r]) : -INFINITY;
             lds_p[wave][r][lane] = softmax_step<VEC>(sc, live, m_run[r], l_lane[r], acc[r]);
             if (WRITE_P && live) {
@@ -280,7 +277,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int s = row_ptr[row0 + r], e = row_ptr[row0 + r + 1];
-        const int split = d.pos[r], jump = to[r] - from[r], cnt = e - s - jump;
+        const int split = d.pos[r], jump = d.len, cnt = e - s - jump;
         typename DotVec<T>::Reg a_row[1][DotVec<T>::kRegs]; // this row of q as the lanes of sddmm_unit hold it
         load_lhs_slice<T, D, 1, false>(q, row0 + r, D, lane, a_row);
         for (int off = 0; off < cnt; off += kWave) {
@@ -321,14 +318,12 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
         if (WRITE_P) {
             // every lane normalises the scores it wrote itself: same walk over the run and over the rest
             const float m_safe = m_run[r] == -INFINITY ? 0.f : m_run[r];
-            for (int j = lane; j < to[r]; j += kWave) {
-                if (j >= from[r]) {
-                    const float sc = j < kGroupScoresKept ? my_s[r * kGroupScoresKept + j] : probs[first[r] + j];
-                    probs[first[r] + j] = __expf(sc - m_safe) * inv;
-                }
+            for (int j = lane; j < d.len; j += kWave) {
+                const float sc = j < kGroupScoresKept ? my_s[r * kGroupScoresKept + j] : probs[first[r] + j];
+                probs[first[r] + j] = __expf(sc - m_safe) * inv;
             }
             const int s = row_ptr[row0 + r], e = row_ptr[row0 + r + 1];
-            const int split = d.pos[r], jump = to[r] - from[r], cnt = e - s - jump;
+            const int split = d.pos[r], jump = d.len, cnt = e - s - jump;
             for (int slot = lane; slot < cnt; slot += kWave) {
                 const int idx = s + slot + (slot >= split ? jump : 0);
                 probs[idx] = __expf(probs[idx] - m_safe) * inv;

@@ -14,8 +14,7 @@ constexpr int kGroupRows = 4; // rows of one group of the group plan
 // A kept group: every row has a run of consecutive columns, and the runs cover [lo, lo + len)
 // between them - row r's own run is [lo + head(r), lo + len - tail(r)), with head and tail
 // below 256 (the runs of a sliding window start and end a column apart from row to row).
-// The group kernels walk the whole range for all rows; a row takes no part at the columns
-// outside its own run.
+// The group kernels walk the part of the range that all four runs hold (shared_run).
 struct RowGroup {
     int lo, len;          // the columns [lo, lo + len) that the runs of the group's rows cover; len 0: no group
     int pos[kGroupRows];  // where its own run starts in each row (slots from the row's first nonzero)
@@ -26,6 +25,24 @@ struct RowGroup {
     __host__ __device__ int run(int r) const { return len - head(r) - tail(r); } // length of row r's own run
 };
 static_assert(sizeof(RowGroup) == 32, "the group plan holds 32 bytes per group");
+// What the group kernels walk for all four rows at once: the columns that every row's own
+// run holds, [lo + largest head, lo + len - largest tail).  A row's columns of the range
+// before and after that part are left to the pass over its other nonzeros, so no row ever
+// meets a dense row that it does not reference (a non-finite one would turn a zero value
+// into NaN).  The plan keeps a group only if this part has at least 64 columns.
+__host__ __device__ inline RowGroup shared_run(RowGroup d)
+{
+    int head = 0, tail = 0;
+    for (int r = 0; r < kGroupRows; ++r) {
+        head = d.head(r) > head ? d.head(r) : head;
+        tail = d.tail(r) > tail ? d.tail(r) : tail;
+    }
+    for (int r = 0; r < kGroupRows; ++r) d.pos[r] += head - d.head(r);
+    d.lo += head;
+    d.len -= head + tail;
+    d.heads = d.tails = 0u;
+    return d;
+}
 struct RowOwners {
     int hub_min_len = 0;              // > 0: rows of that aligned length or more belong to the hub kernels
     const RowGroup* groups = nullptr; // the groups of a group plan, or null

@@ -262,12 +262,11 @@ __device__ __forceinline__ void sddmm_group_leftovers(const RowGroup& d, int row
     }
 }
 
-// The groups of a group plan (rode_group.hip): four adjacent rows whose runs of consecutive
-// columns cover the range [lo, lo + len) between them.  One wave per group (WPG = 1), or a
-// workgroup whose four waves split the range.  Every rhs row of the range is loaded once
-// (its address follows from the range, no column index is read) and multiplied with the lhs
-// rows of all four rows of the group, which stay in registers; a row gets no output at the
-// columns outside its own run.  Then the rows' nonzeros outside their runs: with one wave per
+// The groups of a group plan (rode_group.hip): four adjacent rows with runs of consecutive
+// columns that overlap in a long shared run (shared_run).  One wave per group (WPG = 1), or a
+// workgroup whose four waves split the shared run.  Every rhs row of it is loaded once
+// (its address follows from the run, no column index is read) and multiplied with the lhs
+// rows of all four rows of the group, which stay in registers.  Then the rows' other nonzeros: with one wave per
 // group, of the four rows together (sddmm_group_leftovers); with a workgroup, wave w takes
 // row w's.  Single-slab rows only (k <= 128 elements per lane tile): four lhs slices of more
 // slabs would not fit.
@@ -289,18 +288,14 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
     const int g = xcd_logical_block(blockIdx.x, gridDim.x) * (kWavesPerWg / WPG) + wave / WPG;
     if (g >= n_groups) return;
-    const RowGroup d = groups[g];
-    if (d.len <= 0) return; // not a group: its rows are in the lists
+    if (groups[g].len <= 0) return; // not a group: its rows are in the lists
+    const RowGroup d = shared_run(groups[g]); // the columns [lo, lo + len) that all four runs hold
     const int w = wave % WPG; // this wave among the waves of its group
     const int row0 = g * R;
-    // per row: the slot of column j of the range is at[r] + j, for the columns j of the row's own run, from[r] <= j < to[r]
-    int at[R], from[R], to[R];
+    // per row: the slot of column j of the shared run is at[r] + j
+    int at[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        from[r] = d.head(r);
-        to[r] = d.len - d.tail(r);
-        at[r] = row_ptr[row0 + r] + d.pos[r] - from[r];
-    }
+    for (int r = 0; r < R; ++r) at[r] = row_ptr[row0 + r] + d.pos[r];
     // this wave's share of the run, in quads of columns; lane e of a step has column j0 + e
     const int quads = (d.len + 3) / 4;
     const int q_begin = quads * w / WPG, q_end = quads * (w + 1) / WPG;
@@ -363,7 +358,7 @@ sddmm_group_kernel(int k, int n_groups, const RowGroup* __restrict__ groups, con
             const int j = j0 + lane;
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                if (j >= from[r] && j < min(to[r], j_end)) out[at[r] + j] = val[at[r] + j] * result[r];
+                if (j < j_end) out[at[r] + j] = val[at[r] + j] * result[r];
         }
     }
     if constexpr (WPG == 1) {

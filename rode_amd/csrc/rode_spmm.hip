@@ -311,12 +311,11 @@ spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, RowOwners owner
                                        B, C, plan);
 }
 
-// The groups of a group plan (rode_group.hip): four adjacent rows whose runs of consecutive
-// columns cover the range [lo, lo + len) between them.  One wave per group (WPG = 1), or a
-// workgroup whose four waves split the range.  Every dense row of the range is loaded once
-// and multiplied into the sums of all four rows (its address follows from the range, no
-// column index is read; a row's value is zero at the columns outside its own run).  Then the
-// rows' nonzeros outside their runs: with one wave per group, of the four rows together;
+// The groups of a group plan (rode_group.hip): four adjacent rows with runs of consecutive
+// columns that overlap in a long shared run (shared_run).  One wave per group (WPG = 1), or a
+// workgroup whose four waves split the shared run.  Every dense row of it is loaded once
+// and multiplied into the sums of all four rows (its address follows from the run, no
+// column index is read).  Then the rows' other nonzeros: with one wave per group, of the four rows together;
 // with a workgroup, wave w adds row w's, the waves' sums meet in LDS, and wave w adds the
 // total of row w to C.  A row is in no other work item: no atomics.
 template <typename T, int TN, bool EDGE, int WPG>
@@ -338,22 +337,18 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
     const int g = xcd_logical_block(blockIdx.x, gridDim.x) * GPW + wave / WPG;
     if (g >= n_groups) return;
-    const RowGroup d = groups[g];
-    if (d.len <= 0) return; // not a group: its rows are in the lists
+    if (groups[g].len <= 0) return; // not a group: its rows are in the lists
+    const RowGroup d = shared_run(groups[g]); // the columns [lo, lo + len) that all four runs hold
     const int w = wave % WPG; // this wave among the waves of its group
     const int ls = lane % LPR, group = lane / LPR;
     const int tile = blockIdx.y * TN;
     const bool col_ok = !EDGE || tile + ls * VEC < n;
     const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
     const int row0 = g * R;
-    // per row: the slot of column j of the range is at[r] + j, for the columns j of the row's own run, from[r] <= j < to[r]
-    int at[R], from[R], to[R];
+    // per row: the slot of column j of the shared run is at[r] + j
+    int at[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        from[r] = d.head(r);
-        to[r] = d.len - d.tail(r);
-        at[r] = row_ptr[row0 + r] + d.pos[r] - from[r];
-    }
+    for (int r = 0; r < R; ++r) at[r] = row_ptr[row0 + r] + d.pos[r];
 
     // this wave's share of the run, in quads of columns
     const int quads = (d.len + 3) / 4;
@@ -373,7 +368,7 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int j = 4 * q_begin + lane;
-        v_next[r] = j >= from[r] && j < min(to[r], j_end) ? val[at[r] + j] : A(0);
+        v_next[r] = j < j_end ? val[at[r] + j] : A(0);
     }
     for (int j0 = 4 * q_begin; j0 < j_end; j0 += kWave) {
 #pragma unroll
@@ -382,7 +377,7 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
         {
             const int j = j0 + kWave + lane;
 #pragma unroll
-            for (int r = 0; r < R; ++r) v_next[r] = j >= from[r] && j < min(to[r], j_end) ? val[at[r] + j] : A(0);
+            for (int r = 0; r < R; ++r) v_next[r] = j < j_end ? val[at[r] + j] : A(0);
         }
         const int nq = min(kWave / 4, (j_end - j0 + 3) / 4);
 #pragma unroll
@@ -390,7 +385,8 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
             const int q = group + i * G;
             if (q < nq) {
                 // four consecutive rows of B (the last quad of a run may be cut short: its rows
-                // past the run repeat the run's last row, their values are zero)
+                // past the run repeat the run's last row, which every row of the group
+                // references; their values are zero)
                 const char* b_quad = reinterpret_cast<const char*>(b_run + (size_t)(j0 + 4 * i * G) * n);
                 const int room = d.len - 1 - (j0 + 4 * q);
                 const unsigned o1 = room >= 1 ? row_bytes : 0u;
@@ -420,10 +416,10 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
         int row_first[R], split[R], jump[R], cnt[R], max_cnt = 0;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            row_first[r] = at[r] + from[r] - d.pos[r];
+            row_first[r] = at[r] - d.pos[r];
             split[r] = d.pos[r];
-            jump[r] = to[r] - from[r];
-            cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (at[r] + to[r])); // the slots before the run + those after it
+            jump[r] = d.len;
+            cnt[r] = split[r] + (row_ptr[row0 + r + 1] - (at[r] + d.len)); // the slots before the run + those after it
             max_cnt = max(max_cnt, cnt[r]);
         }
         for (int off = 0; off < max_cnt; off += kWave) {

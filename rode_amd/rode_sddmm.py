@@ -91,7 +91,10 @@ class RoDeCSR:
             if int(((blocked + 511) // 512).sum()) < 16384:
                 seg = 128
             else:
-                p90 = int(torch.quantile(blocked.to(torch.float64), 0.9, interpolation="higher"))
+                # the smallest length that at least 90 % of those rows do not exceed (the order
+                # statistic torch.quantile(..., "higher") returns, without its 16 M element limit)
+                rank = min(blocked.numel(), int(torch.ceil(torch.tensor(0.9 * (blocked.numel() - 1), dtype=torch.float64))) + 1)
+                p90 = int(torch.kthvalue(blocked, rank).values)
                 while seg < p90 and seg < 2048:
                     seg *= 2
         return {"seg_length": seg, "k_block": 32, "vec_len": 4}

@@ -289,3 +289,49 @@ def test_fused_attention_of_groups(d, half, m, window):
     out2, probs2 = _attention_call(plain, plain.values, q, k, v, scale, True)
     assert (out - out2).abs().max().item() <= tol * max(1.0, out2.abs().max().item())
     assert (probs - probs2).abs().max().item() <= tol
+
+
+def _shifted_windows(m, shift, width, extra, seed):
+    """Row r has the run [shift * r, shift * r + width) plus `extra` random columns: inside a
+    group of four rows the runs start `shift` columns apart, so every group's range has
+    columns that only some of its rows own."""
+    rng = np.random.default_rng(seed)
+    n = shift * m + width + 64
+    rows = [np.union1d(np.arange(shift * r, shift * r + width), rng.choice(n, extra, replace=False)).astype(np.int32)
+            for r in range(m)]
+    rp = np.zeros(m + 1, dtype=np.int32)
+    rp[1:] = np.cumsum([len(c) for c in rows])
+    return n, rp, np.concatenate(rows), rng.uniform(0.5, 1.5, rp[-1]).astype(np.float32)
+
+
+@pytest.mark.parametrize("m", [400, 8400], ids=["workgroup_per_group", "wave_per_group"])
+def test_non_finite_dense_rows_stay_in_the_rows_that_reference_them(m):
+    """The group kernels load every dense row of a group's range for all four rows.  A row
+    whose own run does not hold a column must not see that column's dense row: Inf there may
+    only reach the rows that reference it (as in the list kernels and the reference)."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import rode_sddmm_hip, rode_spmm, sparse_attention
+    shift, width, d = 3, 200, 64
+    n, rp, col, val = _shifted_windows(m, shift, width, 4, seed=m)
+    csr = make_csr(rp, col, val, m, n, d)
+    assert isinstance(csr.plan, rode_sddmm_hip.GroupPlan) and csr.plan.counts[1] == m // 4
+    assert (csr.plan.counts[1] >= 2048) == (m == 8400)
+    # columns at the head of a range (owned by the group's first row only) and at its tail
+    # (owned by its last row only), in every 50th group (a column is in the runs of 67 rows)
+    groups = np.arange(0, m // 4, 50)
+    bad = np.concatenate([4 * shift * groups + 1, 4 * shift * groups + 3 * shift + width - 1])
+    touched = np.zeros(m, dtype=bool)
+    touched[np.repeat(np.arange(m), np.diff(rp))[np.isin(col, bad)]] = True
+    assert touched[4 * groups].all() and touched[4 * groups + 3].all()
+    # the rows this test is about: inside such a group, not referencing the column (but for a stray random one)
+    assert (~touched[4 * groups + 1]).sum() + (~touched[4 * groups + 2]).sum() >= len(groups)
+    g = torch.Generator(device=DEV).manual_seed(1)
+    B = torch.randn(n, d, device=DEV, generator=g)
+    B[torch.from_numpy(bad).to(DEV)] = float("inf")
+    C = rode_spmm(csr, B).cpu().numpy()
+    assert np.isfinite(C[~touched]).all(), "a non-finite dense row reached rows that do not reference it"
+    assert (~np.isfinite(C[touched])).any(axis=1).all()
+    q, k = torch.randn(m, d, device=DEV, generator=g), torch.randn(n, d, device=DEV, generator=g)
+    out = sparse_attention(csr, q, k, B, fused=True).cpu().numpy()
+    assert np.isfinite(out[~touched]).all(), "a non-finite row of v reached rows that do not attend to it"
+    assert (~np.isfinite(out[touched])).any(axis=1).all()

@@ -115,3 +115,18 @@ def test_auto_config_picks_the_segment_length_from_the_row_lengths():
     rp[1:] = np.cumsum(np.full(40000, 1500))
     assert RoDeCSR.auto_config(torch.from_numpy(rp))["seg_length"] == 2048
     assert RoDeCSR.auto_config(torch.zeros(5, dtype=torch.int32))["seg_length"] == 512
+
+
+def test_auto_config_with_more_rows_than_a_library_quantile_takes():
+    """17 M rows with block segments (torch.quantile refuses more than 16 M elements): the
+    90th percentile is taken as an order statistic, whatever the count."""
+    m = 17_000_000
+    lens = torch.full((m,), 40, dtype=torch.int64)
+    lens[: m // 5] = 1500  # 20 % long rows: the 90th percentile is 1500 -> 2048
+    rp = torch.zeros(m + 1, dtype=torch.int64)
+    rp[1:] = torch.cumsum(lens, 0)
+    assert RoDeCSR.auto_config(rp)["seg_length"] == 2048
+    lens[: m // 5] = 40
+    lens[: m // 20] = 1500  # 5 % long rows: the 90th percentile is 40 (+ 0..3 of alignment) -> 512
+    rp[1:] = torch.cumsum(lens, 0)
+    assert RoDeCSR.auto_config(rp)["seg_length"] == 512
