@@ -69,6 +69,9 @@ def parse_args():
                         "\"probs\" also writes the probabilities a gradient needs")
     p.add_argument("--chain", action="store_true",
                    help="step = SDDMM scores -> row softmax -> clear C -> SpMM with those values (sparse attention)")
+    p.add_argument("--train", action="store_true",
+                   help="with --chain --fused probs: the step is the attention forward with its probabilities written "
+                        "plus the two gradient kernels (rode_hip_attention_backward_rows / _cols)")
     p.add_argument("--memset-c", action="store_true",
                    help="clear all of C before SpMM (the reference's contract) instead of only the rows SpMM adds to")
     p.add_argument("--no-plan", action="store_true",
@@ -213,6 +216,32 @@ def main():
         join()
 
     probs = torch.empty(nnz, device=dev) if args.chain else None
+    if args.chain:
+        args.no_cpu = True  # (the CPU leg and its parity gate are those of SpMM + SDDMM; the chain is checked by the tests)
+    if args.train:
+        if not (args.chain and args.fused == "probs"):
+            print("bench.py: --train needs --chain --fused probs", file=sys.stderr)
+            sys.exit(2)
+        csr_t, _ = csr.transpose(with_values=False)
+        t_slot = csr.transposed_slots()
+        grp_t = csr_t.plan if isinstance(csr_t.plan, rode_sddmm_hip.GroupPlan) else None
+        plans_t = ctypes.byref(rode_sddmm_hip.plans_struct(grp_t))
+        G = torch.randn(m, k, device=dev, generator=gen)  # gradient of the loss with respect to the output
+        dQ, dK, dV = (torch.empty(r, k, device=dev) for r in (m, n, n))
+        pairs = torch.empty(2 * nnz, device=dev)
+
+    def backward_rows():
+        _lib.check(lib.rode_hip_attention_backward_rows(
+            _lib.DENSE_CODE[args.dtype], m, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
+            csr.values.data_ptr(), probs.data_ptr(), G.data_ptr(), C.data_ptr(), B.data_ptr(), B.data_ptr(),
+            float(k) ** -0.5, t_slot.data_ptr(), dQ.data_ptr(), pairs.data_ptr(), sddmm_plans, stream),
+            "attention backward, rows")
+
+    def backward_cols():
+        _lib.check(lib.rode_hip_attention_backward_cols(
+            _lib.DENSE_CODE[args.dtype], n, k, csr_t.row_offsets.data_ptr(), csr_t.column_indices.data_ptr(),
+            pairs.data_ptr(), G.data_ptr(), L.data_ptr(), dK.data_ptr(), dV.data_ptr(), plans_t, stream),
+            "attention backward, columns")
 
     def clear_c():
         if args.memset_c:
@@ -231,6 +260,9 @@ def main():
                 _lib.DENSE_CODE[args.dtype], m, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
                 csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), B.data_ptr(), float(k) ** -0.5, C.data_ptr(),
                 probs.data_ptr() if args.fused == "probs" else None, sddmm_plans, stream), "attention")
+            if args.train:
+                backward_rows()
+                backward_cols()
             return
         if args.chain:
             sddmm(csr.m1, csr.m2)
@@ -266,7 +298,7 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
-    flops_per_step = 2 * (2.0 * nnz * k)
+    flops_per_step = (6 if args.train else 2) * (2.0 * nnz * k)  # (a gradient: four more products)
     gflops = flops_per_step / (ms_per_step * 1e-3) / 1e9
 
     # ---- per-kernel durations, HIP events on the launch stream ----------------
@@ -312,6 +344,9 @@ def main():
     if grp is not None:  # the rows of the group plan's groups (the same flag selects them)
         kernels["spmm_group"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_HUB), reps)
         kernels["sddmm_group"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_HUB), reps)
+    if args.train:
+        kernels["attention_backward_rows"] = event_time(backward_rows, reps)
+        kernels["attention_backward_cols"] = event_time(backward_cols, reps)
     spmm_ms = event_time(lambda: (clear_c(), spmm(csr.m1, csr.m2)), reps)
     sddmm_ms = event_time(lambda: sddmm(csr.m1, csr.m2), reps)
     spmm_contract_ms = float("nan") if args.no_contract else event_time(spmm_reference_contract, reps)
@@ -333,6 +368,15 @@ def main():
     split_spmm = work_split(row_ptr, col, n, 1024 if csr.m1 >= 16384 else 0, hub_min_len, group_rows)
     per_kernel = {}
     for name, ms in kernels.items():
+        if name.startswith("attention"):
+            # row pass: (col, val, p, slot in the transposed pattern) read, (p, dz) written, rows of g, out,
+            # dq, every k and v row once; column pass: row and (p, dz) read, rows of dk, dv, every g and q row once
+            ab = nnz * (16 + 8) + 3 * m * k * 4 + 2 * n * k * elem if name.endswith("rows") else \
+                nnz * (4 + 8) + 2 * n * k * 4 + m * k * (4 + elem)
+            per_kernel[name] = {"ms": round(ms, 4), "algorithmic_bytes": ab, "algorithmic_GBs": round(ab / ms / 1e6, 1),
+                                "gather_model_GBs": round(nnz * (16 + 2 * k * elem) / ms / 1e6, 1),
+                                "GFLOPs": round(2 * 2.0 * nnz * k / ms / 1e6, 1)}
+            continue
         split = split_spmm if name.startswith("spmm") else split_sddmm
         m2_eff = csr.m2
         if name == "spmm_residue":
@@ -480,6 +524,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.workload} ({workloads.CONFIGS[args.workload][5]}), K={k}, "
                                + (("step = fused attention forward (one kernel" + (", probabilities written)" if args.fused == "probs" else ")")
+                                   + (" + gradient (row pass + column pass)" if args.train else "")
                                    if args.fused != "no" else "step = SDDMM -> row softmax -> clear C -> SpMM (chained)")
                                   if args.chain
                                   else "step = clear C rows + SpMM + SDDMM"),

@@ -372,6 +372,39 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
                                float scale, float* d_out, float* d_probs, const rode_hip_plans* plans, void* stream);
 
 /*
+ * The gradient of rode_hip_attention_forward in two kernels (no counterpart in the
+ * reference, whose op is forward-only, RoDe_SDDMM/rode_sddmm.py:194-248).  With g the
+ * gradient of the loss with respect to out:
+ *   rode_hip_attention_backward_rows  walks the pattern: per nonzero dp = <g[r, :], v[col, :]>
+ *       and dz = scale * values * p * (dp - <g[r, :], out[r, :]>), the gradient with respect
+ *       to <q[r, :], k[col, :]>; writes grad_q[r, :] = sum dz * k[col, :] and, to the nonzero's
+ *       slot in the transposed pattern, the pair (p, dz);
+ *   rode_hip_attention_backward_cols  walks the transposed pattern (rode_hip_csr_transpose):
+ *       grad_k[c, :] = sum dz * q[row, :] and grad_v[c, :] = sum p * g[row, :] over the
+ *       nonzeros of column c, with the pairs the first call left in its order.
+ *   dtype        RODE_DENSE_F32 or RODE_DENSE_F16: element type of q, k and v (g, out and the
+ *                three gradients are float; with fp16 operands g is rounded to fp16 relative to
+ *                the largest magnitude of its row where it meets rows of v)
+ *   M, N         rows / columns of the pattern; d: 32, 64 or 128
+ *   d_probs      float [nnz]: p as rode_hip_attention_forward wrote it
+ *   d_out        float [M x d]: the forward result
+ *   d_t_slot     int [nnz]: for every nonzero its index in the transposed pattern, i.e. the
+ *                inverse of the d_perm that rode_hip_csr_transpose returns
+ *   d_pairs      float [2 * nnz], 16-byte aligned: written by the first call, read by the second
+ *   plans / t_plans   NULL, or the plans of the pattern / of the transposed pattern (a group
+ *                plan with at least 2048 groups with a run is used, as in the forward call)
+ * Rows (columns) without nonzeros get zero gradients.  Both calls queue on `stream`.
+ */
+int rode_hip_attention_backward_rows(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
+                                     const float* d_values, const float* d_probs, const float* d_grad_out,
+                                     const float* d_out, const void* d_k, const void* d_v, float scale,
+                                     const int* d_t_slot, float* d_grad_q, float* d_pairs, const rode_hip_plans* plans,
+                                     void* stream);
+int rode_hip_attention_backward_cols(int dtype, int N, int d, const int* d_t_row_offsets, const int* d_t_column_indices,
+                                     const float* d_pairs, const float* d_grad_out, const void* d_q, float* d_grad_k,
+                                     float* d_grad_v, const rode_hip_plans* t_plans, void* stream);
+
+/*
  * The transposed pattern of a CSR matrix (M rows, N columns, nnz nonzeros): what the
  * gradients with respect to the column-side operands (SDDMM's rhs, SpMM's B) run on.  No
  * counterpart in the reference (forward-only, RoDe_SDDMM/rode_sddmm.py:194-248).

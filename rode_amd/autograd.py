@@ -143,41 +143,87 @@ def _attention_call(csr, values, q, k, v, scale, want_probs):
     return out, probs
 
 
+def _attention_backward_call(csr, csr_t, t_slot, probs, g, out, q, k, v, scale):
+    """(dq, dk, dv) in float32 through the two gradient kernels: the row pass over the
+    pattern, the column pass over the transposed pattern."""
+    lib = _lib.load()
+    m, d = q.shape
+    n = k.shape[0]
+    kind = _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"]
+    dq = torch.empty((m, d), dtype=torch.float32, device=q.device)
+    dk = torch.empty((n, d), dtype=torch.float32, device=q.device)
+    dv = torch.empty((n, d), dtype=torch.float32, device=q.device)
+    pairs = torch.empty(2 * probs.numel(), dtype=torch.float32, device=q.device)
+    group = lambda c: c.plan if isinstance(c.plan, rode_sddmm_hip.GroupPlan) else None
+    plans, plans_t = rode_sddmm_hip.plans_struct(group(csr)), rode_sddmm_hip.plans_struct(group(csr_t))
+    with torch.cuda.device(q.device):
+        s = torch.cuda.current_stream(q.device).cuda_stream
+        _lib.check(lib.rode_hip_attention_backward_rows(
+            kind, m, d, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
+            probs.data_ptr(), g.data_ptr(), out.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale), t_slot.data_ptr(),
+            dq.data_ptr(), pairs.data_ptr(), ctypes.byref(plans), s), "rode_hip_attention_backward_rows")
+        _lib.check(lib.rode_hip_attention_backward_cols(
+            kind, n, d, csr_t.row_offsets.data_ptr(), csr_t.column_indices.data_ptr(), pairs.data_ptr(), g.data_ptr(), q.data_ptr(), dk.data_ptr(), dv.data_ptr(), ctypes.byref(plans_t), s),
+            "rode_hip_attention_backward_cols")
+    return dq, dk, dv
+
+
+# True / False / "auto": whether the gradient of the fused attention runs as the two gradient
+# kernels or as the chain of separate kernels.  "auto": the two kernels unless a column of the
+# pattern has more than FUSED_MAX_ROW nonzeros (one wavefront per column, as per row in the
+# forward pass).
+FUSED_BACKWARD = "auto"
+
+
 class FusedAttentionFunction(torch.autograd.Function):
-    """Forward: one kernel (``rode_hip_attention_forward``).  Backward: the kernels of the
-    chain on the saved probabilities - dP = (dOut v^T)|pattern (SDDMM), the softmax
-    gradient, dq and dk as SpMM on the pattern and its transpose, dv = P^T dOut."""
+    """Forward: one kernel (``rode_hip_attention_forward``).  Backward: two kernels on the
+    saved probabilities and output (``rode_hip_attention_backward_rows`` / ``_cols``), or the
+    kernels of the chain - dP = (dOut v^T)|pattern (SDDMM), the softmax gradient, dq and dk as
+    SpMM on the pattern and its transpose, dv = P^T dOut."""
 
     @staticmethod
     def forward(ctx, csr, q, k, v, scale):
         need = any(ctx.needs_input_grad[1:4])
         values = csr.values
-        out, probs = _attention_call(csr, values, q.detach().contiguous(), k.detach().contiguous(),
-                                     v.detach().contiguous(), scale, need)
+        q, k, v = q.detach().contiguous(), k.detach().contiguous(), v.detach().contiguous()
+        out, probs = _attention_call(csr, values, q, k, v, scale, need)
         ctx.csr, ctx.scale = csr, float(scale)
         if need:
-            ctx.save_for_backward(probs, q, k, v)
+            ctx.save_for_backward(probs, q, k, v, out)
         return out
 
     @staticmethod
     def backward(ctx, g):
         csr, scale = ctx.csr, ctx.scale
-        probs, q, k, v = ctx.saved_tensors
+        probs, q, k, v, out = ctx.saved_tensors
         g = g.contiguous().float()
         dq = dk = dv = None
+        if probs.numel() == 0:  # no nonzeros: the output does not depend on anything
+            zeros = lambda t, need: torch.zeros_like(t) if need else None
+            return (None, zeros(q, ctx.needs_input_grad[1]), zeros(k, ctx.needs_input_grad[2]),
+                    zeros(v, ctx.needs_input_grad[3]), None)
         csr_t = perm = None
-        if ctx.needs_input_grad[2] or ctx.needs_input_grad[3]:
+        fused = FUSED_BACKWARD
+        if fused or ctx.needs_input_grad[2] or ctx.needs_input_grad[3]:
             csr_t, perm = csr.transpose(with_values=False)
+        if fused == "auto":
+            fused = csr_t.max_row_length <= FUSED_MAX_ROW
+        if fused:
+            dq, dk, dv = _attention_backward_call(csr, csr_t, csr.transposed_slots(), probs, g, out, q, k, v, scale)
+            return (None, dq.to(q.dtype) if ctx.needs_input_grad[1] else None,
+                    dk.to(k.dtype) if ctx.needs_input_grad[2] else None,
+                    dv.to(v.dtype) if ctx.needs_input_grad[3] else None, None)
         if ctx.needs_input_grad[3]:
             dv = _spmm(csr_t, rode_sddmm_hip.permute(probs, perm), g).to(v.dtype)
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            dp = _sddmm(csr, csr.ones(), g, v.float())
+            dp = _sddmm(csr, csr.ones(), g, v.float())  # (g is float32: both operands of an SDDMM share a type)
             ds = _softmax_call("rode_hip_csr_softmax_backward_f32", csr.row_offsets, probs, dp, scale)
             ds.mul_(csr.values)  # scores are values (.) (q k^T)
+            # float16 operands are gathered as they are (the sums are float32 either way)
             if ctx.needs_input_grad[1]:
-                dq = _spmm(csr, ds, k.float()).to(q.dtype)
+                dq = _spmm(csr, ds, k).to(q.dtype)
             if ctx.needs_input_grad[2]:
-                dk = _spmm(csr_t, rode_sddmm_hip.permute(ds, perm), q.float()).to(k.dtype)
+                dk = _spmm(csr_t, rode_sddmm_hip.permute(ds, perm), q).to(k.dtype)
         return None, dq, dk, dv, None
 
 

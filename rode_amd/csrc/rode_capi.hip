@@ -378,6 +378,68 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
     return hipErrorInvalidValue;
 }
 
+// (only a group plan means anything to the attention kernels)
+static bool group_plan_only(const rode_hip_plans* plans, int rows, rode::PlanRef& plan)
+{
+    if (!plans || !plans->groups) return true;
+    rode_hip_plans only_groups = {};
+    only_groups.groups = plans->groups;
+    only_groups.group_counts = plans->group_counts;
+    return plan_ref(&only_groups, 0, plan) && plan.group_counts[0] == rode::row_groups(rows);
+}
+
+int rode_hip_attention_backward_rows(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
+                                     const float* d_values, const float* d_probs, const float* d_grad_out,
+                                     const float* d_out, const void* d_k, const void* d_v, float scale,
+                                     const int* d_t_slot, float* d_grad_q, float* d_pairs, const rode_hip_plans* plans,
+                                     void* stream)
+{
+    if (M < 0 || !d_row_offsets) return hipErrorInvalidValue;
+    rode::PlanRef plan;
+    if (!group_plan_only(plans, M, plan)) return hipErrorInvalidValue;
+    if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
+    if (M > 0 && (!d_column_indices || !d_values || !d_probs || !d_grad_out || !d_out || !d_k || !d_v || !d_t_slot || !d_grad_q ||
+                  !d_pairs))
+        return hipErrorInvalidValue;
+    if (!aligned16(d_grad_out) || !aligned16(d_out) || !aligned16(d_k) || !aligned16(d_v) || !aligned16(d_grad_q) ||
+        !aligned16(d_pairs))
+        return hipErrorInvalidValue;
+    if (dtype == RODE_DENSE_F32)
+        return rode::attention_backward_rows_launch<float>(M, d, d_row_offsets, d_column_indices, d_values, d_probs,
+                                                           d_grad_out, d_out, static_cast<const float*>(d_k),
+                                                           static_cast<const float*>(d_v), scale, d_t_slot, d_grad_q, d_pairs,
+                                                           plan, as_stream(stream));
+    if (dtype == RODE_DENSE_F16)
+        return rode::attention_backward_rows_launch<__half>(M, d, d_row_offsets, d_column_indices, d_values, d_probs,
+                                                            d_grad_out, d_out, static_cast<const __half*>(d_k),
+                                                            static_cast<const __half*>(d_v), scale, d_t_slot, d_grad_q, d_pairs,
+                                                            plan, as_stream(stream));
+    return hipErrorInvalidValue;
+}
+
+int rode_hip_attention_backward_cols(int dtype, int N, int d, const int* d_t_row_offsets, const int* d_t_column_indices,
+                                     const float* d_pairs, const float* d_grad_out, const void* d_q, float* d_grad_k,
+                                     float* d_grad_v, const rode_hip_plans* t_plans, void* stream)
+{
+    if (N < 0 || !d_t_row_offsets) return hipErrorInvalidValue;
+    rode::PlanRef plan;
+    if (!group_plan_only(t_plans, N, plan)) return hipErrorInvalidValue;
+    if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
+    if (N > 0 && (!d_t_column_indices || !d_pairs || !d_grad_out || !d_q || !d_grad_k || !d_grad_v))
+        return hipErrorInvalidValue;
+    if (!aligned16(d_grad_out) || !aligned16(d_q) || !aligned16(d_grad_k) || !aligned16(d_grad_v) || !aligned16(d_pairs))
+        return hipErrorInvalidValue;
+    if (dtype == RODE_DENSE_F32)
+        return rode::attention_backward_cols_launch<float>(N, d, d_t_row_offsets, d_t_column_indices, d_pairs,
+                                                           d_grad_out, static_cast<const float*>(d_q), d_grad_k, d_grad_v,
+                                                           plan, as_stream(stream));
+    if (dtype == RODE_DENSE_F16)
+        return rode::attention_backward_cols_launch<__half>(N, d, d_t_row_offsets, d_t_column_indices, d_pairs,
+                                                            d_grad_out, static_cast<const __half*>(d_q), d_grad_k, d_grad_v,
+                                                            plan, as_stream(stream));
+    return hipErrorInvalidValue;
+}
+
 size_t rode_hip_csr_transpose_workspace_bytes(int nnz) { return rode::csr_transpose_workspace_bytes(nnz); }
 
 int rode_hip_permute_f32(int n, const float* d_src, const int* d_index, float* d_dst, void* stream)

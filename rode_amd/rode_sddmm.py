@@ -191,6 +191,17 @@ class RoDeCSR:
             return csr_t, perm
         return csr_t.with_values(self._permuted_values(perm)), perm
 
+    def transposed_slots(self):
+        """int32 vector over the nonzeros: the index of each in the transposed pattern (the
+        inverse of the ``perm`` of ``transpose``; made once per pattern)."""
+        cached = self._shared.get("transposed_slots")
+        if cached is None:
+            _, perm = self.transpose(with_values=False)
+            cached = torch.empty_like(perm)
+            cached[perm.long()] = torch.arange(perm.numel(), dtype=torch.int32, device=perm.device)
+            self._shared["transposed_slots"] = cached
+        return cached
+
     def ones(self):
         """A float32 vector of ones over the nonzeros (made once per pattern): the values of an
         SDDMM that samples without weighting."""

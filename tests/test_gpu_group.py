@@ -335,3 +335,60 @@ def test_non_finite_dense_rows_stay_in_the_rows_that_reference_them(m):
     out = sparse_attention(csr, q, k, B, fused=True).cpu().numpy()
     assert np.isfinite(out[~touched]).all(), "a non-finite row of v reached rows that do not attend to it"
     assert (~np.isfinite(out[touched])).any(axis=1).all()
+
+
+@pytest.mark.parametrize("d,half", [(64, False), (64, True), (128, False), (32, True)])
+def test_fused_attention_gradients_of_groups(d, half):
+    """The two gradient kernels with group plans of at least 2048 kept groups on the pattern
+    (row pass: attention_backward_group_kernel) and on its transpose (column pass:
+    attention_backward_cols_group_kernel), rows and columns outside kept groups included,
+    against dense fp64 autograd and against the chain of separate kernels."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import autograd, rode_sddmm_hip, sparse_attention
+    from test_gpu_attention import _dense
+    rng = np.random.default_rng(70 + d)
+    m, window = 12002, 96
+    n = m + 498
+    rp, col, _ = _window_matrix(rng, m, n, window, 6, ragged=False)
+    # a few irregular rows, far enough apart that most runs of rows survive in the transposed
+    # pattern too: a hole in the window, an empty row, a short row without a run
+    rows = [col[rp[r]:rp[r + 1]] for r in range(m)]
+    for r in range(5, m, 997):
+        rows[r] = np.concatenate([rows[r][:20], rows[r][23:]])
+    for r in range(7, m, 1001):
+        rows[r] = rows[r][:0]
+    for r in range(9, m, 1499):
+        rows[r] = np.sort(rng.choice(n, 5, replace=False)).astype(np.int32)
+    rp = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(0.5, 1.5, len(col)).astype(np.float32)
+    mask = make_csr(rp, col, val, m, n, d, locality=True)
+    mask_t, _ = mask.transpose(with_values=False)
+    for c in (mask, mask_t):
+        assert isinstance(c.plan, rode_sddmm_hip.GroupPlan) and c.plan.counts[1] >= 2048 and c.plan.counts[2] > 0
+    dt = torch.float16 if half else torch.float32
+    mk = lambda r, s: torch.from_numpy((s * rng.standard_normal((r, d))).astype(np.float32)).to(DEV, dt)
+    q, k, v = mk(m, 1.2).requires_grad_(), mk(n, 1.2).requires_grad_(), mk(n, 1.0).requires_grad_()
+    w = mk(m, 1.0).float() * 1e-3  # small gradients: fp16 operands must not lose them
+    scale = 0.4
+    grads = {}
+    for fused_backward in (True, False):
+        autograd.FUSED_BACKWARD = fused_backward
+        try:
+            q.grad = k.grad = v.grad = None
+            out = sparse_attention(mask, q, k, v, scale=scale, fused=True)
+            (out * w).sum().backward()
+        finally:
+            autograd.FUSED_BACKWARD = "auto"
+        grads[fused_backward] = (q.grad.clone(), k.grad.clone(), v.grad.clone())
+    q64, k64, v64 = (t.detach().double().requires_grad_() for t in (q, k, v))
+    A = _dense(rp, col, val, m, n)
+    has = torch.from_numpy(np.diff(rp) > 0).to(DEV)
+    scores = (q64 @ k64.t()) * A * scale
+    probs = torch.softmax(scores.masked_fill(A == 0, float("-inf"))[has], dim=1)  # (rows without nonzeros attend to nothing)
+    ((probs @ v64) * w.double()[has]).sum().backward()
+    tol = 3e-3 if half else 2e-5
+    for got, chained, want in zip(grads[True], grads[False], (q64.grad, k64.grad, v64.grad)):
+        bound = tol * want.abs().max().item()
+        assert (got.double() - want).abs().max().item() <= bound
+        assert (got.double() - chained.double()).abs().max().item() <= 2 * bound
