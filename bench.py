@@ -163,8 +163,8 @@ def main():
     hub = csr.plan if isinstance(csr.plan, rode_sddmm_hip.HubPlan) else None
     grp = csr.plan if isinstance(csr.plan, rode_sddmm_hip.GroupPlan) else None
     lists_run = grp is None or grp.counts[2] > 0  # (with every row in a group the list kernels are not launched)
-    spmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan, k, 4))
-    sddmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan))
+    spmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan, k, 4, seg_length=csr.config["seg_length"]))
+    sddmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan, seg_length=csr.config["seg_length"]))
 
     def spmm_fn(*a, flags=0):  # the whole decomposition is passed, and the library is told so
         return lib.rode_hip_spmm_planned(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS | flags, *a[:-2],

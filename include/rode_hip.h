@@ -254,6 +254,13 @@ int rode_hip_group_plan(int M, const int* d_row_offsets, const int* d_column_ind
  *   groups, group_counts  a group plan of this matrix and its HOST int[4] header (required
  *                         with it).  Needs the complete decomposition, like a hub plan,
  *                         and excludes both other plans.
+ *   seg_length            0, or the segment length the lists were made with (the first
+ *                         argument of the preprocessing call).  Not a plan, but knowledge
+ *                         the launch can use: a decomposition with short segments (the
+ *                         reference's K = 128 set has 32) is walked several segments per
+ *                         wavefront, and with the length known the grid is sized for that.
+ *                         Without it the kernels read the length off the lists and the
+ *                         grid is capped instead.  A wrong value costs time, never a result.
  * Same results as without a plan, up to the order of the fp32 additions inside a row.
  */
 typedef struct rode_hip_plans {
@@ -266,6 +273,7 @@ typedef struct rode_hip_plans {
     size_t hub_workspace_bytes;
     const void* groups;
     const int* group_counts;
+    int seg_length;
 } rode_hip_plans;
 
 /* rode_hip_spmm_ex with plans. */

@@ -52,7 +52,8 @@ class Plans(ctypes.Structure):
     """``rode_hip_plans`` of include/rode_hip.h."""
     _fields_ = [("window", c_void_p), ("window_rows", c_void_p), ("window_counts", c_void_p),
                 ("hub", c_void_p), ("hub_counts", c_void_p), ("hub_workspace", c_void_p),
-                ("hub_workspace_bytes", c_size_t), ("groups", c_void_p), ("group_counts", c_void_p)]
+                ("hub_workspace_bytes", c_size_t), ("groups", c_void_p), ("group_counts", c_void_p),
+                ("seg_length", c_int)]
 
 
 DENSE_CODE = {"f32": 0, "f16": 1, "f64": 2}  # RODE_DENSE_* of include/rode_hip.h

@@ -20,13 +20,13 @@ from . import _lib, rode_sddmm_hip
 def _sddmm(csr, values, lhs, rhs):
     return rode_sddmm_hip.sddmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
                                         csr.row_offsets, csr.column_indices, values.contiguous(), csr.m, csr.n,
-                                        lhs.contiguous(), rhs.contiguous(), lhs.shape[1], plan=csr.plan)
+                                        lhs.contiguous(), rhs.contiguous(), lhs.shape[1], plan=csr.plan, seg_length=csr.config["seg_length"])
 
 
 def _spmm(csr, values, dense):
     return rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
                                        csr.row_offsets, csr.column_indices, values.contiguous(), csr.m, csr.n,
-                                       dense.contiguous(), plan=csr.plan)
+                                       dense.contiguous(), plan=csr.plan, seg_length=csr.config["seg_length"])
 
 
 class SddmmFunction(torch.autograd.Function):

@@ -23,7 +23,7 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 extern "C" {
 
-int rode_hip_version(void) { return (0 << 16) | 1; }
+int rode_hip_version(void) { return (0 << 16) | 2; }
 
 const char* rode_hip_error_string(int code) { return hipGetErrorString(static_cast<hipError_t>(code)); }
 
@@ -175,6 +175,8 @@ namespace {
 bool plan_ref(const rode_hip_plans* p, int m2, rode::PlanRef& plan)
 {
     if (!p) return true;
+    if (p->seg_length < 0) return false;
+    plan.seg_length = p->seg_length;
     const bool window = p->window && p->window_rows; // (one without rows: the standard kernels do everything)
     if (p->groups) {
         // a group plan needs its header on the host, and excludes the other plans (their

@@ -43,6 +43,8 @@ struct PlanRef {
     const int* group_counts = nullptr;
     // SDDMM: the RODE_SPMM_ONLY_* bits of the call (SpMM carries them in its flags)
     int only = 0;
+    // Segment length of the decomposition the lists were made with, 0: not known
+    int seg_length = 0;
 };
 
 hipError_t group_plan_launch(int M, const int* row_ptr, const int* col, int* plan, hipStream_t stream);

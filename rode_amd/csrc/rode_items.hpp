@@ -140,6 +140,147 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
     return true;
 }
 
+// ---- lists with short segments ----------------------------------------------------------
+// A decomposition with short segments (the reference's K = 128 parameter set has 32 slots)
+// arrives as several hundred thousand segments of which most are followers.  One wave per
+// segment then means mostly waves that load four indices to find out that they have
+// nothing to do.  Instead a wave takes a chunk of consecutive segments - as many as make
+// kWalkSlots slots at the decomposition's segment length - and walks it from leader to
+// leader; the workgroups past the last chunk leave after a few scalar loads.  The segment length is read off the lists (the launch arguments do not
+// carry it): two consecutive segments of one row start exactly one segment length apart,
+// the row's first one up to three slots less.  Three evenly spaced pairs are looked at; if
+// none lies within a row (rows of one segment each), or the segments are long, the chunk is
+// one segment and nothing changes.  All waves of a launch compute the same answer.
+constexpr int kWalkSlots = 512;
+constexpr int kWalkMaxChunk = 16;
+constexpr int kWalkMinSegments = 16384; // fewer segments: a small launch needs its waves more than it minds the followers
+
+__device__ __forceinline__ int block_chunk(int m1, const int* __restrict__ block_rows, const int* __restrict__ st_off)
+{
+    // (every load is issued before any is used: one round trip of scalar loads for the waves
+    // that only find out that they have no chunk)
+    constexpr int kPairs = 3;
+    int row[kPairs][2], start[kPairs][2];
+#pragma unroll
+    for (int i = 0; i < kPairs; ++i) {
+        const int p = (int)((long long)m1 * (i + 1) / (kPairs + 1)); // (the same in every lane; m1 >= kWalkMinSegments, so p + 1 < m1)
+        row[i][0] = block_rows[p];
+        row[i][1] = block_rows[p + 1];
+        start[i][0] = st_off[p];
+        start[i][1] = st_off[p + 1];
+    }
+    int seg_len = 0;
+#pragma unroll
+    for (int i = 0; i < kPairs; ++i)
+        if (row[i][0] == row[i][1]) seg_len = max(seg_len, start[i][1] - start[i][0]);
+    if (seg_len <= 0) return 1;
+    seg_len = (seg_len + kBlockItems - 1) / kBlockItems * kBlockItems;
+    return min(max(kWalkSlots / seg_len, 1), kWalkMaxChunk);
+}
+
+// The block part of a grid has at most kBlockGridWaves waves: a launch is sized before anybody
+// knows how long the segments are, and workgroups that find nothing to do still cost their
+// launch (a few hundred thousand of them cost more than the work of an attention mask).  A
+// longer list is walked in chunks as well, of as many segments as it takes to cover it.
+constexpr int kBlockGridWaves = 65536;
+constexpr int kScanSegments = 32; // segments of a chunk looked at together (scan_chunk: a leader's followers end inside the 64 lanes)
+
+// Segments per wave for a list of m1 segments on `nblocks` workgroups; 1: one wave per
+// segment, in the order of xcd_logical_block.
+__device__ __forceinline__ int block_chunk_for_grid(int estimate, int m1, int nblocks)
+{
+    const int waves = nblocks * kWavesPerWg;
+    return max(estimate, (m1 + waves - 1) / waves);
+}
+
+// A caller that says how long the segments of its decomposition are (the plans struct of the
+// planned entry points) spares the kernels the guess and the launch its spare workgroups:
+// the grid then has exactly one wave per chunk.  0: not said.
+__host__ __device__ inline int chunk_for_segments(int seg_length, int m1)
+{
+    if (seg_length <= 0) return 0;
+    if (m1 < kWalkMinSegments) return 1;
+    const int c = kWalkSlots / ((seg_length + kBlockItems - 1) / kBlockItems * kBlockItems);
+    return c < 1 ? 1 : (c > kWalkMaxChunk ? kWalkMaxChunk : c);
+}
+
+// First segment of this wave's chunk, or -1 when it has none.  Consecutive chunks share an
+// XCD: the workgroups with chunks are the first ceil(chunks / 4 / kXcds) of every XCD.
+__device__ __forceinline__ long long chunk_first_segment(int bid, int wave, int m1, int chunk)
+{
+    const int chunks = (m1 + chunk - 1) / chunk;
+    const int per_xcd = ((chunks + kWavesPerWg - 1) / kWavesPerWg + kXcds - 1) / kXcds;
+    if (bid / kXcds >= per_xcd) return -1;
+    const long long first = ((long long)((bid % kXcds) * per_xcd + bid / kXcds) * kWavesPerWg + wave) * chunk;
+    return first < m1 ? first : -1;
+}
+
+// The 64 segments from `first` on, one per lane, looked at together: which of them start
+// something - a work item (a leader), or a stretch that a plan has given to other kernels -
+// and which follow the segment before them.  A row of at most owned_slots slots is one work
+// item (SpMM under the whole-lists promise), else the segments of one window of MERGE slots
+// are (merged_leader's rule).  Two rounds of loads for the whole chunk instead of three per
+// segment.  All 64 lanes call this together.
+struct ChunkScan {
+    int row, row_start, row_end, start; // this lane's segment (start: st_off, also for the entry after the last segment)
+    bool whole;                         // its row is one work item
+    unsigned long long heads;           // bit i: segment first + i follows nothing (bits past the list are set)
+    unsigned long long items;           // bit i: segment first + i starts a work item
+};
+
+__device__ __forceinline__ ChunkScan scan_chunk(int MERGE, int first, int m1, int owned_slots, const RowOwners& owners, int lane,
+                                                const int* __restrict__ block_rows, const int* __restrict__ st_off,
+                                                const int* __restrict__ row_ptr)
+{
+    ChunkScan c;
+    const int s = first + lane;
+    const bool valid = s < m1;
+    c.row = valid ? block_rows[s] : -1;
+    const int prev_row = valid && s > 0 ? block_rows[s - 1] : -1;
+    c.start = s <= m1 ? st_off[s] : 0;
+    const int prev_start = valid && s > 0 ? st_off[s - 1] : 0;
+    c.row_start = valid ? row_ptr[c.row] : 0;
+    c.row_end = valid ? row_ptr[c.row + 1] : 0;
+    const int row_base = c.row_start - (c.row_start & (kVecLen - 1));
+    const int aligned = c.row_end - row_base;
+    const bool elsewhere = valid && owned_elsewhere(owners, c.row, aligned);
+    c.whole = valid && !elsewhere && owned_slots > 0 && aligned <= owned_slots;
+    const bool by_row = elsewhere || c.whole; // every segment of the row follows its first one
+    const bool follower = valid && prev_row == c.row &&
+                          (by_row || (prev_start - row_base) / MERGE == (c.start - row_base) / MERGE);
+    c.heads = __ballot(!follower);
+    c.items = __ballot(valid && !follower && !elsewhere);
+    return c;
+}
+
+// Work item of the leader in lane `i` (the same i in all lanes) of a scanned chunk.  A leader
+// among the first kScanSegments lanes has its last follower at most 31 segments further on
+// (a window of 512 slots, or a row of at most 1024, in segments of 32 or more), so the
+// segment after them is inside the scan as well.
+__device__ __forceinline__ BlockItem chunk_item(const ChunkScan& c, int i)
+{
+    const unsigned long long later = c.heads & ~((2ull << i) - 1ull);
+    const int next = later ? __builtin_ctzll(later) : -1;
+    const int row_start = __builtin_amdgcn_readlane(c.row_start, i), row_end = __builtin_amdgcn_readlane(c.row_end, i);
+    const int start = __builtin_amdgcn_readlane(c.start, i);
+    const int next_start = next >= 0 ? __builtin_amdgcn_readlane(c.start, next) : 0x7fffffff;
+    const int row_base = row_start - (row_start & (kVecLen - 1));
+    BlockItem it;
+    it.row = __builtin_amdgcn_readlane(c.row, i);
+    if (__builtin_amdgcn_readlane((int)c.whole, i)) {
+        it.mask = row_start & (kVecLen - 1);
+        it.base = row_base;
+        it.cnt = row_end - row_base;
+        return it;
+    }
+    // end of the row's block part, or the start of the next leader if that comes first
+    const int block_end = row_base + (row_end - row_base) / kBlockItems * kBlockItems;
+    it.mask = start & (kVecLen - 1);
+    it.base = start - it.mask;
+    it.cnt = min(block_end, next_start) - it.base;
+    return it;
+}
+
 // The row of segment `seg` if spmm_block_item() gives it a work item, else -1 (a follower,
 // or past the list).  The same rules, without the extent of the item: what the waves of a
 // workgroup need to know about each other.

@@ -68,13 +68,32 @@ __device__ __forceinline__ void sddmm_row_slots(int row, int base, int mask, int
 // (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
 template <typename T, int KT, int NS, bool EDGE>
 __device__ __forceinline__ void
-sddmm_block_body(int bid, int nblocks, int m1, int k, RowOwners owners, const int* __restrict__ block_rows,
+sddmm_block_body(int bid, int nblocks, int m1, int k, int chunk_hint, RowOwners owners, const int* __restrict__ block_rows,
                  const int* __restrict__ st_off,
                  const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                  const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
 {
     __shared__ __attribute__((aligned(16))) int lds[kWavesPerWg * kWave];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
+    // Lists with short segments, and many of them: a wave walks a chunk of consecutive
+    // segments from leader to leader, with windows of kWalkSlots slots (rode_items.hpp).
+    const int chunk = chunk_hint > 0 ? chunk_hint
+                                     : block_chunk_for_grid(m1 >= kWalkMinSegments ? block_chunk(m1, block_rows, st_off) : 1, m1, nblocks);
+    if (chunk > 1) {
+        const long long first = chunk_first_segment(bid, wave, m1, chunk);
+        if (first < 0) return;
+        const int last = (int)min(first + chunk, (long long)m1);
+        for (int from = (int)first; from < last; from += kScanSegments) {
+            const ChunkScan scan = scan_chunk(kWalkSlots, from, m1, 0, owners, lane, block_rows, st_off, row_ptr);
+            const int count = min(last - from, kScanSegments);
+            for (unsigned long long todo = scan.items & ((1ull << count) - 1ull); todo; todo &= todo - 1ull) {
+                const BlockItem it = chunk_item(scan, __builtin_ctzll(todo));
+                sddmm_row_slots<T, KT, NS, EDGE>(it.row, it.base, it.mask, it.cnt, it.cnt, 0, k, lane, lds + wave * kWave, col,
+                                                 val, lhs, rhs, out);
+            }
+        }
+        return;
+    }
     const int seg = xcd_logical_block(bid, nblocks) * kWavesPerWg + wave;
     if (seg >= m1) return;
 
@@ -169,12 +188,13 @@ sddmm_residue_body(int bid, int nblocks, int m2, int k, RowOwners owners, const 
 
 template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_block_kernel(int m1, int k, RowOwners owners, const int* __restrict__ block_rows, const int* __restrict__ st_off,
+sddmm_block_kernel(int m1, int k, int chunk_hint, RowOwners owners, const int* __restrict__ block_rows,
+                   const int* __restrict__ st_off,
                    const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                    const T* __restrict__ lhs, const T* __restrict__ rhs, float* __restrict__ out)
 {
-    sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m1, k, owners, block_rows, st_off, row_ptr, col, val, lhs,
-                                      rhs, out);
+    sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, gridDim.x, m1, k, chunk_hint, owners, block_rows, st_off, row_ptr, col, val,
+                                      lhs, rhs, out);
 }
 
 template <typename T, int KT, int NS, bool EDGE>
@@ -191,14 +211,15 @@ sddmm_residue_kernel(int m2, int k, RowOwners owners, const int* __restrict__ re
 // residue rows.  For matrices so small that a launch costs as much as its kernel.
 template <typename T, int KT, int NS, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-sddmm_pair_kernel(int g1, int m1, int m2, int k, RowOwners owners, const int* __restrict__ block_rows,
+sddmm_pair_kernel(int g1, int m1, int m2, int k, int chunk_hint, RowOwners owners, const int* __restrict__ block_rows,
                   const int* __restrict__ residue_rows,
                   const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const float* __restrict__ val, const T* __restrict__ lhs, const T* __restrict__ rhs,
                   float* __restrict__ out, const int* __restrict__ plan)
 {
     if ((int)blockIdx.x < g1)
-        sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, g1, m1, k, owners, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+        sddmm_block_body<T, KT, NS, EDGE>(blockIdx.x, g1, m1, k, chunk_hint, owners, block_rows, st_off, row_ptr, col, val, lhs,
+                                          rhs, out);
     else
         sddmm_residue_body<T, KT, NS, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, k, owners, residue_rows, row_ptr, col, val, lhs,
                                             rhs, out, plan);
@@ -415,7 +436,9 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
                   PlanRef plan, hipStream_t s1, hipStream_t s2)
 {
     constexpr int RPW = kWave / SddmmShape<T, KT>::kLpr;
-    const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
+    const int chunk_hint = chunk_for_segments(plan.seg_length, m1); // (segments per wave; 0: the kernels find out)
+    const int g1 = chunk_hint > 0 ? grid_for_waves((m1 + chunk_hint - 1) / chunk_hint) : grid_for_waves(min(m1, kBlockGridWaves));
+    const int g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0) return hipErrorInvalidConfiguration;
     // With a host copy of the plan's header, a kernel that would find every chunk taken by
     // the other one is not launched at all.
@@ -442,11 +465,11 @@ hipError_t launch(int m1, int m2, int k, const int* block_rows, const int* resid
     if (group_plan && plan.group_counts[2] == 0) m1 = m2 = 0; // every row in a group with a run: nothing for the lists' kernels
     if (m1 > 0 && m2 > 0 && standard_residue && s1 == s2 && g1 + g2 <= kPairMaxWorkgroups) {
         sddmm_pair_kernel<T, KT, NS, EDGE><<<g1 + g2, kWgThreads, 0, s1>>>(
-            g1, m1, m2, k, owners, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);
+            g1, m1, m2, k, chunk_hint, owners, block_rows, residue_rows, st_off, row_ptr, col, val, lhs, rhs, out, plan.dev);
     } else {
         if (m1 > 0) {
             sddmm_block_kernel<T, KT, NS, EDGE><<<g1, kWgThreads, 0, s1>>>(
-                m1, k, owners, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
+                m1, k, chunk_hint, owners, block_rows, st_off, row_ptr, col, val, lhs, rhs, out);
         }
         if (m2 > 0 && standard_residue) {
             sddmm_residue_kernel<T, KT, NS, EDGE><<<g2, kWgThreads, 0, s2>>>(

@@ -127,7 +127,8 @@ __device__ __forceinline__ void spmm_sum_slots(int base, int mask, int cnt, int 
 // (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
 template <typename T, int TN, bool EDGE>
 __device__ __forceinline__ void
-spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, RowOwners owners, const int* __restrict__ block_rows,
+spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int chunk_hint, RowOwners owners,
+                const int* __restrict__ block_rows,
                 const int* __restrict__ st_off, const int* __restrict__ row_ptr, const int* __restrict__ col,
                 const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                 typename DenseVec<T>::Acc* __restrict__ C)
@@ -138,6 +139,52 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, RowOwners 
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) A lds_v[kWavesPerWg * kWave];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave; // (uniform: scalar registers)
+    // Lists with short segments (and enough of them that merging is on): a wave walks a chunk
+    // of consecutive segments from leader to leader, adds up what it finds for one row and
+    // updates that row of C once (the sums of the items, not one long sum: same rounding as
+    // the combine of neighbouring waves below).
+    const int chunk = chunk_hint > 0 ? chunk_hint
+                                     : block_chunk_for_grid(owned_slots != 0 && m1 >= kWalkMinSegments
+                                                                ? block_chunk(m1, block_rows, st_off) : 1, m1, nblocks);
+    if (chunk > 1) {
+        const long long first = chunk_first_segment(bid, wave, m1, chunk);
+        if (first < 0) return;
+        const int last = (int)min(first + chunk, (long long)m1);
+        const int ls = lane % LPR, group = lane / LPR;
+        const int tile = blockIdx.y * TN;
+        const bool col_ok = !EDGE || tile + ls * VEC < n;
+        const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
+        constexpr int EPG = VEC / G > 0 ? VEC / G : 1; // elements each lane group adds to C
+        A row_total[VEC];
+        int pending = -1; // the row that row_total belongs to
+        auto flush = [&]() {
+            A* c_lane = C + (size_t)pending * n + tile + ls * VEC;
+#pragma unroll
+            for (int x = 0; x < VEC; ++x)
+                if (group == x / EPG && col_ok) atomicAdd(c_lane + x, row_total[x]);
+        };
+        for (int from = (int)first; from < last; from += kScanSegments) {
+            const ChunkScan scan = scan_chunk(kSpmmMergeSlots, from, m1, owned_slots, owners, lane, block_rows, st_off, row_ptr);
+            const int count = min(last - from, kScanSegments);
+            for (unsigned long long todo = scan.items & ((1ull << count) - 1ull); todo; todo &= todo - 1ull) {
+                const BlockItem it = chunk_item(scan, __builtin_ctzll(todo));
+                A total[VEC];
+                spmm_sum_slots<T, TN>(it.base, it.mask, it.cnt, it.cnt, 0, lane, lds_c + wave * kWave, lds_v + wave * kWave,
+                                      b_lane, n, col, val, total);
+                if (it.row != pending) {
+                    if (pending >= 0) flush();
+                    pending = it.row;
+#pragma unroll
+                    for (int x = 0; x < VEC; ++x) row_total[x] = total[x];
+                } else {
+#pragma unroll
+                    for (int x = 0; x < VEC; ++x) row_total[x] += total[x];
+                }
+            }
+        }
+        if (pending >= 0) flush();
+        return;
+    }
     const int seg0 = xcd_logical_block(bid, nblocks) * kWavesPerWg;
     const int seg = seg0 + wave;
     BlockItem it{-1, 0, 0, 0};
@@ -272,14 +319,14 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, RowOwner
 
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_block_kernel(int m1, int n, int owned_slots, RowOwners owners, const int* __restrict__ block_rows,
+spmm_block_kernel(int m1, int n, int owned_slots, int chunk_hint, RowOwners owners, const int* __restrict__ block_rows,
                   const int* __restrict__ st_off,
                   const int* __restrict__ row_ptr, const int* __restrict__ col,
                   const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                   typename DenseVec<T>::Acc* __restrict__ C)
 {
-    spmm_block_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m1, n, owned_slots, owners, block_rows, st_off, row_ptr, col, val,
-                                 B, C);
+    spmm_block_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m1, n, owned_slots, chunk_hint, owners, block_rows, st_off, row_ptr,
+                                 col, val, B, C);
 }
 
 template <typename T, int TN, bool EDGE>
@@ -298,13 +345,15 @@ spmm_residue_kernel(int m2, int n, int owned_slots, RowOwners owners, const int*
 // kernel (a kernel of a few microseconds); the two parts then also fill the GPU together.
 template <typename T, int TN, bool EDGE>
 __global__ void __launch_bounds__(kWgThreads)
-spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, RowOwners owners, const int* __restrict__ block_rows,
+spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, int chunk_hint, RowOwners owners,
+                 const int* __restrict__ block_rows,
                  const int* __restrict__ residue_rows, const int* __restrict__ st_off, const int* __restrict__ row_ptr,
                  const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
                  const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
     if ((int)blockIdx.x < g1)
-        spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, owners, block_rows, st_off, row_ptr, col, val, B, C);
+        spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, chunk_hint, owners, block_rows, st_off, row_ptr, col, val,
+                                     B, C);
     else
         spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, max(owned_slots, 0), owners, residue_rows,
                                        row_ptr, col, val,
@@ -647,7 +696,10 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     const bool hubs = hub_plan && (only == 0 || only == kSpmmOnlyHub);
     const bool grouped = group_plan && (only == 0 || only == kSpmmOnlyHub); // (timed with the hub kernels)
     constexpr int RPW = kWave / SpmmShape<T, TN>::kLpr;
-    const int g1 = grid_for_waves(m1), g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
+    // (segments per wave: known only when the caller said how long its segments are and merging is on)
+    const int chunk_hint = block_owned != 0 ? chunk_for_segments(plan.seg_length, m1) : (plan.seg_length > 0 ? 1 : 0);
+    const int g1 = chunk_hint > 0 ? grid_for_waves((m1 + chunk_hint - 1) / chunk_hint) : grid_for_waves(min(m1, kBlockGridWaves));
+    const int g2 = grid_for_waves(((long long)m2 + RPW - 1) / RPW);
     if (g1 < 0 || g2 < 0 || tiles > 65535) return hipErrorInvalidConfiguration;
     // With a host copy of the plan's header, a kernel that would find every chunk taken by
     // the other one is not launched at all.
@@ -663,14 +715,14 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     hipError_t e = hipSuccess;
     if (block && residue && standard_residue && s1 == s2 && (long long)(g1 + g2) * tiles <= kPairMaxWorkgroups) {
         dim3 grid(g1 + g2, tiles);
-        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, owners, block_rows, residue_rows,
-                                                                   st_off, row_ptr, col, val, B, C, plan.dev);
+        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, chunk_hint, owners, block_rows,
+                                                                   residue_rows, st_off, row_ptr, col, val, B, C, plan.dev);
         e = hipGetLastError();
     } else {
         if (block) {
             dim3 grid(g1, tiles);
-            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, owners, block_rows, st_off, row_ptr,
-                                                                        col, val, B, C);
+            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows, st_off,
+                                                                        row_ptr, col, val, B, C);
             e = hipGetLastError();
         }
         if (residue && standard_residue) {

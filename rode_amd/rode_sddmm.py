@@ -274,7 +274,8 @@ def rode_sddmm(sparse_matrix, lhs, rhs, values=None):
     return rode_sddmm_hip.sddmm_forward(
         sparse_matrix.block_indices, sparse_matrix.residue_indices, sparse_matrix.st_offsets,
         sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,
-        sparse_matrix.values, m, n, lhs.contiguous(), rhs.contiguous(), k, plan=sparse_matrix.plan)
+        sparse_matrix.values, m, n, lhs.contiguous(), rhs.contiguous(), k, plan=sparse_matrix.plan,
+        seg_length=sparse_matrix.config["seg_length"])
 
 
 def torch_sddmm_reference(sparse_csr, lhs_matrix, rhs_matrix):

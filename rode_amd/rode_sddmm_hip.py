@@ -259,12 +259,14 @@ def group_plan(row_offsets, column_indices, m):
     return GroupPlan(data, list(counts))
 
 
-def plans_struct(plan, spmm_width=None, spmm_elem_bytes=4, whole_lists=True):
+def plans_struct(plan, spmm_width=None, spmm_elem_bytes=4, whole_lists=True, seg_length=0):
     """The ``rode_hip_plans`` struct of one call (keep it alive until the call returns; pass
     it with ``ctypes.byref``).  ``plan``: a ``WindowPlan``, a ``HubPlan``, a ``GroupPlan`` or None.
     ``spmm_width``: for an SpMM call the dense width, so that a hub plan's workspace is
-    attached; a hub plan is left out of an SpMM call without the whole-lists promise."""
+    attached; a hub plan is left out of an SpMM call without the whole-lists promise.
+    ``seg_length``: the segment length the lists were made with, 0 when not known."""
     p = _lib.Plans()
+    p.seg_length = int(seg_length or 0)  # (the segment length of the decomposition, when the caller knows it)
     if isinstance(plan, GroupPlan):
         if plan.usable and (spmm_width is None or whole_lists):
             p.groups, p.group_counts = plan.data.data_ptr(), ctypes.addressof(plan._header)
@@ -301,7 +303,7 @@ def _dense_kind(lhs_matrix, rhs_matrix, lhs_name, rhs_name):
 
 
 def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, n,
-                  lhs_matrix, rhs_matrix, k_version, plan=None):
+                  lhs_matrix, rhs_matrix, k_version, plan=None, seg_length=0):
     """``rode_sddmm_cuda.sddmm_forward`` (``rode_sddmm_cuda.cu:136-249``).
 
     Differences from the reference, none of which changes a result: any k_version
@@ -309,7 +311,8 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
     ``lhs_matrix``/``rhs_matrix`` (fp32 accumulate) are accepted too; the
     kernels are queued on PyTorch's current stream instead of two streams that
     are created, synchronised and destroyed per call (``:203-246``).  ``plan``: a
-    ``WindowPlan`` made from this very residue list, or None.
+    plan made from these very lists, or None; ``seg_length``: the segment length the lists were
+    made with (``preprocess``'s third argument), 0 when not known.
     """
     for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
                     (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
@@ -337,7 +340,7 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
     lib = _lib.load()
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
-        plans = plans_struct(plan)
+        plans = plans_struct(plan, seg_length=seg_length)
         code = lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[kind], 0, m1, m2, n, k, block_indices.data_ptr(),
                                           residue_indices.data_ptr(), st_offsets.data_ptr(), row_offsets.data_ptr(),
                                           column_indices.data_ptr(), values.data_ptr(), lhs_matrix.data_ptr(),
@@ -347,7 +350,7 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
 
 
 def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, k,
-                 dense_matrix, out=None, whole_lists=True, plan=None):
+                 dense_matrix, out=None, whole_lists=True, plan=None, seg_length=0):
     """C = A_csr @ dense_matrix through ``rode_hip_spmm_f32`` / ``_f16``
     (host API ``RoDe_SpMM/RoDeSpmm.h:4-8``).  ``dense_matrix`` is (k, n) with n a
     multiple of 4 (8 for fp16, 2 for fp64), fp32 / fp16 (fp32 ``values``) or fp64 (fp64 ``values``); the
@@ -392,7 +395,7 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     dtype = {torch.float32: 0, torch.float16: 1, torch.float64: 2}[dense_matrix.dtype]  # RODE_DENSE_*
     with torch.cuda.device(values.device):
         s = _stream_handle(values.device)
-        plans = plans_struct(plan, n, out.element_size(), whole_lists)
+        plans = plans_struct(plan, n, out.element_size(), whole_lists, seg_length=seg_length)
         code = lib.rode_hip_spmm_planned(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
                                          values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
                                          block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),

@@ -436,3 +436,61 @@ def sub_csr(rp, rows):
     sub_rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     idx = np.concatenate([np.arange(rp[r], rp[r + 1], dtype=np.int64) for r in rows])
     return sub_rp, idx
+
+
+@pytest.mark.parametrize("seg", [32, 64, 160])
+def test_many_short_segments_write_exactly_their_entries(seg):
+    """At least 16384 segments of a short length: a wave walks a chunk of consecutive segments
+    from leader to leader (rode_items.hpp).  Through the typed entry point, whole lists and in
+    two slices cut inside a row: every entry a work item owns is written with the right value,
+    the entries of empty or absent work items keep their canary, nothing outside out[0, nnz)."""
+    import oracle
+    from gpu_common import DEV
+    from helpers import merged_block_ranges, residue_ranges
+    from rode_amd import _lib, rode_sddmm_hip
+    rng = np.random.default_rng(1000 + seg)
+    m, n, k = {32: 3000, 64: 4500, 160: 10000}[seg], 4000, 32
+    lens = rng.choice([0, 5, 31, 33, 200, 700, 1500, 3900], size=m, p=[.05, .1, .1, .15, .2, .2, .15, .05])
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(n, size=l, replace=False)) for l in lens]).astype(np.int32)
+    val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    nnz = len(val)
+    d_rp = torch.from_numpy(rp).to(DEV)
+    blk, st, res, m1, m2 = rode_sddmm_hip.preprocess_device(d_rp, nnz, seg, 32, 4)
+    assert m1 >= 2 * 16384  # (each of the two slices below still has enough segments for the walk)
+    oblk, ost, ores = oracle.preprocess(rp, seg)
+    expect = np.zeros(nnz, bool)
+    for r, _, first, end in merged_block_ranges(rp, oblk, ost, 512):
+        expect[first:end] = True
+    for r, first, end in residue_ranges(rp, ores):
+        expect[first:end] = True
+    ref, scale = oracle.sddmm_f64(rp, col, val, lhs, rhs, with_abs=True)
+    lib = _lib.load()
+    pad = 256
+    dcol = torch.zeros(nnz + 2 * pad, dtype=torch.int32, device=DEV)
+    dval = torch.zeros(nnz + 2 * pad, dtype=torch.float32, device=DEV)
+    dcol[pad:pad + nnz] = torch.from_numpy(col).to(DEV)
+    dval[pad:pad + nnz] = torch.from_numpy(val).to(DEV)
+    dl, dr = torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV)
+
+    def call(out, a, b, with_residue):
+        _lib.check(lib.rode_hip_sddmm_f32(b - a, m2 if with_residue else 0, n, k, blk.data_ptr() + 4 * a, res.data_ptr(),
+                                          st.data_ptr() + 4 * a, d_rp.data_ptr(), dcol.data_ptr() + 4 * pad,
+                                          dval.data_ptr() + 4 * pad, dl.data_ptr(), dr.data_ptr(), out.data_ptr() + 4 * pad,
+                                          None, None), "sddmm")
+
+    inside = np.nonzero(oblk[1:] == oblk[:-1])[0] + 1   # segments that are not the first of their row
+    cut = int(inside[np.searchsorted(inside, m1 // 2)])  # inside a row: the second slice starts with one of its later segments
+    assert oblk[cut] == oblk[cut - 1] and m1 - cut >= 16384 <= cut
+    for slices in ([(0, m1)], [(0, cut), (cut, m1)]):
+        out = torch.full((nnz + 2 * pad,), -777.0, device=DEV)
+        for i, (a, b) in enumerate(slices):
+            call(out, a, b, i == 0)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert (got[:pad] == -777.0).all() and (got[pad + nnz:] == -777.0).all(), "write outside out[0, nnz)"
+        got = got[pad:pad + nnz]
+        assert ((got != -777.0) == expect).all(), "written entries differ from the host model"
+        assert np.max(np.abs(got[expect] - ref[expect]) / np.maximum(scale[expect], 1e-30)) <= 2e-6
