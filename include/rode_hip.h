@@ -55,7 +55,11 @@ size_t rode_hip_preprocess_workspace_bytes(int M);
  *                    (the reference sizes it nnz/seg + M, _preprocess.cu:426).  If it is
  *                    too small nothing is written past it and *d_n_blk still reports
  *                    the true count, so the caller can detect the overflow.
- *   d_workspace      rode_hip_preprocess_workspace_bytes(M) bytes, 8-byte aligned
+ *   d_workspace      rode_hip_preprocess_workspace_bytes(M) bytes, 8-byte aligned (8 bytes per
+ *                    1024 rows: the status words of the scan across workgroups)
+ * Two launches: a fill of the scratch, then one kernel that reads row_ptr once, scans and
+ * writes the lists.  Should a workgroup ever wait in vain for an earlier one (bounded; it
+ * cannot happen while the GPU runs workgroups it has started), *d_n_blk = *d_n_res = -1.
  */
 int rode_hip_preprocess(int seg_length, int k_block, int vec_len, int M, const int* d_row_ptr,
                         int* d_block_r_ind, int* d_st_off, int* d_residue_r_ind, int* d_n_blk, int* d_n_res,
@@ -81,7 +85,7 @@ int rode_hip_preprocess_host(int seg_length, int k_block, int vec_len, int M, co
  * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its GPU
  * routine allocates and frees CUB scratch on every call, _preprocess.cu:331-335).
  * Same arguments, same kernels and byte-identical results; the scan scratch is a fixed
- * array inside the library (16.1 MiB of device memory per GPU, held until the process
+ * array inside the library (33 KB of device memory per GPU, held until the process
  * ends), so M is limited to RODE_HIP_STATIC_MAX_ROWS: a larger M returns
  * hipErrorOutOfMemory (2) before anything is launched.  The first call on a device looks
  * up the array's address (no allocation; make that call outside stream capture).  Every

@@ -552,6 +552,16 @@ void RoDe_preprocess(int SegmentLength, int vectorLen, int KBLOCK, int M, const 
 void RoDe_preprocess(int N_SEG, int blockX, int vecLen, int M, const int* row_ptr, int* block_r_ind, int* st_off,
                      int* residue_r_ind, int* n_blk, int* n_res)
 {
+    // The signature carries no capacity: the caller's arrays are trusted to hold
+    // the result, as in the reference.  Nor does it carry scratch: the library's own fixed
+    // array serves every matrix it can hold (no allocation, the call only queues kernels on
+    // the default stream; calls that overlap in time on one GPU must not use this entry
+    // point), a larger one gets scratch for the call.
+    if (M <= RODE_HIP_STATIC_MAX_ROWS) {
+        report("RoDe_preprocess", rode_hip_preprocess_static(N_SEG, blockX, vecLen, M, row_ptr, block_r_ind, st_off,
+                                                             residue_r_ind, n_blk, n_res, 0x7fffffff, nullptr));
+        return;
+    }
     void* ws = nullptr;
     const size_t bytes = rode_hip_preprocess_workspace_bytes(M);
     hipError_t e = hipMalloc(&ws, bytes);
@@ -559,8 +569,6 @@ void RoDe_preprocess(int N_SEG, int blockX, int vecLen, int M, const int* row_pt
         report("RoDe_preprocess", (int)e);
         return;
     }
-    // The signature carries no capacity: the caller's arrays are trusted to hold
-    // the result, as in the reference.
     report("RoDe_preprocess", rode_hip_preprocess(N_SEG, blockX, vecLen, M, row_ptr, block_r_ind, st_off,
                                                   residue_r_ind, n_blk, n_res, 0x7fffffff, ws, bytes, nullptr));
     (void)hipFree(ws); // waits for the queued kernels
