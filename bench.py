@@ -25,6 +25,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+CLOCK_HZ = 2.4e9        # MI355X peak engine clock
+CUS, SIMDS = 256, 1024
+# fp32 multiply-adds of the vector units without packed instructions (this build compiles none):
+# 1024 SIMDs x 16 lanes x 2 flop x 2.4 GHz; the published 157.3 TFLOP/s counts two per lane and clock
+VALU_PEAK_TFLOPS = 78.6
+# LDS reads: 107 bytes per clock and CU is what ds_read_b128 of random rows sustains on this GPU
+# (measured with a stand-alone gather loop; conflict-free reads reach 205)
+LDS_PEAK_GBS = 107.0 * CUS * CLOCK_HZ / 1e9
 TOL = {"f32": 1e-4, "f16": 2e-3}  # max over rows of |err|_inf / |ref row|_1
 
 
@@ -37,7 +45,8 @@ def kernel_sources_fingerprint():
     import re
     h = hashlib.sha256()
     for name in ("rode_device.hpp", "rode_items.hpp", "rode_units.hpp", "rode_window.hpp", "rode_spmm.hip", "rode_sddmm.hip",
-                 "rode_spmm_window.hip", "rode_sddmm_window.hip"):
+                 "rode_spmm_window.hip", "rode_sddmm_window.hip", "rode_attention.hip", "rode_attention_backward.hip",
+                 "rode_group.hip", "rode_hub.hip"):
         with open(os.path.join(ROOT, "rode_amd", "csrc", name), "r", encoding="utf-8") as f:
             for line in f:
                 code = re.sub(r"//.*$", "", line).strip()
@@ -69,6 +78,8 @@ def parse_args():
                         "\"probs\" also writes the probabilities a gradient needs")
     p.add_argument("--chain", action="store_true",
                    help="step = SDDMM scores -> row softmax -> clear C -> SpMM with those values (sparse attention)")
+    p.add_argument("--heads", type=int, default=1,
+                   help="with --chain --fused yes/probs: attention heads on the one mask, all in the same launches")
     p.add_argument("--train", action="store_true",
                    help="with --chain --fused probs: the step is the attention forward with its probabilities written "
                         "plus the two gradient kernels (rode_hip_attention_backward_rows / _cols)")
@@ -215,7 +226,15 @@ def main():
                    "sddmm")
         join()
 
-    probs = torch.empty(nnz, device=dev) if args.chain else None
+    H = args.heads
+    if H > 1 and not (args.chain and args.fused != "no"):
+        print("bench.py: --heads needs --chain --fused yes|probs", file=sys.stderr)
+        sys.exit(2)
+    probs = torch.empty(H * nnz, device=dev) if args.chain else None
+    if H > 1:  # (every head its own q, k, v)
+        B = torch.randn(H * n, k, device=dev, generator=gen).to(tdtype)
+        L = torch.randn(H * m, k, device=dev, generator=gen).to(tdtype)
+        C = torch.zeros(H * m, k, device=dev)
     if args.chain:
         args.no_cpu = True  # (the CPU leg and its parity gate are those of SpMM + SDDMM; the chain is checked by the tests)
     if args.train:
@@ -226,20 +245,20 @@ def main():
         t_slot = csr.transposed_slots()
         grp_t = csr_t.plan if isinstance(csr_t.plan, rode_sddmm_hip.GroupPlan) else None
         plans_t = ctypes.byref(rode_sddmm_hip.plans_struct(grp_t))
-        G = torch.randn(m, k, device=dev, generator=gen)  # gradient of the loss with respect to the output
-        dQ, dK, dV = (torch.empty(r, k, device=dev) for r in (m, n, n))
-        pairs = torch.empty(2 * nnz, device=dev)
+        G = torch.randn(H * m, k, device=dev, generator=gen)  # gradient of the loss with respect to the output
+        dQ, dK, dV = (torch.empty(H * r, k, device=dev) for r in (m, n, n))
+        pairs = torch.empty(2 * H * nnz, device=dev)
 
     def backward_rows():
         _lib.check(lib.rode_hip_attention_backward_rows(
-            _lib.DENSE_CODE[args.dtype], m, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
+            _lib.DENSE_CODE[args.dtype], H, m, n, nnz, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
             csr.values.data_ptr(), probs.data_ptr(), G.data_ptr(), C.data_ptr(), B.data_ptr(), B.data_ptr(),
             float(k) ** -0.5, t_slot.data_ptr(), dQ.data_ptr(), pairs.data_ptr(), sddmm_plans, stream),
             "attention backward, rows")
 
     def backward_cols():
         _lib.check(lib.rode_hip_attention_backward_cols(
-            _lib.DENSE_CODE[args.dtype], n, k, csr_t.row_offsets.data_ptr(), csr_t.column_indices.data_ptr(),
+            _lib.DENSE_CODE[args.dtype], H, m, n, nnz, k, csr_t.row_offsets.data_ptr(), csr_t.column_indices.data_ptr(),
             pairs.data_ptr(), G.data_ptr(), L.data_ptr(), dK.data_ptr(), dV.data_ptr(), plans_t, stream),
             "attention backward, columns")
 
@@ -254,12 +273,15 @@ def main():
                            csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(),
                            csr.st_offsets.data_ptr(), B.data_ptr(), C.data_ptr(), stream, stream), "spmm")
 
+    def attention_forward():
+        _lib.check(lib.rode_hip_attention_forward_batched(
+            _lib.DENSE_CODE[args.dtype], H, m, n, nnz, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
+            csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), B.data_ptr(), float(k) ** -0.5, C.data_ptr(),
+            probs.data_ptr() if args.fused == "probs" else None, sddmm_plans, stream), "attention")
+
     def step():
         if args.chain and args.fused != "no":
-            _lib.check(lib.rode_hip_attention_forward(
-                _lib.DENSE_CODE[args.dtype], m, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
-                csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), B.data_ptr(), float(k) ** -0.5, C.data_ptr(),
-                probs.data_ptr() if args.fused == "probs" else None, sddmm_plans, stream), "attention")
+            attention_forward()
             if args.train:
                 backward_rows()
                 backward_cols()
@@ -298,7 +320,7 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
-    flops_per_step = (6 if args.train else 2) * (2.0 * nnz * k)  # (a gradient: four more products)
+    flops_per_step = (6 if args.train else 2) * (2.0 * nnz * k) * args.heads  # (a gradient: four more products)
     gflops = flops_per_step / (ms_per_step * 1e-3) / 1e9
 
     # ---- per-kernel durations, HIP events on the launch stream ----------------
@@ -330,6 +352,7 @@ def main():
 
     reps = max(3, min(args.steps, 20))
     preprocess_ms = event_time(preprocess, reps)
+    pre_bytes = (m + 1) * 4 + (2 * csr.m1 + 1 + csr.m2) * 4
     del p_blk, p_st, p_res, p_ws
     kernels = {}
     if csr.m1 > 0 and lists_run:
@@ -344,6 +367,8 @@ def main():
     if grp is not None:  # the rows of the group plan's groups (the same flag selects them)
         kernels["spmm_group"] = event_time(lambda: spmm_only(_lib.SPMM_ONLY_HUB), reps)
         kernels["sddmm_group"] = event_time(lambda: sddmm(csr.m1, csr.m2, _lib.SPMM_ONLY_HUB), reps)
+    if args.chain and args.fused != "no":
+        kernels["attention_forward"] = event_time(attention_forward, reps)
     if args.train:
         kernels["attention_backward_rows"] = event_time(backward_rows, reps)
         kernels["attention_backward_cols"] = event_time(backward_cols, reps)
@@ -371,11 +396,17 @@ def main():
         if name.startswith("attention"):
             # row pass: (col, val, p, slot in the transposed pattern) read, (p, dz) written, rows of g, out,
             # dq, every k and v row once; column pass: row and (p, dz) read, rows of dk, dv, every g and q row once
-            ab = nnz * (16 + 8) + 3 * m * k * 4 + 2 * n * k * elem if name.endswith("rows") else \
-                nnz * (4 + 8) + 2 * n * k * 4 + m * k * (4 + elem)
+            # forward: (col, val) read, probabilities written if asked for, q and out rows, every k and v row once
+            if name.endswith("forward"):
+                ab = nnz * (8 + (4 if args.fused == "probs" else 0)) + m * k * (elem + 4) + 2 * n * k * elem
+            elif name.endswith("rows"):
+                ab = nnz * (16 + 8) + 3 * m * k * 4 + 2 * n * k * elem
+            else:
+                ab = nnz * (4 + 8) + 2 * n * k * 4 + m * k * (4 + elem)
+            ab *= H
             per_kernel[name] = {"ms": round(ms, 4), "algorithmic_bytes": ab, "algorithmic_GBs": round(ab / ms / 1e6, 1),
-                                "gather_model_GBs": round(nnz * (16 + 2 * k * elem) / ms / 1e6, 1),
-                                "GFLOPs": round(2 * 2.0 * nnz * k / ms / 1e6, 1)}
+                                "gather_model_GBs": round(H * nnz * (16 + 2 * k * elem) / ms / 1e6, 1),
+                                "GFLOPs": round(H * 2 * 2.0 * nnz * k / ms / 1e6, 1)}
             continue
         split = split_spmm if name.startswith("spmm") else split_sddmm
         m2_eff = csr.m2
@@ -388,7 +419,7 @@ def main():
                             "gather_model_GBs": round((knnz * (8 + k * elem)) / ms / 1e6, 1),
                             "GFLOPs": round(2.0 * knnz * k / ms / 1e6, 1)}
     dominant = max(kernels, key=kernels.get)
-    traffic, traffic_note = None, "no counter run of this workload under profiles/"
+    traffic, traffic_note, entry = None, "no counter run of this workload under profiles/", None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         table = json.load(open(tpath))
@@ -401,14 +432,40 @@ def main():
             traffic, traffic_note = entry["bytes"], entry.get("kernel")
         elif entry is not None:
             traffic_note = "stale: the counter run under profiles/ was made on other kernel sources"
+            entry = None
     dom = per_kernel[dominant]
-    roofline = {"bound": "hbm", "kernel": dominant, "achieved": dom["algorithmic_GBs"], "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(dom["algorithmic_GBs"] / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "traffic_source": traffic_note,
-                # the same kernel's measured HBM bytes over its time: how busy the memory system was
-                "traffic_GBs": None if traffic is None else round(traffic / kernels[dominant] / 1e6, 1),
-                "traffic_frac": None if traffic is None else round(traffic / kernels[dominant] / 1e6 / HBM_PEAK_GBS, 4),
-                "gather_model_frac": round(dom["gather_model_GBs"] / HBM_PEAK_GBS, 4)}
+    dom_ms = kernels[dominant]
+    hbm = {"achieved": dom["algorithmic_GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+           "frac": round(dom["algorithmic_GBs"] / HBM_PEAK_GBS, 4),
+           # the same kernel's measured HBM bytes over its time: how busy the memory system was
+           "traffic_GBs": None if traffic is None else round(traffic / dom_ms / 1e6, 1),
+           "traffic_frac": None if traffic is None else round(traffic / dom_ms / 1e6 / HBM_PEAK_GBS, 4),
+           "gather_model_frac": round(dom["gather_model_GBs"] / HBM_PEAK_GBS, 4)}
+    # Which resource binds the kernel: HBM when its measured traffic moves at half the peak or
+    # more; else whichever of the vector ALUs (instructions issued x 4 clocks per wavefront
+    # instruction over the SIMD-clocks of the launch) and the LDS pipe (its active cycles over
+    # the CU-clocks of the launch) is busier, from the counters of the same profile.
+    bound, busy = "hbm", {}
+    if entry is not None and traffic is not None and "valu_insts" in entry:
+        clocks = dom_ms * 1e-3 * CLOCK_HZ
+        busy = {"hbm": hbm["traffic_frac"], "valu": round(entry["valu_insts"] * 4 / (clocks * SIMDS), 4),
+                "lds": round(entry["lds_active_cycles"] / (clocks * CUS), 4)}
+        if busy["hbm"] < 0.5:
+            bound = max(busy, key=busy.get)
+    knnz_dom = dom["GFLOPs"] * dom_ms * 1e6 / (2.0 * k)  # nonzeros of the dominant kernel
+    if bound == "valu":
+        ach = dom["GFLOPs"] / 1e3
+        top = {"achieved": round(ach, 2), "peak": VALU_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / VALU_PEAK_TFLOPS, 4),
+               "peak_is": "fp32 vector multiply-adds without packed instructions (published 157.3 TFLOP/s counts packed pairs)"}
+    elif bound == "lds":
+        ach = knnz_dom * k * elem / dom_ms / 1e6  # every nonzero's dense row read from LDS once
+        top = {"achieved": round(ach, 1), "peak": round(LDS_PEAK_GBS, 1), "unit": "GB/s", "frac": round(ach / LDS_PEAK_GBS, 4),
+               "peak_is": "LDS read pipe: 107 B per clock and CU for 128-bit reads of random rows (measured), x 256 CUs x 2.4 GHz"}
+    else:
+        top = {k2: hbm[k2] for k2 in ("achieved", "peak", "unit", "frac")}
+    roofline = {"bound": bound, "kernel": dominant, **top, "traffic": traffic, "traffic_source": traffic_note,
+                "busy": busy or None, "hbm": hbm,
+                "traffic_GBs": hbm["traffic_GBs"], "traffic_frac": hbm["traffic_frac"], "gather_model_frac": hbm["gather_model_frac"]}
 
     # ---- CPU baseline: the oracle on a bounded sample of the same matrix --------
     cpu = None
@@ -528,7 +585,7 @@ def main():
                                    if args.fused != "no" else "step = SDDMM -> row softmax -> clear C -> SpMM (chained)")
                                   if args.chain
                                   else "step = clear C rows + SpMM + SDDMM"),
-                   "rows": m, "cols": n, "nnz": nnz, "K": k, "seg_length": csr.config["seg_length"],
+                   "rows": m, "cols": n, "nnz": nnz, "K": k, "heads": args.heads, "seg_length": csr.config["seg_length"],
                    "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale,
                    "locality_plan": None if csr.plan is None or hub is not None or grp is not None else
                    {"residue_chunks": csr.plan.counts[0], "chunks_with_lds_window": csr.plan.counts[1]},
@@ -545,7 +602,11 @@ def main():
         "sddmm": {"ms": round(sddmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / sddmm_ms / 1e6, 1)},
         "kernels": per_kernel,
         "preprocess": {"ms": round(preprocess_ms, 4), "rows_per_s": round(m / preprocess_ms * 1e3),
-                       "note": "GPU row decomposition (4 kernels), not part of the step"},
+                       "note": "GPU row decomposition (a fill of the scan's status words + one kernel), not part of the step",
+                       # compulsory bytes: row_ptr read once, both lists, the segment starts and the sentinel written once
+                       "roofline": {"bound": "hbm", "algorithmic_bytes": pre_bytes,
+                                    "achieved": round(pre_bytes / preprocess_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                    "frac": round(pre_bytes / preprocess_ms / 1e6 / HBM_PEAK_GBS, 4)}},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "setup_s": round(setup_s, 1),

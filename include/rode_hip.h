@@ -384,6 +384,18 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
                                float scale, float* d_out, float* d_probs, const rode_hip_plans* plans, void* stream);
 
 /*
+ * The same for `heads` problems on one pattern in one launch (the heads of an attention
+ * layer share their mask): d_q and d_out hold heads x M x d elements, d_k and d_v
+ * heads x N x d, d_probs (if not NULL) heads x nnz, each head after the other.  N: columns
+ * of the pattern, nnz: its nonzeros (they say where the next head's operands start).  The
+ * pattern, its values and the plan are read by every head.
+ */
+int rode_hip_attention_forward_batched(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,
+                                       const int* d_column_indices, const float* d_values, const void* d_q, const void* d_k,
+                                       const void* d_v, float scale, float* d_out, float* d_probs, const rode_hip_plans* plans,
+                                       void* stream);
+
+/*
  * The gradient of rode_hip_attention_forward in two kernels (no counterpart in the
  * reference, whose op is forward-only, RoDe_SDDMM/rode_sddmm.py:194-248).  With g the
  * gradient of the loss with respect to out:
@@ -397,7 +409,9 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
  *   dtype        RODE_DENSE_F32 or RODE_DENSE_F16: element type of q, k and v (g, out and the
  *                three gradients are float; with fp16 operands g is rounded to fp16 relative to
  *                the largest magnitude of its row where it meets rows of v)
- *   M, N         rows / columns of the pattern; d: 32, 64 or 128
+ *   heads        problems on the one pattern (1: a single head); every operand below except
+ *                the pattern, d_t_slot and the plans holds `heads` arrays, one after the other
+ *   M, N, nnz    rows / columns / nonzeros of the pattern; d: 32, 64 or 128
  *   d_probs      float [nnz]: p as rode_hip_attention_forward wrote it
  *   d_out        float [M x d]: the forward result
  *   d_t_slot     int [nnz]: for every nonzero its index in the transposed pattern, i.e. the
@@ -407,14 +421,14 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
  *                plan with at least 2048 groups with a run is used, as in the forward call)
  * Rows (columns) without nonzeros get zero gradients.  Both calls queue on `stream`.
  */
-int rode_hip_attention_backward_rows(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
-                                     const float* d_values, const float* d_probs, const float* d_grad_out,
-                                     const float* d_out, const void* d_k, const void* d_v, float scale,
+int rode_hip_attention_backward_rows(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,
+                                     const int* d_column_indices, const float* d_values, const float* d_probs,
+                                     const float* d_grad_out, const float* d_out, const void* d_k, const void* d_v, float scale,
                                      const int* d_t_slot, float* d_grad_q, float* d_pairs, const rode_hip_plans* plans,
                                      void* stream);
-int rode_hip_attention_backward_cols(int dtype, int N, int d, const int* d_t_row_offsets, const int* d_t_column_indices,
-                                     const float* d_pairs, const float* d_grad_out, const void* d_q, float* d_grad_k,
-                                     float* d_grad_v, const rode_hip_plans* t_plans, void* stream);
+int rode_hip_attention_backward_cols(int dtype, int heads, int M, int N, int nnz, int d, const int* d_t_row_offsets,
+                                     const int* d_t_column_indices, const float* d_pairs, const float* d_grad_out,
+                                     const void* d_q, float* d_grad_k, float* d_grad_v, const rode_hip_plans* t_plans, void* stream);
 
 /*
  * The transposed pattern of a CSR matrix (M rows, N columns, nnz nonzeros): what the

@@ -126,44 +126,52 @@ FUSED_MAX_ROW = 16384
 
 
 def _attention_call(csr, values, q, k, v, scale, want_probs):
+    """q: (m, d) or (heads, m, d), k and v alike; returns out of q's shape (float32) and the
+    probabilities, (nnz,) or (heads, nnz), or None."""
     lib = _lib.load()
-    m, d = q.shape
-    probs = torch.empty_like(values) if want_probs else None
-    if values.numel() == 0:  # no nonzeros: nothing attends to anything
-        return torch.zeros((m, d), dtype=torch.float32, device=q.device), probs
-    out = torch.empty((m, d), dtype=torch.float32, device=q.device)
+    heads = q.shape[0] if q.dim() == 3 else 1
+    m, d = q.shape[-2:]
+    nnz = values.numel()
+    lead = q.shape[:-2]
+    probs = torch.empty(lead + (nnz,), dtype=torch.float32, device=q.device) if want_probs else None
+    if nnz == 0:  # no nonzeros: nothing attends to anything
+        return torch.zeros(lead + (m, d), dtype=torch.float32, device=q.device), probs
+    out = torch.empty(lead + (m, d), dtype=torch.float32, device=q.device)
     plans = rode_sddmm_hip.plans_struct(csr.plan if isinstance(csr.plan, rode_sddmm_hip.GroupPlan) else None)
     with torch.cuda.device(q.device):
-        code = lib.rode_hip_attention_forward(
-            _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"], m, d, csr.row_offsets.data_ptr(),
-            csr.column_indices.data_ptr(), values.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale),
-            out.data_ptr(), probs.data_ptr() if want_probs else None, ctypes.byref(plans),
+        code = lib.rode_hip_attention_forward_batched(
+            _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"], heads, m, csr.n, nnz, d,
+            csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), values.data_ptr(), q.data_ptr(), k.data_ptr(),
+            v.data_ptr(), float(scale), out.data_ptr(), probs.data_ptr() if want_probs else None, ctypes.byref(plans),
             torch.cuda.current_stream(q.device).cuda_stream)
-    _lib.check(code, "rode_hip_attention_forward")
+    _lib.check(code, "rode_hip_attention_forward_batched")
     return out, probs
 
 
 def _attention_backward_call(csr, csr_t, t_slot, probs, g, out, q, k, v, scale):
     """(dq, dk, dv) in float32 through the two gradient kernels: the row pass over the
-    pattern, the column pass over the transposed pattern."""
+    pattern, the column pass over the transposed pattern; every head in the same two launches."""
     lib = _lib.load()
-    m, d = q.shape
-    n = k.shape[0]
+    heads = q.shape[0] if q.dim() == 3 else 1
+    m, d = q.shape[-2:]
+    n = k.shape[-2]
+    nnz = csr.nnz
     kind = _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"]
-    dq = torch.empty((m, d), dtype=torch.float32, device=q.device)
-    dk = torch.empty((n, d), dtype=torch.float32, device=q.device)
-    dv = torch.empty((n, d), dtype=torch.float32, device=q.device)
+    dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    dk = torch.empty(k.shape, dtype=torch.float32, device=q.device)
+    dv = torch.empty(v.shape, dtype=torch.float32, device=q.device)
     pairs = torch.empty(2 * probs.numel(), dtype=torch.float32, device=q.device)
     group = lambda c: c.plan if isinstance(c.plan, rode_sddmm_hip.GroupPlan) else None
     plans, plans_t = rode_sddmm_hip.plans_struct(group(csr)), rode_sddmm_hip.plans_struct(group(csr_t))
     with torch.cuda.device(q.device):
         s = torch.cuda.current_stream(q.device).cuda_stream
         _lib.check(lib.rode_hip_attention_backward_rows(
-            kind, m, d, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
+            kind, heads, m, n, nnz, d, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
             probs.data_ptr(), g.data_ptr(), out.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale), t_slot.data_ptr(),
             dq.data_ptr(), pairs.data_ptr(), ctypes.byref(plans), s), "rode_hip_attention_backward_rows")
         _lib.check(lib.rode_hip_attention_backward_cols(
-            kind, n, d, csr_t.row_offsets.data_ptr(), csr_t.column_indices.data_ptr(), pairs.data_ptr(), g.data_ptr(), q.data_ptr(), dk.data_ptr(), dv.data_ptr(), ctypes.byref(plans_t), s),
+            kind, heads, m, n, nnz, d, csr_t.row_offsets.data_ptr(), csr_t.column_indices.data_ptr(), pairs.data_ptr(),
+            g.data_ptr(), q.data_ptr(), dk.data_ptr(), dv.data_ptr(), ctypes.byref(plans_t), s),
             "rode_hip_attention_backward_cols")
     return dq, dk, dv
 
@@ -213,25 +221,39 @@ class FusedAttentionFunction(torch.autograd.Function):
             return (None, dq.to(q.dtype) if ctx.needs_input_grad[1] else None,
                     dk.to(k.dtype) if ctx.needs_input_grad[2] else None,
                     dv.to(v.dtype) if ctx.needs_input_grad[3] else None, None)
-        if ctx.needs_input_grad[3]:
+        need = ctx.needs_input_grad
+        if q.dim() == 3:  # the chain of separate kernels takes one head at a time
+            per_head = [FusedAttentionFunction._chained_backward(csr, csr_t, perm, scale, need, probs[h], g[h], q[h], k[h], v[h])
+                        for h in range(q.shape[0])]
+            dq, dk, dv = (torch.stack(t) if t[0] is not None else None for t in zip(*per_head))
+        else:
+            dq, dk, dv = FusedAttentionFunction._chained_backward(csr, csr_t, perm, scale, need, probs, g, q, k, v)
+        return None, dq, dk, dv, None
+
+    @staticmethod
+    def _chained_backward(csr, csr_t, perm, scale, need, probs, g, q, k, v):
+        dq = dk = dv = None
+        if need[3]:
             dv = _spmm(csr_t, rode_sddmm_hip.permute(probs, perm), g).to(v.dtype)
-        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+        if need[1] or need[2]:
             dp = _sddmm(csr, csr.ones(), g, v.float())  # (g is float32: both operands of an SDDMM share a type)
             ds = _softmax_call("rode_hip_csr_softmax_backward_f32", csr.row_offsets, probs, dp, scale)
             ds.mul_(csr.values)  # scores are values (.) (q k^T)
             # float16 operands are gathered as they are (the sums are float32 either way)
-            if ctx.needs_input_grad[1]:
+            if need[1]:
                 dq = _spmm(csr, ds, k).to(q.dtype)
-            if ctx.needs_input_grad[2]:
+            if need[2]:
                 dk = _spmm(csr_t, rode_sddmm_hip.permute(ds, perm), q).to(k.dtype)
-        return None, dq, dk, dv, None
+        return dq, dk, dv
 
 
 def sparse_attention(mask, q, k, v, scale=None, fused="auto"):
     """softmax(scale * mask (.) (q k^T)) v on the sparsity pattern of ``mask`` (a
     ``RoDeCSR``; its values multiply the scores, use 1 for a pure mask).  q is (m, d),
     k is (n, d) with d in {32, 64, 128}; v is (n, dv) with dv a multiple of 32.  One
-    row decomposition serves all three kernels; differentiable in q, k and v.
+    row decomposition serves all three kernels; differentiable in q, k and v.  With a
+    leading dimension - q (heads, m, d), k and v (heads, n, d) - every head uses the one
+    mask, and the fused kernels take all heads in one launch.
 
     ``fused``: "auto" runs the forward pass as one kernel when it applies (dv == d, q, k
     and v of one dtype, float32 mask values, no row longer than ``FUSED_MAX_ROW``) and as
@@ -240,20 +262,22 @@ def sparse_attention(mask, q, k, v, scale=None, fused="auto"):
     from .rode_sddmm import rode_sddmm
     from .rode_spmm import rode_spmm
     if scale is None:
-        scale = q.shape[1] ** -0.5
+        scale = q.shape[-1] ** -0.5
     if fused not in (True, False, "auto"):
         raise ValueError(f'fused must be True, False or "auto", got {fused!r}')
+    if q.dim() not in (2, 3) or k.dim() != q.dim() or v.dim() != q.dim():
+        raise ValueError("q, k and v must all be 2-D, or all 3-D with the heads first")
+    if q.dim() == 3 and not (q.shape[0] == k.shape[0] == v.shape[0]):
+        raise ValueError(f"q, k and v must have the same number of heads, got {q.shape[0]}, {k.shape[0]}, {v.shape[0]}")
     if fused:
         why = None
-        if q.dim() != 2 or k.dim() != 2 or v.dim() != 2:
-            why = "q, k and v must be 2-D"
-        elif q.shape[1] not in (32, 64, 128) or k.shape[1] != q.shape[1] or v.shape[1] != q.shape[1]:
+        if q.shape[-1] not in (32, 64, 128) or k.shape[-1] != q.shape[-1] or v.shape[-1] != q.shape[-1]:
             why = "q, k and v must have the same width, 32, 64 or 128"
         elif not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.float32, torch.float16)):
             why = "q, k and v must share one dtype, float32 or float16"
         elif mask.values.dtype != torch.float32:
             why = "the mask values must be float32"
-        elif q.shape[0] != mask.m or k.shape[0] != mask.n or v.shape[0] != mask.n:
+        elif q.shape[-2] != mask.m or k.shape[-2] != mask.n or v.shape[-2] != mask.n:
             why = f"q must have {mask.m} rows, k and v {mask.n}"
         elif not (q.is_cuda and q.device == mask.device and k.device == q.device and v.device == q.device):
             why = f"q, k and v must be on {mask.device}"
@@ -263,6 +287,8 @@ def sparse_attention(mask, q, k, v, scale=None, fused="auto"):
             return FusedAttentionFunction.apply(mask, q, k, v, scale)
         if fused is True:
             raise ValueError(f"the fused attention kernel does not apply: {why}")
+    if q.dim() == 3:  # the three kernels take one head at a time
+        return torch.stack([sparse_attention(mask, q[h], k[h], v[h], scale, False) for h in range(q.shape[0])])
     scores = rode_sddmm(mask, q, k)
     probs = csr_row_softmax(mask, scores, scale)
     return rode_spmm(mask, v, values=probs)

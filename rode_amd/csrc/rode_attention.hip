@@ -47,8 +47,10 @@ template <typename T, int D, bool WRITE_P>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                       const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, float scale,
-                      float* __restrict__ out, float* probs, RowOwners owners)
+                      float* __restrict__ out, float* probs, RowOwners owners, HeadStrides heads)
 {
+    q = of_head(q, heads.rows), k = of_head(k, heads.cols), v = of_head(v, heads.cols);
+    out = of_head(out, heads.rows), probs = of_head(probs, heads.nnz);
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
@@ -163,8 +165,10 @@ __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu
 attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
                        const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ q,
                        const T* __restrict__ k, const T* __restrict__ v, float scale, float* __restrict__ out,
-                       float* probs)
+                       float* probs, HeadStrides heads)
 {
+    q = of_head(q, heads.rows), k = of_head(k, heads.cols), v = of_head(v, heads.cols);
+    out = of_head(out, heads.rows), probs = of_head(probs, heads.nnz);
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
@@ -333,12 +337,14 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
 }
 
 template <typename T, int D>
-hipError_t launch_rows(int M, const int* row_ptr, const int* col, const float* val, const T* q, const T* k, const T* v,
-                       float scale, float* out, float* probs, PlanRef plan, hipStream_t stream)
+hipError_t launch_rows(int nheads, int M, int N, int nnz, const int* row_ptr, const int* col, const float* val, const T* q,
+                       const T* k, const T* v, float scale, float* out, float* probs, PlanRef plan, hipStream_t stream)
 {
     long long wgs = ((long long)M + kWavesPerWg - 1) / kWavesPerWg;
     wgs = (wgs + kXcds - 1) / kXcds * kXcds;
-    if (wgs * kWgThreads >= (1ll << 32)) return hipErrorInvalidConfiguration;
+    if (wgs * kWgThreads >= (1ll << 32) || nheads > 65535) return hipErrorInvalidConfiguration;
+    HeadStrides heads;
+    heads.rows = (size_t)M * D, heads.cols = (size_t)N * D, heads.nnz = (size_t)nnz;
     // a group plan is used when a wave per group fills the GPU
     RowOwners owners;
     const bool grouped = plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] >= kGroupWaveEach;
@@ -347,45 +353,49 @@ hipError_t launch_rows(int M, const int* row_ptr, const int* col, const float* v
         owners.n_groups = plan.group_counts[0];
     }
     if (!(grouped && plan.group_counts[2] == 0)) { // (else every row is in a group)
+        const dim3 grid((unsigned)wgs, (unsigned)nheads);
         if (probs)
-            attention_rows_kernel<T, D, true><<<(int)wgs, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out,
-                                                                                   probs, owners);
+            attention_rows_kernel<T, D, true><<<grid, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out, probs,
+                                                                               owners, heads);
         else
-            attention_rows_kernel<T, D, false><<<(int)wgs, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out,
-                                                                                    probs, owners);
+            attention_rows_kernel<T, D, false><<<grid, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out, probs,
+                                                                                owners, heads);
     }
     if (grouped) {
         int gw = (owners.n_groups + kWavesPerWg - 1) / kWavesPerWg;
         gw = (gw + kXcds - 1) / kXcds * kXcds;
+        const dim3 grid((unsigned)gw, (unsigned)nheads);
         if (probs)
-            attention_group_kernel<T, D, true><<<gw, kWgThreads, 0, stream>>>(owners.n_groups, owners.groups, row_ptr, col, val,
-                                                                              q, k, v, scale, out, probs);
+            attention_group_kernel<T, D, true><<<grid, kWgThreads, 0, stream>>>(owners.n_groups, owners.groups, row_ptr, col, val,
+                                                                                q, k, v, scale, out, probs, heads);
         else
-            attention_group_kernel<T, D, false><<<gw, kWgThreads, 0, stream>>>(owners.n_groups, owners.groups, row_ptr, col,
-                                                                               val, q, k, v, scale, out, probs);
+            attention_group_kernel<T, D, false><<<grid, kWgThreads, 0, stream>>>(owners.n_groups, owners.groups, row_ptr, col,
+                                                                                 val, q, k, v, scale, out, probs, heads);
     }
     return hipGetLastError();
 }
 
 } // namespace
 
-// d: width of q, k and v rows (32, 64 or 128).  probs: NULL or nnz floats.
+// nheads problems on one pattern (q, out: [nheads][M][d]; k, v: [nheads][N][d]; probs: NULL or
+// [nheads][nnz]); d: width of q, k and v rows (32, 64 or 128).
 template <typename T>
-hipError_t attention_launch(int M, int d, const int* row_ptr, const int* col, const float* val, const T* q, const T* k,
-                            const T* v, float scale, float* out, float* probs, PlanRef plan, hipStream_t stream)
+hipError_t attention_launch(int nheads, int M, int N, int nnz, int d, const int* row_ptr, const int* col, const float* val,
+                            const T* q, const T* k, const T* v, float scale, float* out, float* probs, PlanRef plan,
+                            hipStream_t stream)
 {
-    if (M <= 0) return hipSuccess;
+    if (M <= 0 || nheads <= 0) return hipSuccess;
     switch (d) {
-    case 32: return launch_rows<T, 32>(M, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
-    case 64: return launch_rows<T, 64>(M, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
-    case 128: return launch_rows<T, 128>(M, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
+    case 32: return launch_rows<T, 32>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
+    case 64: return launch_rows<T, 64>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
+    case 128: return launch_rows<T, 128>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
-template hipError_t attention_launch<float>(int, int, const int*, const int*, const float*, const float*, const float*,
-                                            const float*, float, float*, float*, PlanRef, hipStream_t);
-template hipError_t attention_launch<__half>(int, int, const int*, const int*, const float*, const __half*, const __half*,
-                                             const __half*, float, float*, float*, PlanRef, hipStream_t);
+template hipError_t attention_launch<float>(int, int, int, int, int, const int*, const int*, const float*, const float*,
+                                            const float*, const float*, float, float*, float*, PlanRef, hipStream_t);
+template hipError_t attention_launch<__half>(int, int, int, int, int, const int*, const int*, const float*, const __half*,
+                                             const __half*, const __half*, float, float*, float*, PlanRef, hipStream_t);
 
 } // namespace rode

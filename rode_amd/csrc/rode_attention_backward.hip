@@ -100,8 +100,10 @@ attention_backward_rows_kernel(int M, const int* __restrict__ row_ptr, const int
                                const float* __restrict__ val, const float* __restrict__ probs,
                                const float* __restrict__ g, const float* __restrict__ out, const T* __restrict__ k,
                                const T* __restrict__ v, float scale, const int* __restrict__ t_slot,
-                               float* __restrict__ dq, float2* __restrict__ pz, RowOwners owners)
+                               float* __restrict__ dq, float2* __restrict__ pz, RowOwners owners, HeadStrides heads)
 {
+    probs = of_head(probs, heads.nnz), g = of_head(g, heads.rows), out = of_head(out, heads.rows);
+    k = of_head(k, heads.cols), v = of_head(v, heads.cols), dq = of_head(dq, heads.rows), pz = of_head(pz, heads.nnz);
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
     constexpr bool kScaled = std::is_same<T, __half>::value;
@@ -176,8 +178,10 @@ attention_backward_group_kernel(int n_groups, const RowGroup* __restrict__ group
                                 const float* __restrict__ probs, const float* __restrict__ g,
                                 const float* __restrict__ out, const T* __restrict__ k, const T* __restrict__ v,
                                 float scale, const int* __restrict__ t_slot, float* __restrict__ dq,
-                                float2* __restrict__ pz)
+                                float2* __restrict__ pz, HeadStrides heads)
 {
+    probs = of_head(probs, heads.nnz), g = of_head(g, heads.rows), out = of_head(out, heads.rows);
+    k = of_head(k, heads.cols), v = of_head(v, heads.cols), dq = of_head(dq, heads.rows), pz = of_head(pz, heads.nnz);
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
     constexpr bool kScaled = std::is_same<T, __half>::value;
@@ -408,8 +412,12 @@ template <typename T, int D>
 __global__ void __launch_bounds__(kWgThreads)
 attention_backward_cols_kernel(int N, const int* __restrict__ t_row_ptr, const int* __restrict__ t_col,
                                const float2* __restrict__ pz, const float* __restrict__ g,
-                               const T* __restrict__ q, float* __restrict__ dk, float* __restrict__ dv, RowOwners owners)
+                               const T* __restrict__ q, float* __restrict__ dk, float* __restrict__ dv, RowOwners owners,
+                               HeadStrides heads)
 {
+    // (rows / cols of the pattern itself: g and q have a row per row of it, dk and dv one per column)
+    pz = of_head(pz, heads.nnz), g = of_head(g, heads.rows), q = of_head(q, heads.rows);
+    dk = of_head(dk, heads.cols), dv = of_head(dv, heads.cols);
     constexpr int LPR = D / 4, G = kWave / LPR;
     __shared__ __attribute__((aligned(16))) int lds_r[kWavesPerWg * kWave];
     __shared__ __attribute__((aligned(16))) float lds_p[kWavesPerWg * kWave];
@@ -460,9 +468,11 @@ attention_backward_cols_kernel(int N, const int* __restrict__ t_row_ptr, const i
 template <typename T, int D>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_backward_cols_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ t_row_ptr,
-                                     const int* __restrict__ t_col, const float2* __restrict__ pz, const float* __restrict__ g, const T* __restrict__ q,
-                                     float* __restrict__ dk, float* __restrict__ dv)
+                                     const int* __restrict__ t_col, const float2* __restrict__ pz, const float* __restrict__ g,
+                                     const T* __restrict__ q, float* __restrict__ dk, float* __restrict__ dv, HeadStrides heads)
 {
+    pz = of_head(pz, heads.nnz), g = of_head(g, heads.rows), q = of_head(q, heads.rows);
+    dk = of_head(dk, heads.cols), dv = of_head(dv, heads.cols);
     constexpr int LPR = D / 4, G = kWave / LPR, R = kGroupRows;
     __shared__ __attribute__((aligned(16))) int lds_r[kWavesPerWg][R][kWave];
     __shared__ __attribute__((aligned(16))) float lds_p[kWavesPerWg][R][kWave];
@@ -608,82 +618,89 @@ inline bool use_groups(const PlanRef& plan, RowOwners& owners)
 }
 
 template <typename T, int D>
-hipError_t launch_rows(int M, const int* row_ptr, const int* col, const float* val, const float* probs, const float* g,
-                       const float* out, const T* k, const T* v, float scale, const int* t_slot, float* dq, float* pz,
-                       PlanRef plan, hipStream_t stream)
+hipError_t launch_rows(HeadStrides heads, int nheads, int M, const int* row_ptr, const int* col, const float* val,
+                       const float* probs, const float* g, const float* out, const T* k, const T* v, float scale,
+                       const int* t_slot, float* dq, float* pz, PlanRef plan, hipStream_t stream)
 {
     const int wgs = wave_grid(M);
-    if (wgs < 0) return hipErrorInvalidConfiguration;
+    if (wgs < 0 || nheads > 65535) return hipErrorInvalidConfiguration;
     RowOwners owners;
     const bool grouped = use_groups(plan, owners);
     float2* pairs = reinterpret_cast<float2*>(pz);
     if (!(grouped && plan.group_counts[2] == 0)) // (else every row is in a group)
-        attention_backward_rows_kernel<T, D><<<wgs, kWgThreads, 0, stream>>>(M, row_ptr, col, val, probs, g, out, k, v,
-                                                                              scale, t_slot, dq, pairs, owners);
+        attention_backward_rows_kernel<T, D><<<dim3(wgs, nheads), kWgThreads, 0, stream>>>(M, row_ptr, col, val, probs, g, out, k, v,
+                                                                                            scale, t_slot, dq, pairs, owners, heads);
     if (grouped)
-        attention_backward_group_kernel<T, D><<<wave_grid(owners.n_groups), kWgThreads, 0, stream>>>(
-            owners.n_groups, owners.groups, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pairs);
+        attention_backward_group_kernel<T, D><<<dim3(wave_grid(owners.n_groups), nheads), kWgThreads, 0, stream>>>(
+            owners.n_groups, owners.groups, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pairs, heads);
     return hipGetLastError();
 }
 
 template <typename T, int D>
-hipError_t launch_cols(int N, const int* t_row_ptr, const int* t_col, const float* pz, const float* g,
-                       const T* q, float* dk, float* dv, PlanRef plan, hipStream_t stream)
+hipError_t launch_cols(HeadStrides heads, int nheads, int N, const int* t_row_ptr, const int* t_col, const float* pz,
+                       const float* g, const T* q, float* dk, float* dv, PlanRef plan, hipStream_t stream)
 {
     const int wgs = wave_grid(N);
-    if (wgs < 0) return hipErrorInvalidConfiguration;
+    if (wgs < 0 || nheads > 65535) return hipErrorInvalidConfiguration;
     RowOwners owners;
     const bool grouped = use_groups(plan, owners);
     const float2* pairs = reinterpret_cast<const float2*>(pz);
     if (!(grouped && plan.group_counts[2] == 0))
-        attention_backward_cols_kernel<T, D><<<wgs, kWgThreads, 0, stream>>>(N, t_row_ptr, t_col, pairs, g, q, dk, dv, owners);
+        attention_backward_cols_kernel<T, D><<<dim3(wgs, nheads), kWgThreads, 0, stream>>>(N, t_row_ptr, t_col, pairs, g, q, dk, dv,
+                                                                                            owners, heads);
     if (grouped)
-        attention_backward_cols_group_kernel<T, D><<<wave_grid(owners.n_groups), kWgThreads, 0, stream>>>(
-            owners.n_groups, owners.groups, t_row_ptr, t_col, pairs, g, q, dk, dv);
+        attention_backward_cols_group_kernel<T, D><<<dim3(wave_grid(owners.n_groups), nheads), kWgThreads, 0, stream>>>(
+            owners.n_groups, owners.groups, t_row_ptr, t_col, pairs, g, q, dk, dv, heads);
     return hipGetLastError();
 }
 
 } // namespace
 
-// d: width of q, k, v, g and out (32, 64 or 128).  pz: 2 * nnz floats, the pairs (p, dz) in the
-// order of the transposed pattern; t_slot: for every nonzero, its slot there.
+// nheads problems on one pattern of M rows, N columns and nnz nonzeros (operands head after
+// head); d: width of q, k, v, g and out (32, 64 or 128).  pz: nheads x 2 * nnz floats, the pairs
+// (p, dz) in the order of the transposed pattern; t_slot: for every nonzero, its slot there.
 template <typename T>
-hipError_t attention_backward_rows_launch(int M, int d, const int* row_ptr, const int* col, const float* val,
-                                          const float* probs, const float* g, const float* out, const T* k, const T* v,
-                                          float scale, const int* t_slot, float* dq, float* pz, PlanRef plan,
+hipError_t attention_backward_rows_launch(int nheads, int M, int N, int nnz, int d, const int* row_ptr, const int* col,
+                                          const float* val, const float* probs, const float* g, const float* out, const T* k,
+                                          const T* v, float scale, const int* t_slot, float* dq, float* pz, PlanRef plan,
                                           hipStream_t stream)
 {
-    if (M <= 0) return hipSuccess;
+    if (M <= 0 || nheads <= 0) return hipSuccess;
+    HeadStrides heads;
+    heads.rows = (size_t)M * d, heads.cols = (size_t)N * d, heads.nnz = (size_t)nnz;
     switch (d) {
-    case 32: return launch_rows<T, 32>(M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
-    case 64: return launch_rows<T, 64>(M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
-    case 128: return launch_rows<T, 128>(M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
+    case 32: return launch_rows<T, 32>(heads, nheads, M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
+    case 64: return launch_rows<T, 64>(heads, nheads, M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
+    case 128: return launch_rows<T, 128>(heads, nheads, M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
 template <typename T>
-hipError_t attention_backward_cols_launch(int N, int d, const int* t_row_ptr, const int* t_col, const float* pz,
-                                          const float* g, const T* q, float* dk, float* dv, PlanRef plan, hipStream_t stream)
+hipError_t attention_backward_cols_launch(int nheads, int M, int N, int nnz, int d, const int* t_row_ptr, const int* t_col,
+                                          const float* pz, const float* g, const T* q, float* dk, float* dv, PlanRef plan,
+                                          hipStream_t stream)
 {
-    if (N <= 0) return hipSuccess;
+    if (N <= 0 || nheads <= 0) return hipSuccess;
+    HeadStrides heads;
+    heads.rows = (size_t)M * d, heads.cols = (size_t)N * d, heads.nnz = (size_t)nnz;
     switch (d) {
-    case 32: return launch_cols<T, 32>(N, t_row_ptr, t_col, pz, g, q, dk, dv, plan, stream);
-    case 64: return launch_cols<T, 64>(N, t_row_ptr, t_col, pz, g, q, dk, dv, plan, stream);
-    case 128: return launch_cols<T, 128>(N, t_row_ptr, t_col, pz, g, q, dk, dv, plan, stream);
+    case 32: return launch_cols<T, 32>(heads, nheads, N, t_row_ptr, t_col, pz, g, q, dk, dv, plan, stream);
+    case 64: return launch_cols<T, 64>(heads, nheads, N, t_row_ptr, t_col, pz, g, q, dk, dv, plan, stream);
+    case 128: return launch_cols<T, 128>(heads, nheads, N, t_row_ptr, t_col, pz, g, q, dk, dv, plan, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
-template hipError_t attention_backward_rows_launch<float>(int, int, const int*, const int*, const float*, const float*,
-                                                          const float*, const float*, const float*, const float*, float,
-                                                          const int*, float*, float*, PlanRef, hipStream_t);
-template hipError_t attention_backward_rows_launch<__half>(int, int, const int*, const int*, const float*, const float*,
-                                                           const float*, const float*, const __half*, const __half*, float,
-                                                           const int*, float*, float*, PlanRef, hipStream_t);
-template hipError_t attention_backward_cols_launch<float>(int, int, const int*, const int*, const float*, const float*,
-                                                          const float*, float*, float*, PlanRef, hipStream_t);
-template hipError_t attention_backward_cols_launch<__half>(int, int, const int*, const int*, const float*, const float*,
-                                                           const __half*, float*, float*, PlanRef, hipStream_t);
+template hipError_t attention_backward_rows_launch<float>(int, int, int, int, int, const int*, const int*, const float*,
+                                                          const float*, const float*, const float*, const float*, const float*,
+                                                          float, const int*, float*, float*, PlanRef, hipStream_t);
+template hipError_t attention_backward_rows_launch<__half>(int, int, int, int, int, const int*, const int*, const float*,
+                                                           const float*, const float*, const float*, const __half*,
+                                                           const __half*, float, const int*, float*, float*, PlanRef, hipStream_t);
+template hipError_t attention_backward_cols_launch<float>(int, int, int, int, int, const int*, const int*, const float*,
+                                                          const float*, const float*, float*, float*, PlanRef, hipStream_t);
+template hipError_t attention_backward_cols_launch<__half>(int, int, int, int, int, const int*, const int*, const float*,
+                                                           const float*, const __half*, float*, float*, PlanRef, hipStream_t);
 
 } // namespace rode

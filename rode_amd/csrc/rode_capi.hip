@@ -353,33 +353,6 @@ int rode_hip_csr_softmax_backward_f32(int M, const int* d_row_offsets, const flo
     return rode::csr_softmax_backward_launch(M, d_row_offsets, d_p, d_dp, d_ds, scale, as_stream(stream));
 }
 
-int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
-                               const float* d_values, const void* d_q, const void* d_k, const void* d_v,
-                               float scale, float* d_out, float* d_probs, const rode_hip_plans* plans, void* stream)
-{
-    if (M < 0 || !d_row_offsets) return hipErrorInvalidValue;
-    rode::PlanRef plan;
-    if (plans && plans->groups) { // only a group plan means anything to this kernel
-        rode_hip_plans only_groups = {};
-        only_groups.groups = plans->groups;
-        only_groups.group_counts = plans->group_counts;
-        if (!plan_ref(&only_groups, 0, plan) || plan.group_counts[0] != rode::row_groups(M)) return hipErrorInvalidValue;
-    }
-    if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
-    if (M > 0 && (!d_column_indices || !d_values || !d_q || !d_k || !d_v || !d_out)) return hipErrorInvalidValue;
-    if (!aligned16(d_q) || !aligned16(d_k) || !aligned16(d_v) || !aligned16(d_out)) return hipErrorInvalidValue;
-    if (dtype == RODE_DENSE_F32)
-        return rode::attention_launch<float>(M, d, d_row_offsets, d_column_indices, d_values, static_cast<const float*>(d_q),
-                                             static_cast<const float*>(d_k), static_cast<const float*>(d_v), scale, d_out,
-                                             d_probs, plan, as_stream(stream));
-    if (dtype == RODE_DENSE_F16)
-        return rode::attention_launch<__half>(M, d, d_row_offsets, d_column_indices, d_values,
-                                              static_cast<const __half*>(d_q), static_cast<const __half*>(d_k),
-                                              static_cast<const __half*>(d_v), scale, d_out, d_probs, plan,
-                                              as_stream(stream));
-    return hipErrorInvalidValue;
-}
-
 // (only a group plan means anything to the attention kernels)
 static bool group_plan_only(const rode_hip_plans* plans, int rows, rode::PlanRef& plan)
 {
@@ -390,55 +363,86 @@ static bool group_plan_only(const rode_hip_plans* plans, int rows, rode::PlanRef
     return plan_ref(&only_groups, 0, plan) && plan.group_counts[0] == rode::row_groups(rows);
 }
 
-int rode_hip_attention_backward_rows(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
-                                     const float* d_values, const float* d_probs, const float* d_grad_out,
-                                     const float* d_out, const void* d_k, const void* d_v, float scale,
-                                     const int* d_t_slot, float* d_grad_q, float* d_pairs, const rode_hip_plans* plans,
-                                     void* stream)
+int rode_hip_attention_forward_batched(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,
+                                       const int* d_column_indices, const float* d_values, const void* d_q, const void* d_k,
+                                       const void* d_v, float scale, float* d_out, float* d_probs, const rode_hip_plans* plans,
+                                       void* stream)
 {
-    if (M < 0 || !d_row_offsets) return hipErrorInvalidValue;
+    if (heads < 0 || M < 0 || N < 0 || nnz < 0 || !d_row_offsets) return hipErrorInvalidValue;
     rode::PlanRef plan;
     if (!group_plan_only(plans, M, plan)) return hipErrorInvalidValue;
     if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
-    if (M > 0 && (!d_column_indices || !d_values || !d_probs || !d_grad_out || !d_out || !d_k || !d_v || !d_t_slot || !d_grad_q ||
-                  !d_pairs))
+    if (M > 0 && heads > 0 && (!d_column_indices || !d_values || !d_q || !d_k || !d_v || !d_out)) return hipErrorInvalidValue;
+    if (!aligned16(d_q) || !aligned16(d_k) || !aligned16(d_v) || !aligned16(d_out)) return hipErrorInvalidValue;
+    if (dtype == RODE_DENSE_F32)
+        return rode::attention_launch<float>(heads, M, N, nnz, d, d_row_offsets, d_column_indices, d_values,
+                                             static_cast<const float*>(d_q), static_cast<const float*>(d_k),
+                                             static_cast<const float*>(d_v), scale, d_out, d_probs, plan, as_stream(stream));
+    if (dtype == RODE_DENSE_F16)
+        return rode::attention_launch<__half>(heads, M, N, nnz, d, d_row_offsets, d_column_indices, d_values,
+                                              static_cast<const __half*>(d_q), static_cast<const __half*>(d_k),
+                                              static_cast<const __half*>(d_v), scale, d_out, d_probs, plan, as_stream(stream));
+    return hipErrorInvalidValue;
+}
+
+int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
+                               const float* d_values, const void* d_q, const void* d_k, const void* d_v,
+                               float scale, float* d_out, float* d_probs, const rode_hip_plans* plans, void* stream)
+{
+    // (one head: nobody asks where the next head's operands start)
+    return rode_hip_attention_forward_batched(dtype, 1, M, 0, 0, d, d_row_offsets, d_column_indices, d_values, d_q, d_k, d_v,
+                                              scale, d_out, d_probs, plans, stream);
+}
+
+int rode_hip_attention_backward_rows(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,
+                                     const int* d_column_indices, const float* d_values, const float* d_probs,
+                                     const float* d_grad_out, const float* d_out, const void* d_k, const void* d_v, float scale,
+                                     const int* d_t_slot, float* d_grad_q, float* d_pairs, const rode_hip_plans* plans,
+                                     void* stream)
+{
+    if (heads < 0 || M < 0 || N < 0 || nnz < 0 || !d_row_offsets) return hipErrorInvalidValue;
+    rode::PlanRef plan;
+    if (!group_plan_only(plans, M, plan)) return hipErrorInvalidValue;
+    if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
+    if (M > 0 && heads > 0 && (!d_column_indices || !d_values || !d_probs || !d_grad_out || !d_out || !d_k || !d_v || !d_t_slot ||
+                               !d_grad_q || !d_pairs))
         return hipErrorInvalidValue;
     if (!aligned16(d_grad_out) || !aligned16(d_out) || !aligned16(d_k) || !aligned16(d_v) || !aligned16(d_grad_q) ||
         !aligned16(d_pairs))
         return hipErrorInvalidValue;
     if (dtype == RODE_DENSE_F32)
-        return rode::attention_backward_rows_launch<float>(M, d, d_row_offsets, d_column_indices, d_values, d_probs,
+        return rode::attention_backward_rows_launch<float>(heads, M, N, nnz, d, d_row_offsets, d_column_indices, d_values, d_probs,
                                                            d_grad_out, d_out, static_cast<const float*>(d_k),
                                                            static_cast<const float*>(d_v), scale, d_t_slot, d_grad_q, d_pairs,
                                                            plan, as_stream(stream));
     if (dtype == RODE_DENSE_F16)
-        return rode::attention_backward_rows_launch<__half>(M, d, d_row_offsets, d_column_indices, d_values, d_probs,
+        return rode::attention_backward_rows_launch<__half>(heads, M, N, nnz, d, d_row_offsets, d_column_indices, d_values, d_probs,
                                                             d_grad_out, d_out, static_cast<const __half*>(d_k),
                                                             static_cast<const __half*>(d_v), scale, d_t_slot, d_grad_q, d_pairs,
                                                             plan, as_stream(stream));
     return hipErrorInvalidValue;
 }
 
-int rode_hip_attention_backward_cols(int dtype, int N, int d, const int* d_t_row_offsets, const int* d_t_column_indices,
-                                     const float* d_pairs, const float* d_grad_out, const void* d_q, float* d_grad_k,
-                                     float* d_grad_v, const rode_hip_plans* t_plans, void* stream)
+int rode_hip_attention_backward_cols(int dtype, int heads, int M, int N, int nnz, int d, const int* d_t_row_offsets,
+                                     const int* d_t_column_indices, const float* d_pairs, const float* d_grad_out,
+                                     const void* d_q, float* d_grad_k, float* d_grad_v, const rode_hip_plans* t_plans, void* stream)
 {
-    if (N < 0 || !d_t_row_offsets) return hipErrorInvalidValue;
+    if (heads < 0 || M < 0 || N < 0 || nnz < 0 || !d_t_row_offsets) return hipErrorInvalidValue;
     rode::PlanRef plan;
     if (!group_plan_only(t_plans, N, plan)) return hipErrorInvalidValue;
     if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
-    if (N > 0 && (!d_t_column_indices || !d_pairs || !d_grad_out || !d_q || !d_grad_k || !d_grad_v))
+    if (N > 0 && heads > 0 && (!d_t_column_indices || !d_pairs || !d_grad_out || !d_q || !d_grad_k || !d_grad_v))
         return hipErrorInvalidValue;
     if (!aligned16(d_grad_out) || !aligned16(d_q) || !aligned16(d_grad_k) || !aligned16(d_grad_v) || !aligned16(d_pairs))
         return hipErrorInvalidValue;
     if (dtype == RODE_DENSE_F32)
-        return rode::attention_backward_cols_launch<float>(N, d, d_t_row_offsets, d_t_column_indices, d_pairs,
-                                                           d_grad_out, static_cast<const float*>(d_q), d_grad_k, d_grad_v,
-                                                           plan, as_stream(stream));
+        return rode::attention_backward_cols_launch<float>(heads, M, N, nnz, d, d_t_row_offsets, d_t_column_indices, d_pairs,
+                                                           d_grad_out, static_cast<const float*>(d_q), d_grad_k, d_grad_v, plan,
+                                                           as_stream(stream));
     if (dtype == RODE_DENSE_F16)
-        return rode::attention_backward_cols_launch<__half>(N, d, d_t_row_offsets, d_t_column_indices, d_pairs,
-                                                            d_grad_out, static_cast<const __half*>(d_q), d_grad_k, d_grad_v,
-                                                            plan, as_stream(stream));
+        return rode::attention_backward_cols_launch<__half>(heads, M, N, nnz, d, d_t_row_offsets, d_t_column_indices, d_pairs,
+                                                            d_grad_out, static_cast<const __half*>(d_q), d_grad_k, d_grad_v, plan,
+                                                            as_stream(stream));
     return hipErrorInvalidValue;
 }
 

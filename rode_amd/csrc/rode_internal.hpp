@@ -49,23 +49,26 @@ struct PlanRef {
 
 hipError_t group_plan_launch(int M, const int* row_ptr, const int* col, int* plan, hipStream_t stream);
 
-// (plan: only a group plan is used)
+// The attention kernels take nheads problems on one pattern of M rows, N columns and nnz
+// nonzeros per launch (operands head after head).  (plan: only a group plan is used)
 template <typename T>
-hipError_t attention_launch(int M, int d, const int* row_ptr, const int* col, const float* val, const T* q, const T* k,
-                            const T* v, float scale, float* out, float* probs, PlanRef plan, hipStream_t stream);
+hipError_t attention_launch(int nheads, int M, int N, int nnz, int d, const int* row_ptr, const int* col, const float* val,
+                            const T* q, const T* k, const T* v, float scale, float* out, float* probs, PlanRef plan,
+                            hipStream_t stream);
 
 // Gradient of the attention kernel (rode_attention_backward.hip): the row pass over the
 // pattern, then the column pass over the transposed pattern (plan: only a group plan is used,
-// of the pattern the pass walks).  pz: 2 * nnz floats, written by the first in the order of the
-// transposed pattern (t_slot: every nonzero's slot there), read by the second.
+// of the pattern the pass walks).  pz: nheads x 2 * nnz floats, written by the first in the
+// order of the transposed pattern (t_slot: every nonzero's slot there), read by the second.
 template <typename T>
-hipError_t attention_backward_rows_launch(int M, int d, const int* row_ptr, const int* col, const float* val,
-                                          const float* probs, const float* g, const float* out, const T* k, const T* v,
-                                          float scale, const int* t_slot, float* dq, float* pz, PlanRef plan,
+hipError_t attention_backward_rows_launch(int nheads, int M, int N, int nnz, int d, const int* row_ptr, const int* col,
+                                          const float* val, const float* probs, const float* g, const float* out, const T* k,
+                                          const T* v, float scale, const int* t_slot, float* dq, float* pz, PlanRef plan,
                                           hipStream_t stream);
 template <typename T>
-hipError_t attention_backward_cols_launch(int N, int d, const int* t_row_ptr, const int* t_col, const float* pz,
-                                          const float* g, const T* q, float* dk, float* dv, PlanRef plan, hipStream_t stream);
+hipError_t attention_backward_cols_launch(int nheads, int M, int N, int nnz, int d, const int* t_row_ptr, const int* t_col,
+                                          const float* pz, const float* g, const T* q, float* dk, float* dv, PlanRef plan,
+                                          hipStream_t stream);
 
 hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, const int* col, int* plan,
                            hipStream_t stream);

@@ -54,6 +54,19 @@ __device__ __forceinline__ bool owned_elsewhere(const RowOwners& o, int row, int
     return o.groups != nullptr && row / kGroupRows < o.n_groups && o.groups[row / kGroupRows].len > 0;
 }
 
+// Several problems on one pattern in one launch (the heads of an attention layer): blockIdx.y
+// picks the problem, whose operands start this many elements after those of problem 0.
+struct HeadStrides {
+    size_t rows = 0; // of an operand with a row of d elements per row of the pattern
+    size_t cols = 0; // of an operand with a row of d elements per column of the pattern
+    size_t nnz = 0;  // of an operand with an element per nonzero
+};
+template <typename P>
+__device__ __forceinline__ P* of_head(P* first, size_t stride)
+{
+    return first ? first + (size_t)blockIdx.y * stride : first;
+}
+
 // Aligned slot range [base, base + cnt) of one block work item; the first `mask` slots
 // belong to the previous row (unaligned start) and must not contribute.
 struct BlockItem {

@@ -278,3 +278,40 @@ def test_fused_attention_dispatch():
         autograd.FUSED_MAX_ROW = limit
     b = sparse_attention(mask, q, k, v)
     assert (a - b).abs().max().item() <= 2e-5 * max(1.0, b.abs().max().item())
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_heads_in_one_launch_match_the_loop_over_heads(half):
+    """q, k, v with a leading heads dimension over one mask: the fused kernels take all heads
+    in one launch (blockIdx.y); outputs and all three gradients equal those of one call per
+    head, bit for bit (the same kernels on the same operands), group plan and rows outside
+    groups both present."""
+    from gpu_common import DEV, make_csr
+    from rode_amd import rode_sddmm_hip, sparse_attention
+    from test_gpu_group import _window_matrix
+    rng = np.random.default_rng(5)
+    m, d, heads = 10000, 64, 3
+    n = m + 300
+    rp, col, val = _window_matrix(rng, m, n, 160, 8)
+    mask = make_csr(rp, col, rng.uniform(0.5, 1.5, len(col)).astype(np.float32), m, n, d, locality=True)
+    assert isinstance(mask.plan, rode_sddmm_hip.GroupPlan) and mask.plan.counts[1] >= 2048 and mask.plan.counts[2] > 0
+    dt = torch.float16 if half else torch.float32
+    mk = lambda r: torch.from_numpy(rng.standard_normal((heads, r, d)).astype(np.float32)).to(DEV, dt)
+    q, k, v = mk(m).requires_grad_(), mk(n).requires_grad_(), mk(n).requires_grad_()
+    w = mk(m).float()
+    out = sparse_attention(mask, q, k, v, fused=True)
+    assert out.shape == (heads, m, d)
+    (out * w).sum().backward()
+    batched = (out.detach().clone(), q.grad.clone(), k.grad.clone(), v.grad.clone())
+    for h in range(heads):
+        qh, kh, vh = (t[h].detach().clone().requires_grad_() for t in (q, k, v))
+        oh = sparse_attention(mask, qh, kh, vh, fused=True)
+        (oh * w[h]).sum().backward()
+        for got, want in zip(batched, (oh.detach(), qh.grad, kh.grad, vh.grad)):
+            assert torch.equal(got[h], want)
+    # the three separate kernels take the heads one at a time
+    chain = sparse_attention(mask, q.detach(), k.detach(), v.detach(), fused=False)
+    tol = 3e-3 if half else 5e-5
+    assert (chain - batched[0]).abs().max().item() <= tol * max(1.0, chain.abs().max().item())
+    with pytest.raises(ValueError, match="heads"):
+        sparse_attention(mask, q, k[:2], v, fused=True)
