@@ -220,17 +220,19 @@ int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_
  * bands, block structure): groups of RODE_HIP_GROUP_ROWS adjacent rows whose longest runs
  * have at least 64 columns in common, holding at least three quarters of their nonzeros,
  * and start and end within 255 columns of each other, are processed by kernels of their
- * own.  Those walk the columns the runs cover between them once, load every dense row of
- * that range once for all rows of the group (its address follows from the range, no column
- * index is read), and leave a row out at the columns outside its own run.  The other
- * kernels leave those rows out.  Same results up to the order of the fp32 additions.
+ * own.  Those walk the columns that all the runs hold once, load every dense row of that
+ * shared run once for all rows of the group (its address follows from the run, no column
+ * index is read), and then take each row's other nonzeros, the ends of its own run
+ * included, the usual way: a row never meets a dense row that it does not reference.  The
+ * other kernels leave those rows out.  Same results up to the order of the fp32 additions.
  *   d_plan       rode_hip_group_plan_bytes(M) bytes, 16-byte aligned, out
  *   h_counts     HOST int[4], out (the call waits for its kernels): [0] groups (M / 4,
  *                whole groups only), [1] groups with a run, [2] rows outside those groups
  *                (0: the other kernels have nothing to do and are not launched); the
  *                *_planned entry points need it and ignore a plan with [1] == 0
  * A group plan belongs to the pattern it was made from and excludes the other two plans.
- * SDDMM uses it for k <= 128 (fp32) / 256 (fp16) elements, SpMM for any width.
+ * SDDMM uses it for k <= 128 elements (fp32 and fp16 alike: rows of one 128-element slab; wider
+ * rows go through the list kernels, plan or not), SpMM for any width.
  */
 #define RODE_HIP_GROUP_ROWS 4
 size_t rode_hip_group_plan_bytes(int M);

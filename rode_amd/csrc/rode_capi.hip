@@ -141,10 +141,18 @@ int rode_hip_hub_plan(int M, int dense_rows, int nnz, int min_len, const int* d_
         return hipErrorInvalidValue;
     if (plan_bytes < rode_hip_hub_plan_bytes(M, dense_rows, nnz, min_len)) return hipErrorInvalidValue;
     if (M > 0 && (!d_row_offsets || (nnz > 0 && !d_column_indices))) return hipErrorInvalidValue;
-    hipError_t e = rode::hub_plan_launch(M, dense_rows, nnz, min_len, d_row_offsets, d_column_indices,
-                                         static_cast<int*>(d_plan), as_stream(stream));
-    if (e == hipSuccess) e = hipMemcpyAsync(h_counts, d_plan, 8 * sizeof(int), hipMemcpyDeviceToHost, as_stream(stream));
-    if (e == hipSuccess) e = hipStreamSynchronize(as_stream(stream));
+    // the hub rows first; once their number is known, a workgroup per hub row cuts it into pieces
+    // (and may still mark the plan unusable: the header is read again afterwards)
+    int* plan = static_cast<int*>(d_plan);
+    hipError_t e = rode::hub_plan_launch(M, dense_rows, nnz, min_len, d_row_offsets, plan, as_stream(stream));
+    for (int pass = 0; pass < 2 && e == hipSuccess; ++pass) {
+        e = hipMemcpyAsync(h_counts, d_plan, 8 * sizeof(int), hipMemcpyDeviceToHost, as_stream(stream));
+        if (e == hipSuccess) e = hipStreamSynchronize(as_stream(stream));
+        if (e == hipSuccess && pass == 0) {
+            if (h_counts[3] == 0 || h_counts[0] <= 0 || nnz == 0) break; // nothing to cut up
+            e = rode::hub_pieces_launch(h_counts[0], dense_rows, d_row_offsets, d_column_indices, plan, as_stream(stream));
+        }
+    }
     return e;
 }
 

@@ -76,7 +76,7 @@ hub_scan_kernel(int nblocks, int dense_rows, int room, int min_len, int* __restr
         plan[0] = min(total, room);
         plan[1] = hub_slabs(dense_rows);
         plan[2] = min_len;
-        plan[3] = total <= room ? 1 : 0; // (room = nnz / min_len + 1 always suffices)
+        plan[3] = total <= room ? 1 : 0; // (room = hub_room(nnz, min_len) always suffices)
         plan[4] = room;
         plan[5] = plan[6] = plan[7] = 0;
     }
@@ -131,8 +131,8 @@ hub_pieces_kernel(int dense_rows, const int* __restrict__ row_ptr, const int* __
 
 } // namespace
 
-hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, const int* col, int* plan,
-                           hipStream_t stream)
+// First the hub rows (their number is then in plan[0]), then - for that many rows - their pieces.
+hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, int* plan, hipStream_t stream)
 {
     const int room = hub_room(nnz, min_len);
     const int nblocks = (M + kHubSelectBlockRows - 1) / kHubSelectBlockRows;
@@ -140,7 +140,13 @@ hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const in
     hub_count_kernel<<<max(nblocks, 1), kWgThreads, 0, stream>>>(M, min_len, row_ptr, block_counts);
     hub_scan_kernel<<<1, kSelectThreads, 0, stream>>>(nblocks, dense_rows, room, min_len, block_counts, plan);
     hub_write_kernel<<<max(nblocks, 1), kWgThreads, 0, stream>>>(M, room, min_len, row_ptr, block_counts, plan);
-    if (room > 0 && nnz > 0) hub_pieces_kernel<<<room, kWgThreads, 0, stream>>>(dense_rows, row_ptr, col, plan);
+    return hipGetLastError();
+}
+
+hipError_t hub_pieces_launch(int hub_rows, int dense_rows, const int* row_ptr, const int* col, int* plan, hipStream_t stream)
+{
+    if (hub_rows <= 0) return hipSuccess;
+    hub_pieces_kernel<<<hub_rows, kWgThreads, 0, stream>>>(dense_rows, row_ptr, col, plan);
     return hipGetLastError();
 }
 

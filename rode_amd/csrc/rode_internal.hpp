@@ -70,8 +70,8 @@ hipError_t attention_backward_cols_launch(int nheads, int M, int N, int nnz, int
                                           const float* pz, const float* g, const T* q, float* dk, float* dv, PlanRef plan,
                                           hipStream_t stream);
 
-hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, const int* col, int* plan,
-                           hipStream_t stream);
+hipError_t hub_plan_launch(int M, int dense_rows, int nnz, int min_len, const int* row_ptr, int* plan, hipStream_t stream);
+hipError_t hub_pieces_launch(int hub_rows, int dense_rows, const int* row_ptr, const int* col, int* plan, hipStream_t stream);
 
 size_t window_plan_ints(int m2);
 size_t window_plan_rows_bytes(int m2);

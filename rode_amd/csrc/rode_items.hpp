@@ -427,7 +427,8 @@ constexpr int kHubSlabRows = 2048;
 constexpr int kHubHeaderInts = 8;
 
 __host__ __device__ inline int hub_slabs(int dense_rows) { return (dense_rows + kHubSlabRows - 1) / kHubSlabRows; }
-__host__ __device__ inline int hub_room(int nnz, int min_len) { return min_len > 0 ? nnz / min_len + 1 : 0; }
+// (a hub row has at least min_len aligned slots, up to three of which belong to the row before it)
+__host__ __device__ inline int hub_room(int nnz, int min_len) { return min_len > kVecLen ? nnz / (min_len - (kVecLen - 1)) + 1 : 0; }
 // (after the piece table: one int per 2048 rows of the matrix, scratch of the selection)
 constexpr int kHubSelectBlockRows = 2048;
 __host__ __device__ inline size_t hub_table_ints(int dense_rows, int nnz, int min_len)

@@ -218,7 +218,18 @@ def hub_plan(row_offsets, column_indices, m, n, min_len):
         _lib.check(lib.rode_hip_hub_plan(m, n, nnz, min_len, row_offsets.data_ptr(), column_indices.data_ptr(),
                                          data.data_ptr(), nbytes, ctypes.addressof(counts), _stream_handle(dev)),
                    "rode_hip_hub_plan")
-    return HubPlan(data, list(counts))
+    counts = list(counts)
+    hub_rows, slabs, room = counts[0], counts[1], counts[4]
+    if counts[3] != 0 and 0 < hub_rows < room:
+        # the call needs room for the most hub rows a matrix of this many nonzeros can have; what it
+        # found is kept in an array of its own size (header, the rows, their pieces)
+        small = torch.empty(8 + hub_rows + hub_rows * (slabs + 1), dtype=torch.int32, device=dev)
+        small[:8] = data[:8]
+        small[4] = hub_rows
+        small[8:8 + hub_rows] = data[8:8 + hub_rows]
+        small[8 + hub_rows:] = data[8 + room:8 + room + hub_rows * (slabs + 1)]
+        data, counts[4] = small, hub_rows
+    return HubPlan(data, counts)
 
 
 class GroupPlan:
