@@ -419,7 +419,7 @@ def main():
                             "gather_model_GBs": round((knnz * (8 + k * elem)) / ms / 1e6, 1),
                             "GFLOPs": round(2.0 * knnz * k / ms / 1e6, 1)}
     dominant = max(kernels, key=kernels.get)
-    traffic, traffic_note, entry = None, "no counter run of this workload under profiles/", None
+    traffic, traffic_note, entry, windowed = None, "no counter run of this workload under profiles/", None, False
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         table = json.load(open(tpath))
@@ -450,6 +450,8 @@ def main():
         clocks = dom_ms * 1e-3 * CLOCK_HZ
         busy = {"hbm": hbm["traffic_frac"], "valu": round(entry["valu_insts"] * 4 / (clocks * SIMDS), 4),
                 "lds": round(entry["lds_active_cycles"] / (clocks * CUS), 4)}
+        if windowed:  # the window kernels read every nonzero's dense row from LDS: bytes over the measured read rate
+            busy["lds"] = max(busy["lds"], round(dom["GFLOPs"] * dom_ms * 1e6 / (2.0 * k) * k * elem / dom_ms / 1e6 / LDS_PEAK_GBS, 4))
         if busy["hbm"] < 0.5:
             bound = max(busy, key=busy.get)
     knnz_dom = dom["GFLOPs"] * dom_ms * 1e6 / (2.0 * k)  # nonzeros of the dominant kernel
