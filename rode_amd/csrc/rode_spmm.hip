@@ -125,7 +125,9 @@ __device__ __forceinline__ void spmm_sum_slots(int base, int mask, int cnt, int 
 // One wave per block segment (see sddmm_block_kernel for the slot arithmetic,
 // identical at RoDeSpmm.cu:210-234).
 // (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
-template <typename T, int TN, bool EDGE>
+// WALK: 0 one wave per segment only, 1 chunks only (chunk_hint > 1), 2 either, found out here.
+// (Kernels of their own, so that the code of one way does not cost the other registers.)
+template <typename T, int TN, bool EDGE, int WALK>
 __device__ __forceinline__ void
 spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int chunk_hint, RowOwners owners,
                 const int* __restrict__ block_rows,
@@ -143,10 +145,12 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int chunk_
     // of consecutive segments from leader to leader, adds up what it finds for one row and
     // updates that row of C once (the sums of the items, not one long sum: same rounding as
     // the combine of neighbouring waves below).
-    const int chunk = chunk_hint > 0 ? chunk_hint
-                                     : block_chunk_for_grid(owned_slots != 0 && m1 >= kWalkMinSegments
-                                                                ? block_chunk(m1, block_rows, st_off) : 1, m1, nblocks);
-    if (chunk > 1) {
+    int chunk = 1;
+    if constexpr (WALK == 1) chunk = chunk_hint;
+    if constexpr (WALK == 2)
+        chunk = block_chunk_for_grid(owned_slots != 0 && m1 >= kWalkMinSegments ? block_chunk(m1, block_rows, st_off) : 1, m1,
+                                     nblocks);
+    if (WALK != 0 && chunk > 1) {
         const long long first = chunk_first_segment(bid, wave, m1, chunk);
         if (first < 0) return;
         const int last = (int)min(first + chunk, (long long)m1);
@@ -317,7 +321,7 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, RowOwner
     }
 }
 
-template <typename T, int TN, bool EDGE>
+template <typename T, int TN, bool EDGE, int WALK>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_block_kernel(int m1, int n, int owned_slots, int chunk_hint, RowOwners owners, const int* __restrict__ block_rows,
                   const int* __restrict__ st_off,
@@ -325,8 +329,8 @@ spmm_block_kernel(int m1, int n, int owned_slots, int chunk_hint, RowOwners owne
                   const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                   typename DenseVec<T>::Acc* __restrict__ C)
 {
-    spmm_block_body<T, TN, EDGE>(blockIdx.x, gridDim.x, m1, n, owned_slots, chunk_hint, owners, block_rows, st_off, row_ptr,
-                                 col, val, B, C);
+    spmm_block_body<T, TN, EDGE, WALK>(blockIdx.x, gridDim.x, m1, n, owned_slots, chunk_hint, owners, block_rows, st_off,
+                                       row_ptr, col, val, B, C);
 }
 
 template <typename T, int TN, bool EDGE>
@@ -352,8 +356,8 @@ spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, int chunk_hint,
                  const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
     if ((int)blockIdx.x < g1)
-        spmm_block_body<T, TN, EDGE>(blockIdx.x, g1, m1, n, owned_slots, chunk_hint, owners, block_rows, st_off, row_ptr, col, val,
-                                     B, C);
+        spmm_block_body<T, TN, EDGE, 2>(blockIdx.x, g1, m1, n, owned_slots, 0, owners, block_rows, st_off, row_ptr, col, val,
+                                        B, C);
     else
         spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, max(owned_slots, 0), owners, residue_rows,
                                        row_ptr, col, val,
@@ -721,8 +725,15 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     } else {
         if (block) {
             dim3 grid(g1, tiles);
-            spmm_block_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows, st_off,
-                                                                        row_ptr, col, val, B, C);
+            if (chunk_hint == 1)
+                spmm_block_kernel<T, TN, EDGE, 0><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows,
+                                                                               st_off, row_ptr, col, val, B, C);
+            else if (chunk_hint > 1)
+                spmm_block_kernel<T, TN, EDGE, 1><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows,
+                                                                               st_off, row_ptr, col, val, B, C);
+            else
+                spmm_block_kernel<T, TN, EDGE, 2><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows,
+                                                                               st_off, row_ptr, col, val, B, C);
             e = hipGetLastError();
         }
         if (residue && standard_residue) {
