@@ -85,14 +85,14 @@ int rode_hip_preprocess_host(int seg_length, int k_block, int vec_len, int M, co
  * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its GPU
  * routine allocates and frees CUB scratch on every call, _preprocess.cu:331-335).
  * Same arguments, same kernels and byte-identical results; the scan scratch is a fixed
- * array inside the library (33 KB of device memory per GPU, held until the process
+ * array inside the library (128 KB of device memory per GPU, held until the process
  * ends), so M is limited to RODE_HIP_STATIC_MAX_ROWS: a larger M returns
  * hipErrorOutOfMemory (2) before anything is launched.  The first call on a device looks
  * up the array's address (no allocation; make that call outside stream capture).  Every
  * call on one GPU uses that GPU's one array: calls that overlap in time on the same GPU
- * (different streams or host threads) race; calls queued on one stream do not.  Nothing in
- * the array has to be cleared between calls: every entry a call reads was written by
- * the same call.
+ * (different streams or host threads) race; calls queued on one stream do not.  The
+ * caller clears nothing between calls: each call begins with a fill kernel over the part
+ * of the array it is going to use (a kernel, not a memset, so the call can be captured).
  */
 #define RODE_HIP_STATIC_MAX_ROWS 4194304
 int rode_hip_preprocess_static(int seg_length, int k_block, int vec_len, int M, const int* d_row_ptr,
