@@ -73,15 +73,16 @@ def parse_args():
                         "launches of the same kernels on other arguments would enter the per-kernel averages)")
     p.add_argument("--two-streams", action="store_true",
                    help="residue kernels on a second stream (forked from / joined to the first with events)")
-    p.add_argument("--fused", choices=["no", "yes", "probs"], default="no",
-                   help="with --chain: the step is the one-kernel attention forward (rode_hip_attention_forward), "
-                        "\"probs\" also writes the probabilities a gradient needs")
+    p.add_argument("--fused", choices=["no", "yes", "probs", "scores"], default="no",
+                   help="with --chain: the step is the one-kernel attention forward (rode_hip_attention_forward_batched); "
+                        "\"probs\" also writes the probabilities a gradient needs, \"scores\" the scaled scores and every "
+                        "row's (maximum, 1 / sum) instead (what sparse_attention keeps for its gradient)")
     p.add_argument("--chain", action="store_true",
                    help="step = SDDMM scores -> row softmax -> clear C -> SpMM with those values (sparse attention)")
     p.add_argument("--heads", type=int, default=1,
-                   help="with --chain --fused yes/probs: attention heads on the one mask, all in the same launches")
+                   help="with --chain --fused yes/probs/scores: attention heads on the one mask, all in the same launches")
     p.add_argument("--train", action="store_true",
-                   help="with --chain --fused probs: the step is the attention forward with its probabilities written "
+                   help="with --chain --fused probs|scores: the step is the attention forward with what a gradient needs written "
                         "plus the two gradient kernels (rode_hip_attention_backward_rows / _cols)")
     p.add_argument("--memset-c", action="store_true",
                    help="clear all of C before SpMM (the reference's contract) instead of only the rows SpMM adds to")
@@ -228,9 +229,11 @@ def main():
 
     H = args.heads
     if H > 1 and not (args.chain and args.fused != "no"):
-        print("bench.py: --heads needs --chain --fused yes|probs", file=sys.stderr)
+        print("bench.py: --heads needs --chain --fused yes|probs|scores", file=sys.stderr)
         sys.exit(2)
     probs = torch.empty(H * nnz, device=dev) if args.chain else None
+    # (--fused scores: the forward kernel leaves scaled scores in `probs` and every row's (maximum, 1 / sum) here)
+    row_stats = torch.empty(H * m, 2, device=dev) if args.chain and args.fused == "scores" else None
     if H > 1:  # (every head its own q, k, v)
         B = torch.randn(H * n, k, device=dev, generator=gen).to(tdtype)
         L = torch.randn(H * m, k, device=dev, generator=gen).to(tdtype)
@@ -238,8 +241,8 @@ def main():
     if args.chain:
         args.no_cpu = True  # (the CPU leg and its parity gate are those of SpMM + SDDMM; the chain is checked by the tests)
     if args.train:
-        if not (args.chain and args.fused == "probs"):
-            print("bench.py: --train needs --chain --fused probs", file=sys.stderr)
+        if not (args.chain and args.fused in ("probs", "scores")):
+            print("bench.py: --train needs --chain --fused probs|scores", file=sys.stderr)
             sys.exit(2)
         csr_t, _ = csr.transpose(with_values=False)
         t_slot = csr.transposed_slots()
@@ -252,7 +255,8 @@ def main():
     def backward_rows():
         _lib.check(lib.rode_hip_attention_backward_rows(
             _lib.DENSE_CODE[args.dtype], H, m, n, nnz, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
-            csr.values.data_ptr(), probs.data_ptr(), G.data_ptr(), C.data_ptr(), B.data_ptr(), B.data_ptr(),
+            csr.values.data_ptr(), probs.data_ptr(), row_stats.data_ptr() if row_stats is not None else None, G.data_ptr(),
+            C.data_ptr(), B.data_ptr(), B.data_ptr(),
             float(k) ** -0.5, t_slot.data_ptr(), dQ.data_ptr(), pairs.data_ptr(), sddmm_plans, stream),
             "attention backward, rows")
 
@@ -277,7 +281,8 @@ def main():
         _lib.check(lib.rode_hip_attention_forward_batched(
             _lib.DENSE_CODE[args.dtype], H, m, n, nnz, k, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(),
             csr.values.data_ptr(), L.data_ptr(), B.data_ptr(), B.data_ptr(), float(k) ** -0.5, C.data_ptr(),
-            probs.data_ptr() if args.fused == "probs" else None, sddmm_plans, stream), "attention")
+            probs.data_ptr() if args.fused in ("probs", "scores") else None,
+            row_stats.data_ptr() if row_stats is not None else None, sddmm_plans, stream), "attention")
 
     def step():
         if args.chain and args.fused != "no":
@@ -398,7 +403,9 @@ def main():
             # dq, every k and v row once; column pass: row and (p, dz) read, rows of dk, dv, every g and q row once
             # forward: (col, val) read, probabilities written if asked for, q and out rows, every k and v row once
             if name.endswith("forward"):
-                ab = nnz * (8 + (4 if args.fused == "probs" else 0)) + m * k * (elem + 4) + 2 * n * k * elem
+                kept = 4 * nnz if args.fused in ("probs", "scores") else 0
+                kept += 8 * m if args.fused == "scores" else 0
+                ab = nnz * 8 + kept + m * k * (elem + 4) + 2 * n * k * elem
             elif name.endswith("rows"):
                 ab = nnz * (16 + 8) + 3 * m * k * 4 + 2 * n * k * elem
             else:
@@ -582,7 +589,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32" if elem == 4 else "f16->f32",
         "data": "synthetic",
         "config": {"workload": f"{args.workload} ({workloads.CONFIGS[args.workload][5]}), K={k}, "
-                               + (("step = fused attention forward (one kernel" + (", probabilities written)" if args.fused == "probs" else ")")
+                               + (("step = fused attention forward (one kernel" + (", probabilities written)" if args.fused == "probs" else ", scores and row statistics written)" if args.fused == "scores" else ")")
                                    + (" + gradient (row pass + column pass)" if args.train else "")
                                    if args.fused != "no" else "step = SDDMM -> row softmax -> clear C -> SpMM (chained)")
                                   if args.chain

@@ -391,11 +391,17 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
  * heads x N x d, d_probs (if not NULL) heads x nnz, each head after the other.  N: columns
  * of the pattern, nnz: its nonzeros (they say where the next head's operands start).  The
  * pattern, its values and the plan are read by every head.
+ *   d_row_stats  NULL, or float [heads x M x 2], 8-byte aligned (needs d_probs): d_probs then
+ *                receives the scaled SCORES scale * values * <q, k> instead of p, and
+ *                d_row_stats the pair (maximum score, 1 / sum of exp(score - maximum)) of
+ *                every row, so that p = exp(score - maximum) * (1 / sum).  Cheaper than
+ *                normalised probabilities (no second pass over the row);
+ *                rode_hip_attention_backward_rows takes the two arrays as they are.
  */
 int rode_hip_attention_forward_batched(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,
                                        const int* d_column_indices, const float* d_values, const void* d_q, const void* d_k,
-                                       const void* d_v, float scale, float* d_out, float* d_probs, const rode_hip_plans* plans,
-                                       void* stream);
+                                       const void* d_v, float scale, float* d_out, float* d_probs, float* d_row_stats,
+                                       const rode_hip_plans* plans, void* stream);
 
 /*
  * The gradient of rode_hip_attention_forward in two kernels (no counterpart in the
@@ -415,6 +421,8 @@ int rode_hip_attention_forward_batched(int dtype, int heads, int M, int N, int n
  *                the pattern, d_t_slot and the plans holds `heads` arrays, one after the other
  *   M, N, nnz    rows / columns / nonzeros of the pattern; d: 32, 64 or 128
  *   d_probs      float [nnz]: p as rode_hip_attention_forward wrote it
+ *   d_row_stats  NULL, or what rode_hip_attention_forward_batched wrote beside the scores
+ *                it then left in d_probs
  *   d_out        float [M x d]: the forward result
  *   d_t_slot     int [nnz]: for every nonzero its index in the transposed pattern, i.e. the
  *                inverse of the d_perm that rode_hip_csr_transpose returns
@@ -425,9 +433,9 @@ int rode_hip_attention_forward_batched(int dtype, int heads, int M, int N, int n
  */
 int rode_hip_attention_backward_rows(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,
                                      const int* d_column_indices, const float* d_values, const float* d_probs,
-                                     const float* d_grad_out, const float* d_out, const void* d_k, const void* d_v, float scale,
-                                     const int* d_t_slot, float* d_grad_q, float* d_pairs, const rode_hip_plans* plans,
-                                     void* stream);
+                                     const float* d_row_stats, const float* d_grad_out, const float* d_out, const void* d_k,
+                                     const void* d_v, float scale, const int* d_t_slot, float* d_grad_q, float* d_pairs,
+                                     const rode_hip_plans* plans, void* stream);
 int rode_hip_attention_backward_cols(int dtype, int heads, int M, int N, int nnz, int d, const int* d_t_row_offsets,
                                      const int* d_t_column_indices, const float* d_pairs, const float* d_grad_out,
                                      const void* d_q, float* d_grad_k, float* d_grad_v, const rode_hip_plans* t_plans, void* stream);

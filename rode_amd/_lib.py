@@ -44,8 +44,8 @@ SIGNATURES = {
     "rode_hip_csr_transpose": (c_int, [c_int] * 3 + [c_void_p] * 6 + [c_size_t, c_void_p]),
     "rode_hip_permute_f32": (c_int, [c_int] + [c_void_p] * 4),
     "rode_hip_attention_forward": (c_int, [c_int] * 3 + [c_void_p] * 6 + [ctypes.c_float] + [c_void_p] * 4),
-    "rode_hip_attention_forward_batched": (c_int, [c_int] * 6 + [c_void_p] * 6 + [ctypes.c_float] + [c_void_p] * 4),
-    "rode_hip_attention_backward_rows": (c_int, [c_int] * 6 + [c_void_p] * 8 + [ctypes.c_float] + [c_void_p] * 5),
+    "rode_hip_attention_forward_batched": (c_int, [c_int] * 6 + [c_void_p] * 6 + [ctypes.c_float] + [c_void_p] * 5),
+    "rode_hip_attention_backward_rows": (c_int, [c_int] * 6 + [c_void_p] * 9 + [ctypes.c_float] + [c_void_p] * 5),
     "rode_hip_attention_backward_cols": (c_int, [c_int] * 6 + [c_void_p] * 9),
 }
 

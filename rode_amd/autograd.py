@@ -125,32 +125,38 @@ def csr_row_softmax(sparse_matrix, scores, scale=1.0):
 FUSED_MAX_ROW = 16384
 
 
-def _attention_call(csr, values, q, k, v, scale, want_probs):
-    """q: (m, d) or (heads, m, d), k and v alike; returns out of q's shape (float32) and the
-    probabilities, (nnz,) or (heads, nnz), or None."""
+def _attention_call(csr, values, q, k, v, scale, keep):
+    """q: (m, d) or (heads, m, d), k and v alike; returns out of q's shape (float32) and
+    what the gradient needs: with keep == "probs" the probabilities, (nnz,) or (heads, nnz),
+    and None; with keep == "scores" the scaled scores in their place and the
+    (maximum, 1 / sum) pair of every row, (m, 2) or (heads, m, 2) - cheaper to write, and
+    p = exp(score - maximum) / sum; with keep == None two Nones."""
     lib = _lib.load()
     heads = q.shape[0] if q.dim() == 3 else 1
     m, d = q.shape[-2:]
     nnz = values.numel()
     lead = q.shape[:-2]
-    probs = torch.empty(lead + (nnz,), dtype=torch.float32, device=q.device) if want_probs else None
+    probs = torch.empty(lead + (nnz,), dtype=torch.float32, device=q.device) if keep else None
+    stats = torch.empty(lead + (m, 2), dtype=torch.float32, device=q.device) if keep == "scores" else None
     if nnz == 0:  # no nonzeros: nothing attends to anything
-        return torch.zeros(lead + (m, d), dtype=torch.float32, device=q.device), probs
+        return torch.zeros(lead + (m, d), dtype=torch.float32, device=q.device), probs, stats
     out = torch.empty(lead + (m, d), dtype=torch.float32, device=q.device)
     plans = rode_sddmm_hip.plans_struct(csr.plan if isinstance(csr.plan, rode_sddmm_hip.GroupPlan) else None)
     with torch.cuda.device(q.device):
         code = lib.rode_hip_attention_forward_batched(
             _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"], heads, m, csr.n, nnz, d,
             csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), values.data_ptr(), q.data_ptr(), k.data_ptr(),
-            v.data_ptr(), float(scale), out.data_ptr(), probs.data_ptr() if want_probs else None, ctypes.byref(plans),
+            v.data_ptr(), float(scale), out.data_ptr(), probs.data_ptr() if keep else None,
+            stats.data_ptr() if stats is not None else None, ctypes.byref(plans),
             torch.cuda.current_stream(q.device).cuda_stream)
     _lib.check(code, "rode_hip_attention_forward_batched")
-    return out, probs
+    return out, probs, stats
 
 
-def _attention_backward_call(csr, csr_t, t_slot, probs, g, out, q, k, v, scale):
+def _attention_backward_call(csr, csr_t, t_slot, probs, stats, g, out, q, k, v, scale):
     """(dq, dk, dv) in float32 through the two gradient kernels: the row pass over the
-    pattern, the column pass over the transposed pattern; every head in the same two launches."""
+    pattern, the column pass over the transposed pattern; every head in the same two launches.
+    probs, stats: what ``_attention_call`` kept (stats None: probs holds probabilities)."""
     lib = _lib.load()
     heads = q.shape[0] if q.dim() == 3 else 1
     m, d = q.shape[-2:]
@@ -167,7 +173,8 @@ def _attention_backward_call(csr, csr_t, t_slot, probs, g, out, q, k, v, scale):
         s = torch.cuda.current_stream(q.device).cuda_stream
         _lib.check(lib.rode_hip_attention_backward_rows(
             kind, heads, m, n, nnz, d, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
-            probs.data_ptr(), g.data_ptr(), out.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale), t_slot.data_ptr(),
+            probs.data_ptr(), stats.data_ptr() if stats is not None else None, g.data_ptr(), out.data_ptr(), k.data_ptr(),
+            v.data_ptr(), float(scale), t_slot.data_ptr(),
             dq.data_ptr(), pairs.data_ptr(), ctypes.byref(plans), s), "rode_hip_attention_backward_rows")
         _lib.check(lib.rode_hip_attention_backward_cols(
             kind, heads, m, n, nnz, d, csr_t.row_offsets.data_ptr(), csr_t.column_indices.data_ptr(), pairs.data_ptr(),
@@ -184,29 +191,31 @@ FUSED_BACKWARD = "auto"
 
 
 class FusedAttentionFunction(torch.autograd.Function):
-    """Forward: one kernel (``rode_hip_attention_forward``).  Backward: two kernels on the
-    saved probabilities and output (``rode_hip_attention_backward_rows`` / ``_cols``), or the
-    kernels of the chain - dP = (dOut v^T)|pattern (SDDMM), the softmax gradient, dq and dk as
-    SpMM on the pattern and its transpose, dv = P^T dOut."""
+    """Forward: one kernel (``rode_hip_attention_forward_batched``), which leaves the scaled
+    scores and every row's (maximum, 1 / sum) for the gradient.  Backward: two kernels on
+    those and the output (``rode_hip_attention_backward_rows`` / ``_cols``), or the kernels of
+    the chain - the probabilities from the scores (row softmax), dP = (dOut v^T)|pattern
+    (SDDMM), the softmax gradient, dq and dk as SpMM on the pattern and its transpose,
+    dv = P^T dOut."""
 
     @staticmethod
     def forward(ctx, csr, q, k, v, scale):
         need = any(ctx.needs_input_grad[1:4])
         values = csr.values
         q, k, v = q.detach().contiguous(), k.detach().contiguous(), v.detach().contiguous()
-        out, probs = _attention_call(csr, values, q, k, v, scale, need)
+        out, scores, stats = _attention_call(csr, values, q, k, v, scale, "scores" if need else None)
         ctx.csr, ctx.scale = csr, float(scale)
         if need:
-            ctx.save_for_backward(probs, q, k, v, out)
+            ctx.save_for_backward(scores, stats, q, k, v, out)
         return out
 
     @staticmethod
     def backward(ctx, g):
         csr, scale = ctx.csr, ctx.scale
-        probs, q, k, v, out = ctx.saved_tensors
+        scores, stats, q, k, v, out = ctx.saved_tensors
         g = g.contiguous().float()
         dq = dk = dv = None
-        if probs.numel() == 0:  # no nonzeros: the output does not depend on anything
+        if scores.numel() == 0:  # no nonzeros: the output does not depend on anything
             zeros = lambda t, need: torch.zeros_like(t) if need else None
             return (None, zeros(q, ctx.needs_input_grad[1]), zeros(k, ctx.needs_input_grad[2]),
                     zeros(v, ctx.needs_input_grad[3]), None)
@@ -217,11 +226,16 @@ class FusedAttentionFunction(torch.autograd.Function):
         if fused == "auto":
             fused = csr_t.max_row_length <= FUSED_MAX_ROW
         if fused:
-            dq, dk, dv = _attention_backward_call(csr, csr_t, csr.transposed_slots(), probs, g, out, q, k, v, scale)
+            dq, dk, dv = _attention_backward_call(csr, csr_t, csr.transposed_slots(), scores, stats, g, out, q, k, v, scale)
             return (None, dq.to(q.dtype) if ctx.needs_input_grad[1] else None,
                     dk.to(k.dtype) if ctx.needs_input_grad[2] else None,
                     dv.to(v.dtype) if ctx.needs_input_grad[3] else None, None)
         need = ctx.needs_input_grad
+        # the chain works on probabilities: the row softmax of the kept scores (the same
+        # exp(score - maximum) / sum the forward kernel used)
+        flat = scores.reshape(-1, scores.shape[-1])
+        probs = torch.stack([_softmax_call("rode_hip_csr_softmax_f32", csr.row_offsets, flat[h], None, 1.0)
+                             for h in range(flat.shape[0])]).reshape(scores.shape)
         if q.dim() == 3:  # the chain of separate kernels takes one head at a time
             per_head = [FusedAttentionFunction._chained_backward(csr, csr_t, perm, scale, need, probs[h], g[h], q[h], k[h], v[h])
                         for h in range(q.shape[0])]

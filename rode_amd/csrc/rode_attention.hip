@@ -16,10 +16,12 @@
 //     of the SpMM block kernel over the lane groups, combined by a butterfly at the end.
 // A softmax needs its whole row, so the row decomposition is not used here: rows are not
 // split across waves, and a matrix with very long rows is better served by the three
-// separate kernels (the Python layer chooses).  The probabilities are written out on
-// request (the gradient needs them): the raw scores of a row's first 1024 slots wait in
-// LDS (those of longer rows in the output array itself) until maximum and sum are known,
-// then the lanes that produced them normalise and store them.
+// separate kernels (the Python layer chooses).  What the gradient needs is written out on
+// request, in one of two forms.  Probabilities: the raw scores of a row's first 1024 slots
+// wait in LDS (those of longer rows in the output array itself) until maximum and sum are
+// known, then the lanes that produced them normalise and store them.  Scores: every score is
+// stored as it is computed, and the row's (maximum, 1 / sum) pair at the end, so that a
+// reader gets p = exp(score - maximum) * (1 / sum) without this kernel's second pass.
 #include "rode_items.hpp"
 #include "rode_units.hpp"
 #include "rode_internal.hpp"
@@ -43,14 +45,22 @@ __device__ __forceinline__ float wave_max_f(float v)
 // Raw scores of a row that wait in LDS for the row's maximum and sum (per wave).
 constexpr int kScoresKept = 1024;
 
-template <typename T, int D, bool WRITE_P>
+// What a kernel leaves behind for the gradient.
+enum Keep : int {
+    kKeepNothing = 0,
+    kKeepProbs = 1,  // probs[idx] = the probability
+    kKeepScores = 2, // probs[idx] = the scaled score, stats[row] = (row maximum, 1 / row sum)
+};
+
+template <typename T, int D, int KEEP>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restrict__ col, const float* __restrict__ val,
                       const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, float scale,
-                      float* __restrict__ out, float* probs, RowOwners owners, HeadStrides heads)
+                      float* __restrict__ out, float* probs, float2* __restrict__ stats, RowOwners owners, HeadStrides heads)
 {
+    constexpr bool WRITE_P = KEEP == kKeepProbs;
     q = of_head(q, heads.rows), k = of_head(k, heads.cols), v = of_head(v, heads.cols);
-    out = of_head(out, heads.rows), probs = of_head(probs, heads.nnz);
+    out = of_head(out, heads.rows), probs = of_head(probs, heads.nnz), stats = of_head(stats, heads.rows / D);
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
@@ -72,6 +82,7 @@ attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restr
 #pragma unroll
             for (int x = 0; x < VEC; x += 4) *reinterpret_cast<float4*>(out_lane + x) = make_float4(0.f, 0.f, 0.f, 0.f);
         }
+        if (KEEP == kKeepScores && lane == 0) stats[row] = make_float2(0.f, 0.f);
         return;
     }
 
@@ -106,6 +117,7 @@ attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restr
         if (WRITE_P && live) {
             if (slot - s < kScoresKept) my_s[slot - s] = sc; else probs[slot] = sc;
         }
+        if (KEEP == kKeepScores && live) probs[slot] = sc;
         my_p[lane] = p;
         wave_lds_sync();
         const int nlive = min(e - off, kWave);
@@ -124,6 +136,7 @@ attention_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restr
         for (int x = 0; x < VEC; x += 4)
             *reinterpret_cast<float4*>(out_lane + x) = make_float4(acc[x], acc[x + 1], acc[x + 2], acc[x + 3]);
     }
+    if (KEEP == kKeepScores && lane == 0) stats[row] = make_float2(m_run == -INFINITY ? 0.f : m_run, inv);
     if (WRITE_P) {
         // every lane normalises the scores it wrote itself
         const float m_safe = m_run == -INFINITY ? 0.f : m_run;
@@ -156,19 +169,20 @@ __device__ __forceinline__ float softmax_step(float sc, bool live, float& m_run,
 // k row and every v row is loaded once for the four rows (the score part is the SDDMM group kernel's, the output
 // part the SpMM group kernel's, with a running softmax per row in between); then the wave
 // takes the nonzeros outside the run, row by row, the way attention_rows_kernel does.
-// With WRITE_P the raw scores of the first kGroupScoresKept columns of the run wait in LDS,
-// the others in the probs array itself; the lanes that wrote them normalise them.
+// Keeping probabilities, the raw scores of the first kGroupScoresKept columns of the run wait in
+// LDS, the others in the probs array itself; the lanes that wrote them normalise them.
 constexpr int kGroupScoresKept = 512;
 
-template <typename T, int D, bool WRITE_P>
+template <typename T, int D, int KEEP>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
                        const int* __restrict__ col, const float* __restrict__ val, const T* __restrict__ q,
                        const T* __restrict__ k, const T* __restrict__ v, float scale, float* __restrict__ out,
-                       float* probs, HeadStrides heads)
+                       float* probs, float2* __restrict__ stats, HeadStrides heads)
 {
+    constexpr bool WRITE_P = KEEP == kKeepProbs;
     q = of_head(q, heads.rows), k = of_head(k, heads.cols), v = of_head(v, heads.cols);
-    out = of_head(out, heads.rows), probs = of_head(probs, heads.nnz);
+    out = of_head(out, heads.rows), probs = of_head(probs, heads.nnz), stats = of_head(stats, heads.rows / D);
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
     __shared__ __attribute__((aligned(16))) int lds_c[kWavesPerWg * kWave];
@@ -250,6 +264,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
             if (WRITE_P && live) {
                 if (j < kGroupScoresKept) my_s[r * kGroupScoresKept + j] = sc; else probs[first[r] + j] = sc;
             }
+            if (KEEP == kKeepScores && live) probs[first[r] + j] = sc;
         }
         wave_lds_sync();
         const int nq = min(kWave / 4, (d.len - j0 + 3) / 4);
@@ -297,7 +312,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
                 if (live) sc = scale * (w * dd);
             }
             my_p[lane] = softmax_step<VEC>(sc, live, m_run[r], l_lane[r], acc[r]);
-            if (WRITE_P && live) probs[idx] = sc;
+            if (KEEP != kKeepNothing && live) probs[idx] = sc;
             wave_lds_sync();
             const int nlive = min(cnt - off, kWave);
             if (nlive == kWave)
@@ -319,6 +334,7 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
             for (int x = 0; x < VEC; x += 4)
                 *reinterpret_cast<float4*>(out_lane + x) = make_float4(acc[r][x], acc[r][x + 1], acc[r][x + 2], acc[r][x + 3]);
         }
+        if (KEEP == kKeepScores && lane == 0) stats[row0 + r] = make_float2(m_run[r] == -INFINITY ? 0.f : m_run[r], inv);
         if (WRITE_P) {
             // every lane normalises the scores it wrote itself: same walk over the run and over the rest
             const float m_safe = m_run[r] == -INFINITY ? 0.f : m_run[r];
@@ -338,13 +354,15 @@ attention_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const 
 
 template <typename T, int D>
 hipError_t launch_rows(int nheads, int M, int N, int nnz, const int* row_ptr, const int* col, const float* val, const T* q,
-                       const T* k, const T* v, float scale, float* out, float* probs, PlanRef plan, hipStream_t stream)
+                       const T* k, const T* v, float scale, float* out, float* probs, float2* stats, PlanRef plan,
+                       hipStream_t stream)
 {
     long long wgs = ((long long)M + kWavesPerWg - 1) / kWavesPerWg;
     wgs = (wgs + kXcds - 1) / kXcds * kXcds;
     if (wgs * kWgThreads >= (1ll << 32) || nheads > 65535) return hipErrorInvalidConfiguration;
     HeadStrides heads;
     heads.rows = (size_t)M * D, heads.cols = (size_t)N * D, heads.nnz = (size_t)nnz;
+    const Keep keep = probs == nullptr ? kKeepNothing : stats != nullptr ? kKeepScores : kKeepProbs;
     // a group plan is used when a wave per group fills the GPU
     RowOwners owners;
     const bool grouped = plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] >= kGroupWaveEach;
@@ -354,23 +372,29 @@ hipError_t launch_rows(int nheads, int M, int N, int nnz, const int* row_ptr, co
     }
     if (!(grouped && plan.group_counts[2] == 0)) { // (else every row is in a group)
         const dim3 grid((unsigned)wgs, (unsigned)nheads);
-        if (probs)
-            attention_rows_kernel<T, D, true><<<grid, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out, probs,
-                                                                               owners, heads);
+        if (keep == kKeepScores)
+            attention_rows_kernel<T, D, kKeepScores><<<grid, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out,
+                                                                                      probs, stats, owners, heads);
+        else if (keep == kKeepProbs)
+            attention_rows_kernel<T, D, kKeepProbs><<<grid, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out,
+                                                                                     probs, stats, owners, heads);
         else
-            attention_rows_kernel<T, D, false><<<grid, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out, probs,
-                                                                                owners, heads);
+            attention_rows_kernel<T, D, kKeepNothing><<<grid, kWgThreads, 0, stream>>>(M, row_ptr, col, val, q, k, v, scale, out,
+                                                                                       probs, stats, owners, heads);
     }
     if (grouped) {
         int gw = (owners.n_groups + kWavesPerWg - 1) / kWavesPerWg;
         gw = (gw + kXcds - 1) / kXcds * kXcds;
         const dim3 grid((unsigned)gw, (unsigned)nheads);
-        if (probs)
-            attention_group_kernel<T, D, true><<<grid, kWgThreads, 0, stream>>>(owners.n_groups, owners.groups, row_ptr, col, val,
-                                                                                q, k, v, scale, out, probs, heads);
+        if (keep == kKeepScores)
+            attention_group_kernel<T, D, kKeepScores><<<grid, kWgThreads, 0, stream>>>(
+                owners.n_groups, owners.groups, row_ptr, col, val, q, k, v, scale, out, probs, stats, heads);
+        else if (keep == kKeepProbs)
+            attention_group_kernel<T, D, kKeepProbs><<<grid, kWgThreads, 0, stream>>>(
+                owners.n_groups, owners.groups, row_ptr, col, val, q, k, v, scale, out, probs, stats, heads);
         else
-            attention_group_kernel<T, D, false><<<grid, kWgThreads, 0, stream>>>(owners.n_groups, owners.groups, row_ptr, col,
-                                                                                 val, q, k, v, scale, out, probs, heads);
+            attention_group_kernel<T, D, kKeepNothing><<<grid, kWgThreads, 0, stream>>>(
+                owners.n_groups, owners.groups, row_ptr, col, val, q, k, v, scale, out, probs, stats, heads);
     }
     return hipGetLastError();
 }
@@ -378,24 +402,27 @@ hipError_t launch_rows(int nheads, int M, int N, int nnz, const int* row_ptr, co
 } // namespace
 
 // nheads problems on one pattern (q, out: [nheads][M][d]; k, v: [nheads][N][d]; probs: NULL or
-// [nheads][nnz]); d: width of q, k and v rows (32, 64 or 128).
+// [nheads][nnz]; row_stats: NULL or [nheads][M][2], and then probs receives the scaled scores
+// and row_stats the (maximum, 1 / sum) of every row); d: width of q, k and v rows (32, 64 or 128).
 template <typename T>
 hipError_t attention_launch(int nheads, int M, int N, int nnz, int d, const int* row_ptr, const int* col, const float* val,
-                            const T* q, const T* k, const T* v, float scale, float* out, float* probs, PlanRef plan,
-                            hipStream_t stream)
+                            const T* q, const T* k, const T* v, float scale, float* out, float* probs, float* row_stats,
+                            PlanRef plan, hipStream_t stream)
 {
     if (M <= 0 || nheads <= 0) return hipSuccess;
+    if (row_stats != nullptr && probs == nullptr) return hipErrorInvalidValue;
+    float2* stats = reinterpret_cast<float2*>(row_stats);
     switch (d) {
-    case 32: return launch_rows<T, 32>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
-    case 64: return launch_rows<T, 64>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
-    case 128: return launch_rows<T, 128>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, plan, stream);
+    case 32: return launch_rows<T, 32>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, stats, plan, stream);
+    case 64: return launch_rows<T, 64>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, stats, plan, stream);
+    case 128: return launch_rows<T, 128>(nheads, M, N, nnz, row_ptr, col, val, q, k, v, scale, out, probs, stats, plan, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
 template hipError_t attention_launch<float>(int, int, int, int, int, const int*, const int*, const float*, const float*,
-                                            const float*, const float*, float, float*, float*, PlanRef, hipStream_t);
+                                            const float*, const float*, float, float*, float*, float*, PlanRef, hipStream_t);
 template hipError_t attention_launch<__half>(int, int, int, int, int, const int*, const int*, const float*, const __half*,
-                                             const __half*, const __half*, float, float*, float*, PlanRef, hipStream_t);
+                                             const __half*, const __half*, float, float*, float*, float*, PlanRef, hipStream_t);
 
 } // namespace rode

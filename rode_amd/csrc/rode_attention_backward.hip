@@ -92,17 +92,35 @@ __device__ __forceinline__ void store_floats(float* p, const float (&v)[VEC])
     for (int x = 0; x < VEC; x += 4) *reinterpret_cast<float4*>(p + x) = make_float4(v[x], v[x + 1], v[x + 2], v[x + 3]);
 }
 
+// What the forward kernel left per nonzero is the probability itself (stats == NULL) or the
+// scaled score, with the row's (maximum, 1 / sum) in stats: p = exp(score - maximum) / sum.
+struct RowStat {
+    float max = 0.f, inv = 1.f;
+    bool scores = false;
+    __device__ __forceinline__ float prob(float kept) const { return scores ? __expf(kept - max) * inv : kept; }
+};
+__device__ __forceinline__ RowStat row_stat(const float2* stats, int row)
+{
+    RowStat r;
+    if (stats != nullptr) {
+        const float2 s = stats[row];
+        r.max = s.x, r.inv = s.y, r.scores = true;
+    }
+    return r;
+}
+
 // ---- row pass -------------------------------------------------------------------------------
 // One wave per row of the pattern, 64 slots per step (attention_rows_kernel's walk).
 template <typename T, int D>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_backward_rows_kernel(int M, const int* __restrict__ row_ptr, const int* __restrict__ col,
                                const float* __restrict__ val, const float* __restrict__ probs,
-                               const float* __restrict__ g, const float* __restrict__ out, const T* __restrict__ k,
-                               const T* __restrict__ v, float scale, const int* __restrict__ t_slot,
+                               const float2* __restrict__ stats, const float* __restrict__ g, const float* __restrict__ out,
+                               const T* __restrict__ k, const T* __restrict__ v, float scale, const int* __restrict__ t_slot,
                                float* __restrict__ dq, float2* __restrict__ pz, RowOwners owners, HeadStrides heads)
 {
     probs = of_head(probs, heads.nnz), g = of_head(g, heads.rows), out = of_head(out, heads.rows);
+    stats = of_head(stats, heads.rows / D);
     k = of_head(k, heads.cols), v = of_head(v, heads.cols), dq = of_head(dq, heads.rows), pz = of_head(pz, heads.nnz);
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave;
@@ -123,6 +141,7 @@ attention_backward_rows_kernel(int M, const int* __restrict__ row_ptr, const int
         if (group == 0) store_floats<VEC>(dq_lane, acc);
         return;
     }
+    const RowStat stat = row_stat(stats, row);
     float g_raw[VEC], o_raw[VEC];
     load_floats<VEC>(g + (size_t)row * D + ls * VEC, g_raw);
     load_floats<VEC>(out + (size_t)row * D + ls * VEC, o_raw);
@@ -147,7 +166,7 @@ attention_backward_rows_kernel(int M, const int* __restrict__ row_ptr, const int
         const bool live = slot < e;
         const int idx = live ? slot : e - 1; // lanes past the row repeat its last slot with weight 0
         const int c = col[idx];
-        const float w = val[idx], p = probs[idx];
+        const float w = val[idx], p = stat.prob(probs[idx]);
         float dz = 0.f;
         if (off + (lane & 32) < e) { // the upper half sits out a step that has nothing for it
             const float dp = sddmm_unit<T, D, 1, false>(v_lane, a, c, D, my_c, lane) * g_scale;
@@ -175,12 +194,13 @@ template <typename T, int D>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 attention_backward_group_kernel(int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
                                 const int* __restrict__ col, const float* __restrict__ val,
-                                const float* __restrict__ probs, const float* __restrict__ g,
-                                const float* __restrict__ out, const T* __restrict__ k, const T* __restrict__ v,
-                                float scale, const int* __restrict__ t_slot, float* __restrict__ dq,
-                                float2* __restrict__ pz, HeadStrides heads)
+                                const float* __restrict__ probs, const float2* __restrict__ stats,
+                                const float* __restrict__ g, const float* __restrict__ out, const T* __restrict__ k,
+                                const T* __restrict__ v, float scale, const int* __restrict__ t_slot,
+                                float* __restrict__ dq, float2* __restrict__ pz, HeadStrides heads)
 {
     probs = of_head(probs, heads.nnz), g = of_head(g, heads.rows), out = of_head(out, heads.rows);
+    stats = of_head(stats, heads.rows / D);
     k = of_head(k, heads.cols), v = of_head(v, heads.cols), dq = of_head(dq, heads.rows), pz = of_head(pz, heads.nnz);
     using S = SpmmShape<T, D>;
     constexpr int VEC = S::kVec, LPR = S::kLpr, G = S::kGroupsWave, R = kGroupRows;
@@ -201,6 +221,9 @@ attention_backward_group_kernel(int n_groups, const RowGroup* __restrict__ group
     typename DotVec<T>::Reg a[R][E][DotVec<T>::kRegs];
     int first[R]; // per row: the slot of column j of the shared run is first[r] + j
     float delta[R], g_scale[R], g_inv[R];
+    RowStat stat[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) stat[r] = row_stat(stats, row0 + r);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         float g_raw[E][VEC], part = 0.f, big = 0.f;
@@ -275,7 +298,7 @@ attention_backward_group_kernel(int n_groups, const RowGroup* __restrict__ group
             p[r] = dz[r] = 0.f;
             to[r] = 0;
             if (live) {
-                p[r] = probs[first[r] + j];
+                p[r] = stat[r].prob(probs[first[r] + j]);
                 to[r] = t_slot[first[r] + j];
                 dz[r] = scale * val[first[r] + j] * p[r] * (dot[r] * g_scale[r] - delta[r]);
             }
@@ -337,7 +360,7 @@ attention_backward_group_kernel(int n_groups, const RowGroup* __restrict__ group
             const int at = live_slot ? slot : cnt - 1;
             const int idx = s + at + (at >= split ? jump : 0);
             const int c = col[idx];
-            const float w = val[idx], p = probs[idx];
+            const float w = val[idx], p = stat[r].prob(probs[idx]);
             float dz = 0.f;
             if (off + (lane & 32) < cnt) {
                 const float dp = sddmm_unit<T, D, 1, false>(v_lane, a_row, c, D, my_c, lane) * g_scale[r];
@@ -619,8 +642,8 @@ inline bool use_groups(const PlanRef& plan, RowOwners& owners)
 
 template <typename T, int D>
 hipError_t launch_rows(HeadStrides heads, int nheads, int M, const int* row_ptr, const int* col, const float* val,
-                       const float* probs, const float* g, const float* out, const T* k, const T* v, float scale,
-                       const int* t_slot, float* dq, float* pz, PlanRef plan, hipStream_t stream)
+                       const float* probs, const float2* stats, const float* g, const float* out, const T* k, const T* v,
+                       float scale, const int* t_slot, float* dq, float* pz, PlanRef plan, hipStream_t stream)
 {
     const int wgs = wave_grid(M);
     if (wgs < 0 || nheads > 65535) return hipErrorInvalidConfiguration;
@@ -628,11 +651,11 @@ hipError_t launch_rows(HeadStrides heads, int nheads, int M, const int* row_ptr,
     const bool grouped = use_groups(plan, owners);
     float2* pairs = reinterpret_cast<float2*>(pz);
     if (!(grouped && plan.group_counts[2] == 0)) // (else every row is in a group)
-        attention_backward_rows_kernel<T, D><<<dim3(wgs, nheads), kWgThreads, 0, stream>>>(M, row_ptr, col, val, probs, g, out, k, v,
-                                                                                            scale, t_slot, dq, pairs, owners, heads);
+        attention_backward_rows_kernel<T, D><<<dim3(wgs, nheads), kWgThreads, 0, stream>>>(
+            M, row_ptr, col, val, probs, stats, g, out, k, v, scale, t_slot, dq, pairs, owners, heads);
     if (grouped)
         attention_backward_group_kernel<T, D><<<dim3(wave_grid(owners.n_groups), nheads), kWgThreads, 0, stream>>>(
-            owners.n_groups, owners.groups, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pairs, heads);
+            owners.n_groups, owners.groups, row_ptr, col, val, probs, stats, g, out, k, v, scale, t_slot, dq, pairs, heads);
     return hipGetLastError();
 }
 
@@ -661,17 +684,18 @@ hipError_t launch_cols(HeadStrides heads, int nheads, int N, const int* t_row_pt
 // (p, dz) in the order of the transposed pattern; t_slot: for every nonzero, its slot there.
 template <typename T>
 hipError_t attention_backward_rows_launch(int nheads, int M, int N, int nnz, int d, const int* row_ptr, const int* col,
-                                          const float* val, const float* probs, const float* g, const float* out, const T* k,
-                                          const T* v, float scale, const int* t_slot, float* dq, float* pz, PlanRef plan,
-                                          hipStream_t stream)
+                                          const float* val, const float* probs, const float* row_stats, const float* g,
+                                          const float* out, const T* k, const T* v, float scale, const int* t_slot, float* dq,
+                                          float* pz, PlanRef plan, hipStream_t stream)
 {
     if (M <= 0 || nheads <= 0) return hipSuccess;
+    const float2* stats = reinterpret_cast<const float2*>(row_stats);
     HeadStrides heads;
     heads.rows = (size_t)M * d, heads.cols = (size_t)N * d, heads.nnz = (size_t)nnz;
     switch (d) {
-    case 32: return launch_rows<T, 32>(heads, nheads, M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
-    case 64: return launch_rows<T, 64>(heads, nheads, M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
-    case 128: return launch_rows<T, 128>(heads, nheads, M, row_ptr, col, val, probs, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
+    case 32: return launch_rows<T, 32>(heads, nheads, M, row_ptr, col, val, probs, stats, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
+    case 64: return launch_rows<T, 64>(heads, nheads, M, row_ptr, col, val, probs, stats, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
+    case 128: return launch_rows<T, 128>(heads, nheads, M, row_ptr, col, val, probs, stats, g, out, k, v, scale, t_slot, dq, pz, plan, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -694,9 +718,9 @@ hipError_t attention_backward_cols_launch(int nheads, int M, int N, int nnz, int
 
 template hipError_t attention_backward_rows_launch<float>(int, int, int, int, int, const int*, const int*, const float*,
                                                           const float*, const float*, const float*, const float*, const float*,
-                                                          float, const int*, float*, float*, PlanRef, hipStream_t);
+                                                          const float*, float, const int*, float*, float*, PlanRef, hipStream_t);
 template hipError_t attention_backward_rows_launch<__half>(int, int, int, int, int, const int*, const int*, const float*,
-                                                           const float*, const float*, const float*, const __half*,
+                                                           const float*, const float*, const float*, const float*, const __half*,
                                                            const __half*, float, const int*, float*, float*, PlanRef, hipStream_t);
 template hipError_t attention_backward_cols_launch<float>(int, int, int, int, int, const int*, const int*, const float*,
                                                           const float*, const float*, float*, float*, PlanRef, hipStream_t);

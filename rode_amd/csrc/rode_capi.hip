@@ -373,10 +373,11 @@ static bool group_plan_only(const rode_hip_plans* plans, int rows, rode::PlanRef
 
 int rode_hip_attention_forward_batched(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,
                                        const int* d_column_indices, const float* d_values, const void* d_q, const void* d_k,
-                                       const void* d_v, float scale, float* d_out, float* d_probs, const rode_hip_plans* plans,
-                                       void* stream)
+                                       const void* d_v, float scale, float* d_out, float* d_probs, float* d_row_stats,
+                                       const rode_hip_plans* plans, void* stream)
 {
     if (heads < 0 || M < 0 || N < 0 || nnz < 0 || !d_row_offsets) return hipErrorInvalidValue;
+    if (d_row_stats && (!d_probs || ((uintptr_t)d_row_stats & 7) != 0)) return hipErrorInvalidValue;
     rode::PlanRef plan;
     if (!group_plan_only(plans, M, plan)) return hipErrorInvalidValue;
     if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
@@ -385,11 +386,13 @@ int rode_hip_attention_forward_batched(int dtype, int heads, int M, int N, int n
     if (dtype == RODE_DENSE_F32)
         return rode::attention_launch<float>(heads, M, N, nnz, d, d_row_offsets, d_column_indices, d_values,
                                              static_cast<const float*>(d_q), static_cast<const float*>(d_k),
-                                             static_cast<const float*>(d_v), scale, d_out, d_probs, plan, as_stream(stream));
+                                             static_cast<const float*>(d_v), scale, d_out, d_probs, d_row_stats, plan,
+                                             as_stream(stream));
     if (dtype == RODE_DENSE_F16)
         return rode::attention_launch<__half>(heads, M, N, nnz, d, d_row_offsets, d_column_indices, d_values,
                                               static_cast<const __half*>(d_q), static_cast<const __half*>(d_k),
-                                              static_cast<const __half*>(d_v), scale, d_out, d_probs, plan, as_stream(stream));
+                                              static_cast<const __half*>(d_v), scale, d_out, d_probs, d_row_stats, plan,
+                                              as_stream(stream));
     return hipErrorInvalidValue;
 }
 
@@ -399,16 +402,17 @@ int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets
 {
     // (one head: nobody asks where the next head's operands start)
     return rode_hip_attention_forward_batched(dtype, 1, M, 0, 0, d, d_row_offsets, d_column_indices, d_values, d_q, d_k, d_v,
-                                              scale, d_out, d_probs, plans, stream);
+                                              scale, d_out, d_probs, nullptr, plans, stream);
 }
 
 int rode_hip_attention_backward_rows(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,
                                      const int* d_column_indices, const float* d_values, const float* d_probs,
-                                     const float* d_grad_out, const float* d_out, const void* d_k, const void* d_v, float scale,
-                                     const int* d_t_slot, float* d_grad_q, float* d_pairs, const rode_hip_plans* plans,
-                                     void* stream)
+                                     const float* d_row_stats, const float* d_grad_out, const float* d_out, const void* d_k,
+                                     const void* d_v, float scale, const int* d_t_slot, float* d_grad_q, float* d_pairs,
+                                     const rode_hip_plans* plans, void* stream)
 {
     if (heads < 0 || M < 0 || N < 0 || nnz < 0 || !d_row_offsets) return hipErrorInvalidValue;
+    if (((uintptr_t)d_row_stats & 7) != 0) return hipErrorInvalidValue;
     rode::PlanRef plan;
     if (!group_plan_only(plans, M, plan)) return hipErrorInvalidValue;
     if (d != 32 && d != 64 && d != 128) return hipErrorInvalidValue;
@@ -420,12 +424,12 @@ int rode_hip_attention_backward_rows(int dtype, int heads, int M, int N, int nnz
         return hipErrorInvalidValue;
     if (dtype == RODE_DENSE_F32)
         return rode::attention_backward_rows_launch<float>(heads, M, N, nnz, d, d_row_offsets, d_column_indices, d_values, d_probs,
-                                                           d_grad_out, d_out, static_cast<const float*>(d_k),
+                                                           d_row_stats, d_grad_out, d_out, static_cast<const float*>(d_k),
                                                            static_cast<const float*>(d_v), scale, d_t_slot, d_grad_q, d_pairs,
                                                            plan, as_stream(stream));
     if (dtype == RODE_DENSE_F16)
         return rode::attention_backward_rows_launch<__half>(heads, M, N, nnz, d, d_row_offsets, d_column_indices, d_values, d_probs,
-                                                            d_grad_out, d_out, static_cast<const __half*>(d_k),
+                                                            d_row_stats, d_grad_out, d_out, static_cast<const __half*>(d_k),
                                                             static_cast<const __half*>(d_v), scale, d_t_slot, d_grad_q, d_pairs,
                                                             plan, as_stream(stream));
     return hipErrorInvalidValue;

@@ -53,18 +53,20 @@ hipError_t group_plan_launch(int M, const int* row_ptr, const int* col, int* pla
 // nonzeros per launch (operands head after head).  (plan: only a group plan is used)
 template <typename T>
 hipError_t attention_launch(int nheads, int M, int N, int nnz, int d, const int* row_ptr, const int* col, const float* val,
-                            const T* q, const T* k, const T* v, float scale, float* out, float* probs, PlanRef plan,
-                            hipStream_t stream);
+                            const T* q, const T* k, const T* v, float scale, float* out, float* probs, float* row_stats,
+                            PlanRef plan, hipStream_t stream);
 
 // Gradient of the attention kernel (rode_attention_backward.hip): the row pass over the
 // pattern, then the column pass over the transposed pattern (plan: only a group plan is used,
 // of the pattern the pass walks).  pz: nheads x 2 * nnz floats, written by the first in the
 // order of the transposed pattern (t_slot: every nonzero's slot there), read by the second.
+// row_stats: NULL when probs holds probabilities, else what attention_launch wrote beside the
+// scores in probs.
 template <typename T>
 hipError_t attention_backward_rows_launch(int nheads, int M, int N, int nnz, int d, const int* row_ptr, const int* col,
-                                          const float* val, const float* probs, const float* g, const float* out, const T* k,
-                                          const T* v, float scale, const int* t_slot, float* dq, float* pz, PlanRef plan,
-                                          hipStream_t stream);
+                                          const float* val, const float* probs, const float* row_stats, const float* g,
+                                          const float* out, const T* k, const T* v, float scale, const int* t_slot, float* dq,
+                                          float* pz, PlanRef plan, hipStream_t stream);
 template <typename T>
 hipError_t attention_backward_cols_launch(int nheads, int M, int N, int nnz, int d, const int* t_row_ptr, const int* t_col,
                                           const float* pz, const float* g, const T* q, float* dk, float* dv, PlanRef plan,

@@ -211,9 +211,16 @@ def test_fused_attention_kernel_against_the_three_kernels(d, half):
     q, k, v = mk(m, 1.5), mk(n, 1.5), mk(n, 1.0)
     mask = make_csr(rp, col, val, m, n, d)
     scale = 0.37
-    out, probs = _attention_call(mask, mask.values, q, k, v, scale, True)
-    out_only, none = _attention_call(mask, mask.values, q, k, v, scale, False)
-    assert none is None and torch.equal(out, out_only)
+    out, probs, none = _attention_call(mask, mask.values, q, k, v, scale, "probs")
+    assert none is None
+    out_only, none, none2 = _attention_call(mask, mask.values, q, k, v, scale, None)
+    assert none is None and none2 is None and torch.equal(out, out_only)
+    # the other form of what a gradient needs: scaled scores and (maximum, 1 / sum) per row
+    out_s, scores, stats = _attention_call(mask, mask.values, q, k, v, scale, "scores")
+    assert torch.equal(out, out_s) and stats.shape == (m, 2)
+    row_of = torch.repeat_interleave(torch.arange(m, device=DEV), torch.from_numpy(np.diff(rp)).to(DEV))
+    from_scores = torch.exp(scores - stats[row_of, 0]) * stats[row_of, 1]
+    assert (from_scores - probs).abs().max().item() <= 2e-6
     # fp64 on the host
     q64, k64, v64 = (t.double().cpu().numpy() for t in (q, k, v))
     rows = np.repeat(np.arange(m), lens)

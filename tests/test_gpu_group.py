@@ -267,9 +267,16 @@ def test_fused_attention_of_groups(d, half, m, window):
     mk = lambda r, s: torch.from_numpy((s * rng.standard_normal((r, d))).astype(np.float32)).to(DEV, dt)
     q, k, v = mk(m, 1.2), mk(n, 1.2), mk(n, 1.0)
     scale = 0.4
-    out, probs = _attention_call(mask, mask.values, q, k, v, scale, True)
-    out_only, none = _attention_call(mask, mask.values, q, k, v, scale, False)
-    assert none is None and torch.equal(out, out_only)
+    out, probs, none = _attention_call(mask, mask.values, q, k, v, scale, "probs")
+    assert none is None
+    out_only, none, none2 = _attention_call(mask, mask.values, q, k, v, scale, None)
+    assert none is None and none2 is None and torch.equal(out, out_only)
+    # the other form of what a gradient needs: scaled scores and (maximum, 1 / sum) per row
+    out_s, scores, stats = _attention_call(mask, mask.values, q, k, v, scale, "scores")
+    assert torch.equal(out, out_s) and stats.shape == (m, 2)
+    row_of = torch.repeat_interleave(torch.arange(m, device=DEV), torch.from_numpy(np.diff(rp)).to(DEV))
+    from_scores = torch.exp(scores - stats[row_of, 0]) * stats[row_of, 1]
+    assert (from_scores - probs).abs().max().item() <= 2e-6
     q64, k64, v64 = (t.double().cpu().numpy() for t in (q, k, v))
     lens = np.diff(rp)
     rows = np.repeat(np.arange(m), lens)
@@ -286,7 +293,7 @@ def test_fused_attention_of_groups(d, half, m, window):
     assert np.abs(probs.cpu().numpy() - ref_p).max() <= tol
     assert np.abs(out.cpu().numpy() - ref_out).max() <= tol * max(1.0, np.abs(ref_out).max())
     assert not out[torch.from_numpy(lens == 0).to(DEV)].any()
-    out2, probs2 = _attention_call(plain, plain.values, q, k, v, scale, True)
+    out2, probs2, _ = _attention_call(plain, plain.values, q, k, v, scale, "probs")
     assert (out - out2).abs().max().item() <= tol * max(1.0, out2.abs().max().item())
     assert (probs - probs2).abs().max().item() <= tol
 
@@ -381,6 +388,17 @@ def test_fused_attention_gradients_of_groups(d, half):
         finally:
             autograd.FUSED_BACKWARD = "auto"
         grads[fused_backward] = (q.grad.clone(), k.grad.clone(), v.grad.clone())
+    # the gradient entry points take either form of what the forward call kept: probabilities,
+    # or scaled scores with every row's (maximum, 1 / sum)
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    g_out = w.contiguous()
+    kept = {}
+    for keep in ("probs", "scores"):
+        out_k, per_nonzero, stats = autograd._attention_call(mask, mask.values, qd, kd, vd, scale, keep)
+        kept[keep] = autograd._attention_backward_call(mask, mask_t, mask.transposed_slots(), per_nonzero, stats, g_out,
+                                                       out_k, qd, kd, vd, scale)
+    for a, b in zip(kept["probs"], kept["scores"]):
+        assert (a - b).abs().max().item() <= 1e-5 * b.abs().max().item()
     q64, k64, v64 = (t.detach().double().requires_grad_() for t in (q, k, v))
     A = _dense(rp, col, val, m, n)
     has = torch.from_numpy(np.diff(rp) > 0).to(DEV)
