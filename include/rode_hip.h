@@ -376,10 +376,11 @@ int rode_hip_csr_softmax_backward_f32(int M, const int* d_row_offsets, const flo
  *   d_q [M x d], d_k, d_v [columns x d]   row-major, 16-byte aligned
  *   d_out        float [M x d]; rows without nonzeros are written as zeros
  *   d_probs      NULL, or float [nnz] that receives p (what a gradient needs)
- *   plans        NULL, or the plans of this pattern: a group plan with at least 2048 groups
- *                with a run is used (the rows of a group then share one wave, and every k
- *                and v row of the group's run is loaded once for its four rows); the other
- *                plans are ignored
+ *   plans        NULL, or the plans of this pattern: a group plan with at least 1024 groups
+ *                with a run (2048 for fp16 operands) is used (the rows of a group then share
+ *                one wave, and every k and v row of the group's run is loaded once for its
+ *                four rows; with fewer groups a wave per row keeps more of the GPU busy); the
+ *                other plans are ignored
  */
 int rode_hip_attention_forward(int dtype, int M, int d, const int* d_row_offsets, const int* d_column_indices,
                                const float* d_values, const void* d_q, const void* d_k, const void* d_v,
@@ -428,7 +429,8 @@ int rode_hip_attention_forward_batched(int dtype, int heads, int M, int N, int n
  *                inverse of the d_perm that rode_hip_csr_transpose returns
  *   d_pairs      float [2 * nnz], 16-byte aligned: written by the first call, read by the second
  *   plans / t_plans   NULL, or the plans of the pattern / of the transposed pattern (a group
- *                plan with at least 2048 groups with a run is used, as in the forward call)
+ *                plan is used from the same number of groups on as in the forward call,
+ *                t_plans from 1024 groups on)
  * Rows (columns) without nonzeros get zero gradients.  Both calls queue on `stream`.
  */
 int rode_hip_attention_backward_rows(int dtype, int heads, int M, int N, int nnz, int d, const int* d_row_offsets,

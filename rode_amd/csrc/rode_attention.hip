@@ -365,7 +365,7 @@ hipError_t launch_rows(int nheads, int M, int N, int nnz, const int* row_ptr, co
     const Keep keep = probs == nullptr ? kKeepNothing : stats != nullptr ? kKeepScores : kKeepProbs;
     // a group plan is used when a wave per group fills the GPU
     RowOwners owners;
-    const bool grouped = plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] >= kGroupWaveEach;
+    const bool grouped = plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] >= attention_groups_min<T>();
     if (grouped) {
         owners.groups = reinterpret_cast<const RowGroup*>(plan.groups + kGroupHeaderInts);
         owners.n_groups = plan.group_counts[0];

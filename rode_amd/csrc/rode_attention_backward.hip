@@ -630,9 +630,9 @@ inline int wave_grid(long long items)
 }
 
 // (a group plan is used when a wave per group fills the GPU, as in the forward pass)
-inline bool use_groups(const PlanRef& plan, RowOwners& owners)
+inline bool use_groups(const PlanRef& plan, int groups_min, RowOwners& owners)
 {
-    const bool grouped = plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] >= kGroupWaveEach;
+    const bool grouped = plan.groups != nullptr && plan.group_counts != nullptr && plan.group_counts[1] >= groups_min;
     if (grouped) {
         owners.groups = reinterpret_cast<const RowGroup*>(plan.groups + kGroupHeaderInts);
         owners.n_groups = plan.group_counts[0];
@@ -648,7 +648,7 @@ hipError_t launch_rows(HeadStrides heads, int nheads, int M, const int* row_ptr,
     const int wgs = wave_grid(M);
     if (wgs < 0 || nheads > 65535) return hipErrorInvalidConfiguration;
     RowOwners owners;
-    const bool grouped = use_groups(plan, owners);
+    const bool grouped = use_groups(plan, attention_groups_min<T>(), owners);
     float2* pairs = reinterpret_cast<float2*>(pz);
     if (!(grouped && plan.group_counts[2] == 0)) // (else every row is in a group)
         attention_backward_rows_kernel<T, D><<<dim3(wgs, nheads), kWgThreads, 0, stream>>>(
@@ -666,7 +666,7 @@ hipError_t launch_cols(HeadStrides heads, int nheads, int N, const int* t_row_pt
     const int wgs = wave_grid(N);
     if (wgs < 0 || nheads > 65535) return hipErrorInvalidConfiguration;
     RowOwners owners;
-    const bool grouped = use_groups(plan, owners);
+    const bool grouped = use_groups(plan, kAttentionColsGroupsMin, owners);
     const float2* pairs = reinterpret_cast<const float2*>(pz);
     if (!(grouped && plan.group_counts[2] == 0))
         attention_backward_cols_kernel<T, D><<<dim3(wgs, nheads), kWgThreads, 0, stream>>>(N, t_row_ptr, t_col, pairs, g, q, dk, dv,

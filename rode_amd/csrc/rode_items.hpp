@@ -399,7 +399,22 @@ __device__ __forceinline__ WindowDesc plan_residue_desc(const int* __restrict__ 
 // only)  [1] groups with a run  [2] rows outside those groups  [3] zero; then one RowGroup per group; then three
 // ints per row of scratch for the plan's own kernels.
 constexpr int kGroupHeaderInts = 4;
-constexpr int kGroupWaveEach = 2048; // from this many groups with a run on, a group is one wave's work, below it a workgroup's
+// SpMM / SDDMM: from this many groups with a run on, a group is one wave's work, below it a
+// workgroup's (measured on the attention-mask benchmark cut down to 128 .. 4096 groups: a wave
+// per group is 20-30 % faster from 256 groups on and level at 128).
+constexpr int kGroupWaveEach = 128;
+// Attention kernels: from this many groups with a run on, the rows of groups go to the group
+// kernels; below it every row gets a wave of its own.  Measured on the same benchmark cut
+// down, forward + both gradient kernels, group kernels against a wave per row: 2048 groups
+// 0.174 against 0.278 ms (fp16 operands 0.166 / 0.211); 1024 groups 0.133 / 0.148 (fp16: 0.128 /
+// 0.110, the column pass alone 0.030 / 0.044); 512 groups 0.120 / 0.083.  Hence by operand
+// size for the passes over the pattern, and one figure for the pass over its transpose.
+template <typename T>
+constexpr int attention_groups_min()
+{
+    return sizeof(T) == 2 ? 2048 : 1024;
+}
+constexpr int kAttentionColsGroupsMin = 1024;
 static_assert(sizeof(RowGroup) == 32 && kGroupRows == kWavesPerWg, "one wave per row of a group");
 __host__ __device__ inline int row_groups(int M) { return M / kGroupRows; }
 __host__ __device__ inline size_t group_plan_ints(int M)
