@@ -322,3 +322,30 @@ def test_heads_in_one_launch_match_the_loop_over_heads(half):
     assert (chain - batched[0]).abs().max().item() <= tol * max(1.0, chain.abs().max().item())
     with pytest.raises(ValueError, match="heads"):
         sparse_attention(mask, q, k[:2], v, fused=True)
+
+
+@pytest.mark.gpu
+def test_row_statistics_need_the_per_nonzero_array():
+    """The forward entry point writes scores and row statistics together or not at all, and
+    wants the statistics 8-byte aligned: both misuses are refused before anything is launched."""
+    import ctypes
+    from gpu_common import DEV
+    from rode_amd import _lib
+    lib = _lib.load()
+    m = n = 64
+    rp = torch.arange(0, 2 * m + 1, 2, dtype=torch.int32, device=DEV)
+    col = (torch.arange(2 * m, device=DEV) % n).int()
+    val = torch.ones(2 * m, device=DEV)
+    q = torch.randn(m, 32, device=DEV)
+    out, kept, stats = torch.empty(m, 32, device=DEV), torch.empty(2 * m, device=DEV), torch.empty(m * 2 + 1, device=DEV)
+    s = torch.cuda.current_stream(DEV).cuda_stream
+
+    def call(kept_ptr, stats_ptr):
+        return lib.rode_hip_attention_forward_batched(_lib.DENSE_CODE["f32"], 1, m, n, 2 * m, 32, rp.data_ptr(), col.data_ptr(),
+                                                      val.data_ptr(), q.data_ptr(), q.data_ptr(), q.data_ptr(), 1.0,
+                                                      out.data_ptr(), kept_ptr, stats_ptr, None, s)
+    assert call(None, stats.data_ptr()) != 0
+    assert call(kept.data_ptr(), stats.data_ptr() + 4) != 0
+    assert call(kept.data_ptr(), stats.data_ptr()) == 0
+    torch.cuda.synchronize()
+    assert torch.isfinite(stats[: 2 * m]).all() and (stats[1 : 2 * m : 2] > 0).all()
