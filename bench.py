@@ -340,7 +340,7 @@ def main():
         b.synchronize()
         return a.elapsed_time(b) / reps  # ms
 
-    # preprocessing (excluded from the step, reported on its own): the four kernels of one call
+    # preprocessing (excluded from the step, reported on its own): the two launches of one call
     from rode_amd import rode_sddmm_hip
     cap = rode_sddmm_hip.preprocess_capacity(m, nnz, csr.config["seg_length"], 4)
     p_blk = torch.empty(cap + 1, dtype=torch.int32, device=dev)
@@ -388,14 +388,14 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # the SpMM block kernel sums rows of 32..1024 slots whole when there are >= 16384 segments
+    # the SpMM block kernel sums rows of 32..1024 slots whole when there are >= 1024 segments (kOwnedMinSegments)
     hub_min_len = hub.counts[2] if hub is not None else 0
     group_rows = None
     if grp is not None:
         group_rows = np.zeros(m, dtype=bool)
         group_rows[: 4 * grp.counts[0]] = np.repeat(grp.groups()[:, 1] > 0, 4)
     split_sddmm = work_split(row_ptr, col, n, 0, hub_min_len, group_rows)
-    split_spmm = work_split(row_ptr, col, n, 1024 if csr.m1 >= 16384 else 0, hub_min_len, group_rows)
+    split_spmm = work_split(row_ptr, col, n, 1024 if csr.m1 >= 1024 else 0, hub_min_len, group_rows)
     per_kernel = {}
     for name, ms in kernels.items():
         if name.startswith("attention"):

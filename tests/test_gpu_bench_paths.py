@@ -146,6 +146,40 @@ def test_benchmarked_attention_forward_against_host_softmax(half):
     assert np.abs(got - ref).max() <= tol * max(1.0, np.abs(ref).max())
 
 
+@pytest.mark.parametrize("half", [False, True], ids=["f32", "f16"])
+def test_benchmarked_attention_training_step_against_dense_autograd(half):
+    """Configuration 5 at full size, forward and gradient kernels as ``bench.py --chain --fused
+    scores --train`` runs them (group kernels on the mask and on its transpose), against dense
+    fp64 autograd on the GPU; a random weight per output element makes every gradient matter."""
+    from gpu_common import DEV
+    from rode_amd import rode_sddmm_hip, sparse_attention
+    m, n, rp, col, val, base = _bench_matrix("c5_attention")
+    assert _plan_kind(base) == "group" and base.plan.counts[1] >= 2048
+    d = 64
+    csr = _with_k(base, d)
+    csr_t, _ = csr.transpose(with_values=False)
+    assert isinstance(csr_t.plan, rode_sddmm_hip.GroupPlan) and csr_t.plan.counts[1] >= 1024
+    dt = torch.float16 if half else torch.float32
+    g = torch.Generator(device=DEV).manual_seed(501)
+    q, k, v = (torch.randn(r, d, device=DEV, generator=g).to(dt).requires_grad_() for r in (m, n, n))
+    w = torch.randn(m, d, device=DEV, generator=g)
+    (sparse_attention(csr, q, k, v, fused=True) * w).sum().backward()
+    q64, k64, v64 = (x.detach().double().requires_grad_() for x in (q, k, v))
+    rows = torch.repeat_interleave(torch.arange(m, device=DEV), torch.from_numpy(np.diff(rp)).to(DEV))
+    cols = torch.from_numpy(col).to(DEV).long()
+    scores = torch.full((m, n), float("-inf"), dtype=torch.float64, device=DEV)
+    weight = torch.zeros((m, n), dtype=torch.float64, device=DEV)
+    weight[rows, cols] = torch.from_numpy(val).to(DEV).double()
+    logits = (q64 @ k64.t()) * weight * d ** -0.5
+    scores = torch.where(weight != 0, logits, scores)
+    ((torch.softmax(scores, dim=1) @ v64) * w.double()).sum().backward()
+    tol = 3e-3 if half else 2e-5
+    for got, want in ((q.grad, q64.grad), (k.grad, k64.grad), (v.grad, v64.grad)):
+        assert (got.double() - want).abs().max().item() <= tol * want.abs().max().item()
+    del scores, weight, logits
+    torch.cuda.empty_cache()
+
+
 def test_auto_config_longest_segment_length_runs():
     """A matrix for which ``auto_config`` returns its largest segment length, 2048 (enough
     segments, 90th percentile of the rows with block segments above 1024), through both ops."""
