@@ -33,6 +33,10 @@ VALU_PEAK_TFLOPS = 78.6
 # LDS reads: 107 bytes per clock and CU is what ds_read_b128 of random rows sustains on this GPU
 # (measured with a stand-alone gather loop; conflict-free reads reach 205)
 LDS_PEAK_GBS = 107.0 * CUS * CLOCK_HZ / 1e9
+# Vector memory pipe (address unit + L1 of a CU): 64 bytes per clock and CU; a stand-alone loop of
+# 16-byte-per-lane gathers of 128..512-byte rows sustains 57-60 B/clk/CU from an L1-resident table and
+# 53-55 from an L2-resident one on this GPU
+VMEM_PEAK_GBS = 64.0 * CUS * CLOCK_HZ / 1e9
 TOL = {"f32": 1e-4, "f16": 2e-3}  # max over rows of |err|_inf / |ref row|_1
 
 
@@ -449,14 +453,20 @@ def main():
            "traffic_frac": None if traffic is None else round(traffic / dom_ms / 1e6 / HBM_PEAK_GBS, 4),
            "gather_model_frac": round(dom["gather_model_GBs"] / HBM_PEAK_GBS, 4)}
     # Which resource binds the kernel: HBM when its measured traffic moves at half the peak or
-    # more; else whichever of the vector ALUs (instructions issued x 4 clocks per wavefront
-    # instruction over the SIMD-clocks of the launch) and the LDS pipe (its active cycles over
-    # the CU-clocks of the launch) is busier, from the counters of the same profile.
+    # more; else whichever is busiest of the vector ALUs (instructions issued x 4 clocks per
+    # wavefront instruction over the SIMD-clocks of the launch), the LDS pipe (its active cycles
+    # over the CU-clocks of the launch) and the vector memory pipe (the bytes its loads ask for over
+    # 64 bytes per clock and CU; the bytes are the smaller of two upper estimates: vector loads
+    # issued x 1024, i.e. every load taken as 16 bytes per lane, which the gathers are, and a dense
+    # row plus 8 bytes per nonzero, which is what kernels without row sharing gather), from the
+    # counters of the same profile.
     bound, busy = "hbm", {}
     if entry is not None and traffic is not None and "valu_insts" in entry:
         clocks = dom_ms * 1e-3 * CLOCK_HZ
+        vmem_GBs = min(entry["vmem_reads"] * 1024 / dom_ms / 1e6, dom["gather_model_GBs"])
         busy = {"hbm": hbm["traffic_frac"], "valu": round(entry["valu_insts"] * 4 / (clocks * SIMDS), 4),
-                "lds": round(entry["lds_active_cycles"] / (clocks * CUS), 4)}
+                "lds": round(entry["lds_active_cycles"] / (clocks * CUS), 4),
+                "vmem": round(vmem_GBs / VMEM_PEAK_GBS, 4)}
         if windowed:  # the window kernels read every nonzero's dense row from LDS: bytes over the measured read rate
             busy["lds"] = max(busy["lds"], round(dom["GFLOPs"] * dom_ms * 1e6 / (2.0 * k) * k * elem / dom_ms / 1e6 / LDS_PEAK_GBS, 4))
         if busy["hbm"] < 0.5:
@@ -470,6 +480,10 @@ def main():
         ach = knnz_dom * k * elem / dom_ms / 1e6  # every nonzero's dense row read from LDS once
         top = {"achieved": round(ach, 1), "peak": round(LDS_PEAK_GBS, 1), "unit": "GB/s", "frac": round(ach / LDS_PEAK_GBS, 4),
                "peak_is": "LDS read pipe: 107 B per clock and CU for 128-bit reads of random rows (measured), x 256 CUs x 2.4 GHz"}
+    elif bound == "vmem":
+        top = {"achieved": round(vmem_GBs, 1), "peak": round(VMEM_PEAK_GBS, 1), "unit": "GB/s",
+               "frac": round(vmem_GBs / VMEM_PEAK_GBS, 4),
+               "peak_is": "vector memory pipe: 64 B per clock and CU x 256 CUs x 2.4 GHz; achieved = bytes the vector loads ask for"}
     else:
         top = {k2: hbm[k2] for k2 in ("achieved", "peak", "unit", "frac")}
     roofline = {"bound": bound, "kernel": dominant, **top, "traffic": traffic, "traffic_source": traffic_note,
