@@ -90,7 +90,8 @@ int rode_hip_preprocess_host(int seg_length, int k_block, int vec_len, int M, co
  * hipErrorOutOfMemory (2) before anything is launched.  The first call on a device looks
  * up the array's address (no allocation; make that call outside stream capture).  Every
  * call on one GPU uses that GPU's one array: calls that overlap in time on the same GPU
- * (different streams or host threads) race; calls queued on one stream do not.  The
+ * (different streams) race; calls queued on one stream do not, from whichever host threads
+ * they come (the launches of a call are queued under a lock).  The
  * caller clears nothing between calls: each call begins with a fill kernel over the part
  * of the array it is going to use (a kernel, not a memset, so the call can be captured).
  */

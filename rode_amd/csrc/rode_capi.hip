@@ -8,6 +8,7 @@
 #include "rode_items.hpp"
 
 #include <cstdio>
+#include <mutex>
 
 static_assert(RODE_HIP_STATIC_MAX_ROWS == rode::kPreprocessStaticMaxRows, "header and library disagree");
 static_assert(RODE_HIP_PLAN_RESIDUE_CHUNK == rode::kPlanResidueChunk && RODE_HIP_WINDOW_ROWS == rode::kResidueWindowRowsMax,
@@ -53,6 +54,11 @@ int rode_hip_preprocess_static(int seg_length, int k_block, int vec_len, int M, 
     void* ws = nullptr;
     const hipError_t e = rode::preprocess_static_workspace(&ws);
     if (e != hipSuccess) return e;
+    // The two launches of a call (the fill of the scratch, then the kernel that uses it) are
+    // queued together: host threads that call at the same time for one stream - the default
+    // stream of RoDe_preprocess, say - get their calls one after the other on the GPU.
+    static std::mutex queueing;
+    std::lock_guard<std::mutex> lock(queueing);
     return rode::preprocess_launch(seg_length, k_block, vec_len, M, d_row_ptr, d_block_r_ind, d_st_off,
                                    d_residue_r_ind, d_n_blk, d_n_res, ws, capacity_blocks, as_stream(stream));
 }
@@ -571,8 +577,8 @@ void RoDe_preprocess(int N_SEG, int blockX, int vecLen, int M, const int* row_pt
     // The signature carries no capacity: the caller's arrays are trusted to hold
     // the result, as in the reference.  Nor does it carry scratch: the library's own fixed
     // array serves every matrix it can hold (no allocation, the call only queues kernels on
-    // the default stream; calls that overlap in time on one GPU must not use this entry
-    // point), a larger one gets scratch for the call.
+    // the default stream, where calls run one after the other whichever host thread made
+    // them), a larger one gets scratch for the call.
     if (M <= RODE_HIP_STATIC_MAX_ROWS) {
         report("RoDe_preprocess", rode_hip_preprocess_static(N_SEG, blockX, vecLen, M, row_ptr, block_r_ind, st_off,
                                                              residue_r_ind, n_blk, n_res, 0x7fffffff, nullptr));

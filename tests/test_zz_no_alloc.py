@@ -60,3 +60,44 @@ def test_static_scratch_entry_point_rejects_what_it_cannot_hold():
     assert b"memory" in lib.rode_hip_error_string(2).lower()
     assert lib.rode_hip_preprocess_static(0, 32, 4, 4, p, p, p, p, p, p + 4, 16, None) == 1
     assert lib.rode_hip_preprocess_static(512, 32, 4, 4, None, p, p, p, p, p + 4, 16, None) == 1
+
+
+def test_static_scratch_calls_from_several_host_threads_to_one_stream():
+    """Host threads that call at the same time for the same stream: every call's two launches
+    are queued together, so the calls run one after the other on the GPU and each finds the
+    scratch as its own fill left it."""
+    import threading
+    from helpers import random_row_ptr
+    from rode_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(12)
+    inputs = [random_row_ptr(rng, 20_000 + 7_000 * i, 12, long_rows=4, long_len=3_000) for i in range(6)]
+    want = [_run(lib, "workspace", rp, 128, dev) for rp in inputs]
+    stream = torch.cuda.current_stream().cuda_stream
+    arrays, codes = [], [None] * len(inputs)
+    for rp in inputs:
+        m, nnz = len(rp) - 1, int(rp[-1])
+        cap = (nnz + 3 * m) // 128 + m
+        arrays.append((m, cap, torch.from_numpy(rp).to(dev), torch.full((cap + 1,), -1, dtype=torch.int32, device=dev),
+                       torch.full((cap + 2,), -1, dtype=torch.int32, device=dev),
+                       torch.full((m,), -1, dtype=torch.int32, device=dev), torch.full((2,), -1, dtype=torch.int32, device=dev)))
+    torch.cuda.synchronize()
+    start = threading.Barrier(len(inputs))
+
+    def call(i):
+        m, cap, d_rp, blk, st, res, cnt = arrays[i]
+        start.wait()
+        for _ in range(20):  # (ctypes releases the interpreter lock during the call)
+            codes[i] = lib.rode_hip_preprocess_static(128, 32, 4, m, d_rp.data_ptr(), blk.data_ptr(), st.data_ptr(),
+                                                      res.data_ptr(), cnt.data_ptr(), cnt.data_ptr() + 4, cap, stream)
+    threads = [threading.Thread(target=call, args=(i,)) for i in range(len(inputs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert codes == [0] * len(inputs)
+    for (m, cap, d_rp, blk, st, res, cnt), ref in zip(arrays, want):
+        for a, b, name in zip((blk, st, res, cnt), ref, ("block_r_ind", "st_off", "residue_r_ind", "counts")):
+            assert a.cpu().numpy().tobytes() == b.tobytes(), f"{name} differs (rows {m})"
