@@ -101,3 +101,52 @@ def test_static_scratch_calls_from_several_host_threads_to_one_stream():
     for (m, cap, d_rp, blk, st, res, cnt), ref in zip(arrays, want):
         for a, b, name in zip((blk, st, res, cnt), ref, ("block_r_ind", "st_off", "residue_r_ind", "counts")):
             assert a.cpu().numpy().tobytes() == b.tobytes(), f"{name} differs (rows {m})"
+
+
+def test_static_scratch_entry_point_in_a_hip_graph():
+    """What the entry point is for: recorded into a HIP graph (its scratch is cleared by a fill
+    kernel, so no memset node is recorded) and replayed on new row pointers of the same shape,
+    with eager work and synchronisations between the replays; every replay against the
+    workspace entry point."""
+    from helpers import random_row_ptr
+    from rode_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(13)
+    m, seg = 300_000, 128
+    variants = [random_row_ptr(rng, m, mean, long_rows=8, long_len=20_000) for mean in (6, 30, 11, 19)]
+    cap = max((int(rp[-1]) + 3 * m) // seg + m for rp in variants)
+    d_rp = torch.zeros(m + 1, dtype=torch.int32, device=dev)
+    blk = torch.empty(cap + 1, dtype=torch.int32, device=dev)
+    st = torch.empty(cap + 2, dtype=torch.int32, device=dev)
+    res = torch.empty(m, dtype=torch.int32, device=dev)
+    cnt = torch.empty(2, dtype=torch.int32, device=dev)
+
+    def call(stream):
+        code = lib.rode_hip_preprocess_static(seg, 32, 4, m, d_rp.data_ptr(), blk.data_ptr(), st.data_ptr(), res.data_ptr(),
+                                              cnt.data_ptr(), cnt.data_ptr() + 4, cap, stream)
+        assert code == 0, code
+
+    d_rp.copy_(torch.from_numpy(variants[0]))
+    call(torch.cuda.current_stream().cuda_stream)  # (the first call on a device looks the scratch up: outside the capture)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for replay, rp in enumerate(variants + variants[:1]):
+        d_rp.copy_(torch.from_numpy(rp))
+        for t in (blk, st, res, cnt):
+            t.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want_blk, want_st, want_res, want_cnt = _run(lib, "workspace", rp, seg, dev)
+        n_blk, n_res = (int(x) for x in cnt.cpu().numpy())
+        assert (n_blk, n_res) == tuple(int(x) for x in want_cnt), f"replay {replay}: counts differ"
+        assert blk[:n_blk].cpu().numpy().tobytes() == want_blk[:n_blk].tobytes(), f"replay {replay}: block_r_ind differs"
+        assert st[: n_blk + 1].cpu().numpy().tobytes() == want_st[: n_blk + 1].tobytes(), f"replay {replay}: st_off differs"
+        assert res[:n_res].cpu().numpy().tobytes() == want_res[:n_res].tobytes(), f"replay {replay}: residue_r_ind differs"
