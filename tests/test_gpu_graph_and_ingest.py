@@ -62,6 +62,67 @@ def test_hip_graph_replays_match_eager():
         assert (C - c_eager * sign).abs().max().item() <= 1e-5 * c_scale, f"replay {replay}: SpMM differs"
 
 
+def test_hip_graph_replays_of_the_attention_step():
+    """The attention forward and its two gradient kernels allocate nothing either: recorded into
+    one graph and replayed on new operands, against the eager calls."""
+    import ctypes
+    from gpu_common import DEV, make_csr
+    from test_gpu_group import _window_matrix
+    from rode_amd import _lib, rode_sddmm_hip
+    lib = _lib.load()
+    rng = np.random.default_rng(3)
+    m, d = 6000, 64
+    n = m + 300
+    rp, col, val = _window_matrix(rng, m, n, 96, 6)
+    val = rng.uniform(0.5, 1.5, len(col)).astype(np.float32)
+    csr = make_csr(rp, col, val, m, n, d, locality=True)
+    csr_t, _ = csr.transpose(with_values=False)
+    t_slot = csr.transposed_slots()
+    nnz = csr.nnz
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    q, k, v, g = (torch.randn(r, d, device=DEV, generator=gen) for r in (m, n, n, m))
+    out, kept, stats = torch.empty(m, d, device=DEV), torch.empty(nnz, device=DEV), torch.empty(m, 2, device=DEV)
+    dq, dk, dv = torch.empty(m, d, device=DEV), torch.empty(n, d, device=DEV), torch.empty(n, d, device=DEV)
+    pairs = torch.empty(2 * nnz, device=DEV)
+    group = lambda c: c.plan if isinstance(c.plan, rode_sddmm_hip.GroupPlan) else None
+    plans, plans_t = rode_sddmm_hip.plans_struct(group(csr)), rode_sddmm_hip.plans_struct(group(csr_t))
+    kind = _lib.DENSE_CODE["f32"]
+
+    def step(s):
+        _lib.check(lib.rode_hip_attention_forward_batched(
+            kind, 1, m, n, nnz, d, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), 0.3, out.data_ptr(), kept.data_ptr(), stats.data_ptr(),
+            ctypes.byref(plans), s), "forward")
+        _lib.check(lib.rode_hip_attention_backward_rows(
+            kind, 1, m, n, nnz, d, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
+            kept.data_ptr(), stats.data_ptr(), g.data_ptr(), out.data_ptr(), k.data_ptr(), v.data_ptr(), 0.3,
+            t_slot.data_ptr(), dq.data_ptr(), pairs.data_ptr(), ctypes.byref(plans), s), "rows")
+        _lib.check(lib.rode_hip_attention_backward_cols(
+            kind, 1, m, n, nnz, d, csr_t.row_offsets.data_ptr(), csr_t.column_indices.data_ptr(), pairs.data_ptr(),
+            g.data_ptr(), q.data_ptr(), dk.data_ptr(), dv.data_ptr(), ctypes.byref(plans_t), s), "cols")
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        q.copy_(torch.randn(m, d, device=DEV, generator=gen))  # new operands, eager work between the replays
+        g.mul_(0.5)
+        step(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        want = [t.clone() for t in (out, dq, dk, dv)]
+        for t in (out, dq, dk, dv, kept, pairs):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("out", "dq", "dk", "dv"), (out, dq, dk, dv), want):
+            assert torch.equal(got, ref), f"replay {replay}: {name} differs"
+
+
 def test_matrix_market_file_through_the_path(tmp_path):
     import scipy.io
     import scipy.sparse as sp
