@@ -45,6 +45,10 @@ class RoDeCSR:
         self.k = k
         self.nnz = values.numel()
         self.device = torch.device(device)
+        if self.device.type == "cuda" and self.device.index is None and torch.cuda.is_available():
+            # "cuda" means the current GPU; tensors created there report "cuda:<index>", which is
+            # what the operand checks of the ops compare with
+            self.device = torch.device("cuda", torch.cuda.current_device())
         self.row_offsets_cpu = row_offsets.to(dtype=torch.int32, device="cpu").contiguous()
         if isinstance(config, str):
             if config != "auto":
@@ -159,6 +163,18 @@ class RoDeCSR:
             return None
         plan = rode_sddmm_hip.hub_plan(self.row_offsets, self.column_indices, self.m, self.n, int(min_len))
         return plan if plan.usable else None
+
+    def call_plans(self, spmm_width=None, spmm_elem_bytes=4):
+        """The ``rode_hip_plans`` struct of this matrix for an SDDMM call (no arguments) or an
+        SpMM call of the given dense width and output element size; built once per pattern
+        and kind of call (the plan and the segment length never change after construction)."""
+        key = ("plans", spmm_width, spmm_elem_bytes)
+        plans = self._shared.get(key)
+        if plans is None:
+            plans = rode_sddmm_hip.plans_struct(self.plan, spmm_width, spmm_elem_bytes, True,
+                                                seg_length=self.config["seg_length"])
+            self._shared[key] = plans
+        return plans
 
     def with_values(self, values):
         """The same pattern and decomposition with other values (no preprocessing is
@@ -275,7 +291,7 @@ def rode_sddmm(sparse_matrix, lhs, rhs, values=None):
         sparse_matrix.block_indices, sparse_matrix.residue_indices, sparse_matrix.st_offsets,
         sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,
         sparse_matrix.values, m, n, lhs.contiguous(), rhs.contiguous(), k, plan=sparse_matrix.plan,
-        seg_length=sparse_matrix.config["seg_length"])
+        seg_length=sparse_matrix.config["seg_length"], checked_lists=True, plans=sparse_matrix.call_plans())
 
 
 def torch_sddmm_reference(sparse_csr, lhs_matrix, rhs_matrix):

@@ -30,7 +30,31 @@ def _check_input(x, name):
 
 
 def _stream_handle(device):
+    """Raw handle of PyTorch's current stream on ``device`` (the direct lookup costs a
+    fraction of a microsecond; building a ``torch.cuda.Stream`` object costs several)."""
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None and device.index is not None:
+        return raw(device.index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(device):
+    """Context in which ``device`` is the current GPU; nothing to enter or leave when it
+    already is (the usual case, and the switch costs microseconds per call)."""
+    if device.index is None or torch.cuda.current_device() == device.index:
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def preprocess_capacity(m, nnz, seg_length, vec_len):
@@ -314,7 +338,7 @@ def _dense_kind(lhs_matrix, rhs_matrix, lhs_name, rhs_name):
 
 
 def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, n,
-                  lhs_matrix, rhs_matrix, k_version, plan=None, seg_length=0):
+                  lhs_matrix, rhs_matrix, k_version, plan=None, seg_length=0, checked_lists=False, plans=None):
     """``rode_sddmm_cuda.sddmm_forward`` (``rode_sddmm_cuda.cu:136-249``).
 
     Differences from the reference, none of which changes a result: any k_version
@@ -323,16 +347,21 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
     kernels are queued on PyTorch's current stream instead of two streams that
     are created, synchronised and destroyed per call (``:203-246``).  ``plan``: a
     plan made from these very lists, or None; ``seg_length``: the segment length the lists were
-    made with (``preprocess``'s third argument), 0 when not known.
+    made with (``preprocess``'s third argument), 0 when not known.  ``checked_lists``: the
+    index tensors and values are a ``RoDeCSR``'s own (device, layout and type were settled
+    when it was built); ``plans``: the ``plans_struct`` of (plan, seg_length), kept by the caller.
     """
-    for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
-                    (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
-                    (values, "values"), (lhs_matrix, "lhs_matrix"), (rhs_matrix, "rhs_matrix")):
-        _check_input(t, name)
-    for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
-                    (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices")):
-        _check(t.dtype == torch.int32, f"{name} must be int32")
-    _check(values.dtype == torch.float32, "values must be float32")
+    if not checked_lists:
+        for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
+                        (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
+                        (values, "values")):
+            _check_input(t, name)
+        for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
+                        (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices")):
+            _check(t.dtype == torch.int32, f"{name} must be int32")
+        _check(values.dtype == torch.float32, "values must be float32")
+    _check_input(lhs_matrix, "lhs_matrix")
+    _check_input(rhs_matrix, "rhs_matrix")
     kind = _dense_kind(lhs_matrix, rhs_matrix, "lhs_matrix", "rhs_matrix")
 
     k = lhs_matrix.size(1)
@@ -345,13 +374,15 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
     _check(rhs_matrix.size(0) == n, "rhs_matrix rows must equal n")
     _check(rhs_matrix.size(1) == k, "rhs_matrix cols must equal k")
 
-    out = torch.zeros(nnz, dtype=torch.float32, device=values.device)
     if m1 == 0 and m2 == 0:
-        return out
+        return torch.zeros(nnz, dtype=torch.float32, device=values.device)
+    # (every nonzero is in exactly one work item and every work item stores its outputs: nothing to clear)
+    out = torch.empty(nnz, dtype=torch.float32, device=values.device)
     lib = _lib.load()
-    with torch.cuda.device(values.device):
+    with _on_device(values.device):
         s = _stream_handle(values.device)
-        plans = plans_struct(plan, seg_length=seg_length)
+        if plans is None:
+            plans = plans_struct(plan, seg_length=seg_length)
         code = lib.rode_hip_sddmm_planned(_lib.DENSE_CODE[kind], 0, m1, m2, n, k, block_indices.data_ptr(),
                                           residue_indices.data_ptr(), st_offsets.data_ptr(), row_offsets.data_ptr(),
                                           column_indices.data_ptr(), values.data_ptr(), lhs_matrix.data_ptr(),
@@ -361,7 +392,7 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
 
 
 def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, k,
-                 dense_matrix, out=None, whole_lists=True, plan=None, seg_length=0):
+                 dense_matrix, out=None, whole_lists=True, plan=None, seg_length=0, checked_lists=False, plans=None):
     """C = A_csr @ dense_matrix through ``rode_hip_spmm_f32`` / ``_f16``
     (host API ``RoDe_SpMM/RoDeSpmm.h:4-8``).  ``dense_matrix`` is (k, n) with n a
     multiple of 4 (8 for fp16, 2 for fp64), fp32 / fp16 (fp32 ``values``) or fp64 (fp64 ``values``); the
@@ -370,14 +401,17 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     short rows overwrite).  ``whole_lists`` promises that the index tensors are the
     complete decomposition (always true for a ``RoDeCSR``); pass False for a slice.
     ``plan``: a ``WindowPlan`` made from these very lists, a ``HubPlan`` of this pattern
-    (used only with ``whole_lists``), or None."""
-    for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
-                    (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
-                    (values, "values"), (dense_matrix, "dense_matrix")):
-        _check_input(t, name)
-    for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
-                    (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices")):
-        _check(t.dtype == torch.int32, f"{name} must be int32")
+    (used only with ``whole_lists``), or None.  ``checked_lists`` / ``plans``: as for
+    ``sddmm_forward`` (``plans``: of (plan, this width and element size, whole_lists, seg_length))."""
+    if not checked_lists:
+        for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
+                        (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
+                        (values, "values")):
+            _check_input(t, name)
+        for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
+                        (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices")):
+            _check(t.dtype == torch.int32, f"{name} must be int32")
+    _check_input(dense_matrix, "dense_matrix")
     if dense_matrix.dtype == torch.float64:
         _check(values.dtype == torch.float64, "values must be float64 when dense_matrix is float64")
     else:
@@ -395,7 +429,7 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
             return torch.zeros((m, n), dtype=out_dtype, device=values.device)
         # only the rows the kernels add to (or skip) need clearing, the others are overwritten
         out = torch.empty((m, n), dtype=out_dtype, device=values.device)
-        with torch.cuda.device(values.device):
+        with _on_device(values.device):
             _lib.check(lib.rode_hip_spmm_clear_rows(m, n, out.element_size(), row_offsets.data_ptr(), out.data_ptr(),
                                                     _stream_handle(values.device)), "rode_hip_spmm_clear_rows")
     else:
@@ -404,9 +438,10 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     if m1 == 0 and m2 == 0:
         return out
     dtype = {torch.float32: 0, torch.float16: 1, torch.float64: 2}[dense_matrix.dtype]  # RODE_DENSE_*
-    with torch.cuda.device(values.device):
+    with _on_device(values.device):
         s = _stream_handle(values.device)
-        plans = plans_struct(plan, n, out.element_size(), whole_lists, seg_length=seg_length)
+        if plans is None:
+            plans = plans_struct(plan, n, out.element_size(), whole_lists, seg_length=seg_length)
         code = lib.rode_hip_spmm_planned(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
                                          values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
                                          block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),

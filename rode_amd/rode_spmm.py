@@ -31,4 +31,5 @@ def rode_spmm(sparse_matrix, dense, out=None, values=None):
         sparse_matrix.block_indices, sparse_matrix.residue_indices, sparse_matrix.st_offsets,
         sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,
         sparse_matrix.values, sparse_matrix.m, sparse_matrix.n, dense.contiguous(), out, plan=sparse_matrix.plan,
-        seg_length=sparse_matrix.config["seg_length"])
+        seg_length=sparse_matrix.config["seg_length"], checked_lists=True,
+        plans=sparse_matrix.call_plans(dense.shape[1], 4))

@@ -494,3 +494,18 @@ def test_many_short_segments_write_exactly_their_entries(seg):
         got = got[pad:pad + nnz]
         assert ((got != -777.0) == expect).all(), "written entries differ from the host model"
         assert np.max(np.abs(got[expect] - ref[expect]) / np.maximum(scale[expect], 1e-30)) <= 2e-6
+
+
+def test_device_given_without_an_index():
+    """``device="cuda"`` means the current GPU: the matrix reports the device its tensors
+    report, so operands made with ``.to("cuda")`` pass the ops' device checks."""
+    from rode_amd import RoDeCSR, rode_sddmm, rode_spmm
+    torch.manual_seed(5)
+    csr = RoDeCSR.from_random(300, 200, 20, "cuda", k=32)
+    assert csr.device == csr.values.device and csr.device.index is not None
+    lhs, rhs = torch.randn(300, 32).to("cuda"), torch.randn(200, 32).to("cuda")
+    out = rode_sddmm(csr, lhs, rhs)
+    C = rode_spmm(csr, rhs)
+    dense = csr.to_torch_sparse_csr().to_dense()
+    assert torch.allclose(C, dense @ rhs, atol=1e-4, rtol=1e-4)
+    assert out.shape == (csr.nnz,) and torch.isfinite(out).all()
