@@ -83,8 +83,8 @@ def _softmax_call(fn_name, row_offsets, a, b, scale):
     if a.numel() == 0:  # a pattern without nonzeros
         return out
     m = row_offsets.numel() - 1
-    with torch.cuda.device(a.device):
-        s = torch.cuda.current_stream(a.device).cuda_stream
+    with rode_sddmm_hip._on_device(a.device):
+        s = rode_sddmm_hip._stream_handle(a.device)
         if b is None:
             code = lib.rode_hip_csr_softmax_f32(m, row_offsets.data_ptr(), a.data_ptr(), out.data_ptr(), scale, s)
         else:
@@ -141,14 +141,14 @@ def _attention_call(csr, values, q, k, v, scale, keep):
     if nnz == 0:  # no nonzeros: nothing attends to anything
         return torch.zeros(lead + (m, d), dtype=torch.float32, device=q.device), probs, stats
     out = torch.empty(lead + (m, d), dtype=torch.float32, device=q.device)
-    plans = rode_sddmm_hip.plans_struct(csr.plan if isinstance(csr.plan, rode_sddmm_hip.GroupPlan) else None)
-    with torch.cuda.device(q.device):
+    plans = csr.call_plans()  # (the attention kernels use a group plan and ignore the other kinds)
+    with rode_sddmm_hip._on_device(q.device):
         code = lib.rode_hip_attention_forward_batched(
             _lib.DENSE_CODE["f16" if q.dtype == torch.float16 else "f32"], heads, m, csr.n, nnz, d,
             csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), values.data_ptr(), q.data_ptr(), k.data_ptr(),
             v.data_ptr(), float(scale), out.data_ptr(), probs.data_ptr() if keep else None,
             stats.data_ptr() if stats is not None else None, ctypes.byref(plans),
-            torch.cuda.current_stream(q.device).cuda_stream)
+            rode_sddmm_hip._stream_handle(q.device))
     _lib.check(code, "rode_hip_attention_forward_batched")
     return out, probs, stats
 
@@ -167,10 +167,9 @@ def _attention_backward_call(csr, csr_t, t_slot, probs, stats, g, out, q, k, v, 
     dk = torch.empty(k.shape, dtype=torch.float32, device=q.device)
     dv = torch.empty(v.shape, dtype=torch.float32, device=q.device)
     pairs = torch.empty(2 * probs.numel(), dtype=torch.float32, device=q.device)
-    group = lambda c: c.plan if isinstance(c.plan, rode_sddmm_hip.GroupPlan) else None
-    plans, plans_t = rode_sddmm_hip.plans_struct(group(csr)), rode_sddmm_hip.plans_struct(group(csr_t))
-    with torch.cuda.device(q.device):
-        s = torch.cuda.current_stream(q.device).cuda_stream
+    plans, plans_t = csr.call_plans(), csr_t.call_plans()
+    with rode_sddmm_hip._on_device(q.device):
+        s = rode_sddmm_hip._stream_handle(q.device)
         _lib.check(lib.rode_hip_attention_backward_rows(
             kind, heads, m, n, nnz, d, csr.row_offsets.data_ptr(), csr.column_indices.data_ptr(), csr.values.data_ptr(),
             probs.data_ptr(), stats.data_ptr() if stats is not None else None, g.data_ptr(), out.data_ptr(), k.data_ptr(),
