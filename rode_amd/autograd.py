@@ -297,7 +297,10 @@ def sparse_attention(mask, q, k, v, scale=None, fused="auto"):
         elif fused == "auto" and mask.max_row_length > FUSED_MAX_ROW:
             why = "rows too long"
         if why is None:
-            return FusedAttentionFunction.apply(mask, q, k, v, scale)
+            if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+                return FusedAttentionFunction.apply(mask, q, k, v, scale)
+            # nothing to differentiate: the kernel keeps nothing for a gradient
+            return _attention_call(mask, mask.values, q.contiguous(), k.contiguous(), v.contiguous(), scale, None)[0]
         if fused is True:
             raise ValueError(f"the fused attention kernel does not apply: {why}")
     if q.dim() == 3:  # the three kernels take one head at a time
