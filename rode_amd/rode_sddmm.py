@@ -2,6 +2,8 @@
 ``RoDe_SDDMM/rode_sddmm.py``: ``RoDeCSR`` (:12-191), ``rode_sddmm`` (:194-248),
 ``torch_sddmm_reference`` (:251-304) and ``compare_results`` (:307-378).
 """
+import math
+
 import torch
 
 from . import rode_sddmm_hip
@@ -78,28 +80,32 @@ class RoDeCSR:
         rode_sddmm.py:35-38).  Measured on MI355X over the five benchmark patterns:
 
         * a small matrix (fewer than 16384 segments of 512 slots: not enough work items to
-          fill the GPU, and one wavefront per whole row is not used below that count) wants
-          short segments, 128: more wavefronts, and the kernels merge what is too short;
+          fill the GPU) wants short segments, 128: more wavefronts, and the kernels merge
+          what is too short;
         * otherwise a row should be a single segment where that is possible, so that one
           wavefront sums it whole: the power of two that holds 90 % of the rows that have
           block segments, between 512 and 2048 (attention masks: 1024; power-law graphs:
           512 - their hub rows are cut into many segments either way, and the block kernel
           adds the sums of neighbouring segments up before it updates the row of C).
         """
-        ro = row_offsets.to(dtype=torch.int64, device="cpu")
-        start, lens = ro[:-1], ro[1:] - ro[:-1]
-        aligned = lens + start % 4
-        blocked = aligned[aligned >= 32]
+        ro = row_offsets.to(device="cpu")
+        if ro.dtype not in (torch.int32, torch.int64):
+            ro = ro.to(torch.int64)
+        start = ro[:-1]
+        aligned = (ro[1:] - start) + (start & 3)
+        blocked = aligned >= 32  # rows that have block segments
+        rows = int(blocked.sum())
         seg = 512
-        if blocked.numel() > 0:
-            if int(((blocked + 511) // 512).sum()) < 16384:
+        if rows > 0:
+            segments = int((((aligned + 511) >> 9) * blocked).sum())  # at 512 slots a segment (the sum is 64-bit)
+            if segments < 16384:
                 seg = 128
             else:
-                # the smallest length that at least 90 % of those rows do not exceed (the order
-                # statistic torch.quantile(..., "higher") returns, without its 16 M element limit)
-                rank = min(blocked.numel(), int(torch.ceil(torch.tensor(0.9 * (blocked.numel() - 1), dtype=torch.float64))) + 1)
-                p90 = int(torch.kthvalue(blocked, rank).values)
-                while seg < p90 and seg < 2048:
+                # the smallest of 512, 1024, 2048 that at least 90 % of those rows do not exceed: the
+                # order statistic torch.quantile(..., "higher") returns lies at or below a length
+                # exactly when that many rows do (counting avoids quantile's 16 M element limit)
+                rank = min(rows, math.ceil(0.9 * (rows - 1)) + 1)
+                while seg < 2048 and int((blocked & (aligned <= seg)).sum()) < rank:
                     seg *= 2
         return {"seg_length": seg, "k_block": 32, "vec_len": 4}
 
@@ -153,13 +159,13 @@ class RoDeCSR:
         if slabs < self.HUB_MIN_SLABS or self.nnz == 0:
             return None
         min_len = max(self.HUB_MIN_LEN, 8 * slabs)
-        ro = self.row_offsets_cpu.to(torch.int64)
-        aligned = ro[1:] - ro[:-1] + ro[:-1] % 4
-        hub = aligned >= min_len
-        share = float((ro[1:] - ro[:-1])[hub].sum()) / self.nnz
-        if self.locality is not True and share < self.HUB_MIN_SHARE:
+        start = self.row_offsets_cpu[:-1]
+        lens = self.row_offsets_cpu[1:] - start
+        hub = (lens + (start & 3)) >= min_len  # (aligned length, as the kernels count it)
+        hub_nnz = int((lens * hub).sum())  # (summed in 64 bits)
+        if self.locality is not True and hub_nnz < self.HUB_MIN_SHARE * self.nnz:
             return None
-        if not bool(hub.any()):
+        if hub_nnz == 0:
             return None
         plan = rode_sddmm_hip.hub_plan(self.row_offsets, self.column_indices, self.m, self.n, int(min_len))
         return plan if plan.usable else None
