@@ -85,9 +85,12 @@ def test_reference_module_surface():
         rode_sddmm_hip.preprocess(rp.long(), 1700, 512, 32, 4)
 
 
-def test_cxx_reference_signature_entry_point():
+@pytest.mark.parametrize("rows,longest", [(20000, 900), (4_500_000, 70)], ids=["fixed_scratch", "beyond_the_fixed_scratch"])
+def test_cxx_reference_signature_entry_point(rows, longest):
     """RoDe_preprocess(N_SEG, blockX, vecLen, M, ...) with the reference's GPU
-    signature (Preprocess_opt/_preprocess.cu:323), called through its mangled name."""
+    signature (Preprocess_opt/_preprocess.cu:323), called through its mangled name: a matrix
+    that the library's fixed scratch holds, and one with more rows than that (4 194 304), for
+    which the call brings scratch of its own (550 tiles of 8192 rows in the scan)."""
     import ctypes
     import oracle
     from rode_amd import _lib
@@ -96,7 +99,7 @@ def test_cxx_reference_signature_entry_point():
     fn.restype = None
     fn.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 6
     rng = np.random.default_rng(5)
-    rp = np.concatenate([[0], rng.integers(0, 900, 20000)]).cumsum().astype(np.int32)
+    rp = np.concatenate([[0], rng.integers(0, longest, rows)]).cumsum().astype(np.int32)
     d_rp = torch.from_numpy(rp).cuda()
     cap = int(rp[-1]) // 512 + len(rp) + 8
     blk = torch.empty(cap, dtype=torch.int32, device="cuda")
