@@ -167,6 +167,9 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
 constexpr int kWalkSlots = 512;
 constexpr int kWalkMaxChunk = 16;
 constexpr int kWalkMinSegments = 16384; // fewer segments: a small launch needs its waves more than it minds the followers
+constexpr int kWalkMinWaves = 8192;     // a chunk is no longer than leaves this many waves (eight per SIMD)
+// (a chunk of c segments needs at least c * kWalkMinWaves segments in the list)
+__host__ __device__ inline int walk_chunk_limit(int m1) { return m1 / kWalkMinWaves > 1 ? m1 / kWalkMinWaves : 1; }
 
 __device__ __forceinline__ int block_chunk(int m1, const int* __restrict__ block_rows, const int* __restrict__ st_off)
 {
@@ -188,7 +191,7 @@ __device__ __forceinline__ int block_chunk(int m1, const int* __restrict__ block
         if (row[i][0] == row[i][1]) seg_len = max(seg_len, start[i][1] - start[i][0]);
     if (seg_len <= 0) return 1;
     seg_len = (seg_len + kBlockItems - 1) / kBlockItems * kBlockItems;
-    return min(max(kWalkSlots / seg_len, 1), kWalkMaxChunk);
+    return min(min(max(kWalkSlots / seg_len, 1), kWalkMaxChunk), walk_chunk_limit(m1));
 }
 
 // The block part of a grid has at most kBlockGridWaves waves: a launch is sized before anybody
@@ -213,8 +216,10 @@ __host__ __device__ inline int chunk_for_segments(int seg_length, int m1)
 {
     if (seg_length <= 0) return 0;
     if (m1 < kWalkMinSegments) return 1;
-    const int c = kWalkSlots / ((seg_length + kBlockItems - 1) / kBlockItems * kBlockItems);
-    return c < 1 ? 1 : (c > kWalkMaxChunk ? kWalkMaxChunk : c);
+    int c = kWalkSlots / ((seg_length + kBlockItems - 1) / kBlockItems * kBlockItems);
+    c = c < 1 ? 1 : (c > kWalkMaxChunk ? kWalkMaxChunk : c);
+    const int limit = walk_chunk_limit(m1);
+    return c < limit ? c : limit;
 }
 
 // First segment of this wave's chunk, or -1 when it has none.  Consecutive chunks share an
