@@ -496,6 +496,41 @@ def test_many_short_segments_write_exactly_their_entries(seg):
         assert np.max(np.abs(got[expect] - ref[expect]) / np.maximum(scale[expect], 1e-30)) <= 2e-6
 
 
+@pytest.mark.parametrize("seg", [32, 512])
+def test_a_wrong_segment_length_hint_changes_no_result(seg):
+    """``rode_hip_plans.seg_length`` only sizes the block kernels' grid and chunks: lists of
+    more than 16384 segments made with one length, called with the hint of another (shorter,
+    longer, not a power of two, absent) - SDDMM and SpMM against the oracle every time."""
+    import oracle
+    from gpu_common import DEV, TOL_F32
+    from helpers import sddmm_row_l1_errors, spmm_row_l1_error
+    from rode_amd import rode_sddmm_hip
+    rng = np.random.default_rng(2000 + seg)
+    m, n, k = (4000, 3000, 32) if seg == 32 else (24000, 3000, 32)
+    lens = rng.choice([0, 7, 40, 300, 900, 2500], size=m, p=[.05, .15, .2, .3, .2, .1])
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(n, size=l, replace=False)) for l in lens]).astype(np.int32)
+    val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = rng.standard_normal((n, k)).astype(np.float32)
+    nnz = len(val)
+    d_rp = torch.from_numpy(rp).to(DEV)
+    blk, st, res, m1, m2 = rode_sddmm_hip.preprocess_device(d_rp, nnz, seg, 32, 4)
+    assert m1 >= 16384
+    dcol, dval = torch.from_numpy(col).to(DEV), torch.from_numpy(val).to(DEV)
+    dl, dr = torch.from_numpy(lhs).to(DEV), torch.from_numpy(rhs).to(DEV)
+    ref, scale = oracle.sddmm_f64(rp, col, val, lhs, rhs, with_abs=True)
+    ref_c = oracle.spmm_f64(rp, col, val, rhs)
+    for hint in (seg, 0, 32, 96, 512, 4096):
+        out = rode_sddmm_hip.sddmm_forward(blk, res, st, m1, m2, d_rp, dcol, dval, m, n, dl, dr, k, seg_length=hint)
+        err, cond = sddmm_row_l1_errors(out.cpu().numpy(), ref, scale, rp)
+        assert float(err[cond <= 100].max(initial=0.0)) <= TOL_F32, (seg, hint)
+        for whole in (True, False):
+            C = rode_sddmm_hip.spmm_forward(blk, res, st, m1, m2, d_rp, dcol, dval, m, n, dr, whole_lists=whole,
+                                            seg_length=hint)
+            assert spmm_row_l1_error(C.cpu().numpy(), ref_c) <= TOL_F32, (seg, hint, whole)
+
+
 def test_device_given_without_an_index():
     """``device="cuda"`` means the current GPU: the matrix reports the device its tensors
     report, so operands made with ``.to("cuda")`` pass the ops' device checks."""
