@@ -182,8 +182,13 @@ def main():
     spmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan, k, 4, seg_length=csr.config["seg_length"]))
     sddmm_plans = ctypes.byref(rode_sddmm_hip.plans_struct(csr.plan, seg_length=csr.config["seg_length"]))
 
+    # Every row of C stored by its one work item (no row without slots, none cut into several work items):
+    # then C needs no clearing, and the kernels are told to store instead of add.
+    stores_c = csr.spmm_stores_every_row() and not args.memset_c
+    spmm_flags = _lib.SPMM_WHOLE_LISTS | (_lib.SPMM_OVERWRITE if stores_c else 0)
+
     def spmm_fn(*a, flags=0):  # the whole decomposition is passed, and the library is told so
-        return lib.rode_hip_spmm_planned(_lib.DENSE_CODE[args.dtype], _lib.SPMM_WHOLE_LISTS | flags, *a[:-2],
+        return lib.rode_hip_spmm_planned(_lib.DENSE_CODE[args.dtype], spmm_flags | flags, *a[:-2],
                                          spmm_plans, *a[-2:])
 
     def sddmm_fn(*a, flags=0):
@@ -271,6 +276,8 @@ def main():
             "attention backward, columns")
 
     def clear_c():
+        if stores_c:
+            return
         if args.memset_c:
             C.zero_()
         else:
@@ -607,7 +614,8 @@ def main():
                                    + (" + gradient (row pass + column pass)" if args.train else "")
                                    if args.fused != "no" else "step = SDDMM -> row softmax -> clear C -> SpMM (chained)")
                                   if args.chain
-                                  else "step = clear C rows + SpMM + SDDMM"),
+                                  else ("step = SpMM (C = A B into an uninitialised C: every row is stored by its one work item) + SDDMM"
+                                        if stores_c else "step = clear C rows + SpMM + SDDMM")),
                    "rows": m, "cols": n, "nnz": nnz, "K": k, "heads": args.heads, "seg_length": csr.config["seg_length"],
                    "block_segments": csr.m1, "residue_rows": csr.m2, "scale": args.scale,
                    "locality_plan": None if csr.plan is None or hub is not None or grp is not None else
@@ -618,7 +626,7 @@ def main():
                    "group_plan": None if grp is None else
                    {"groups_of_four_rows": grp.counts[0], "groups_with_a_shared_run": grp.counts[1],
                     "rows_left_to_the_list_kernels": grp.counts[2], "nnz_share": round(split_sddmm["nnz_hub"] / nnz, 3)}},
-        "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C",
+        "spmm": {"ms": round(spmm_ms, 4), "GFLOPs": round(2.0 * nnz * k / spmm_ms / 1e6, 1), "includes": "clearing C" if not stores_c else "nothing to clear: every row of C is stored by its one work item",
                  "reference_contract_ms": None if args.no_contract else round(spmm_contract_ms, 4),
                  "reference_contract": "memset of all of C + the typed entry point without the whole-lists promise "
                                        "(RoDeSpmm.cu:492-509 semantics)"},

@@ -136,6 +136,16 @@ int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const
 #define RODE_DENSE_F16 1
 #define RODE_DENSE_F64 2
 #define RODE_SPMM_WHOLE_LISTS 1
+/* With RODE_SPMM_WHOLE_LISTS: a row of C that a single work item produces is STORED instead
+ * of added to, so that C need not be zero there on entry (C = A B instead of C += A B):
+ *   - rows of fewer than 32 aligned slots (stored by every entry point, as in the reference);
+ *   - rows of at most rode_hip_spmm_overwrite_limit() aligned slots;
+ *   - the rows of the kept groups of a group plan, whatever their length.
+ * Longer rows are still added to by several work items and must be zero on entry, and rows
+ * without slots are not touched: a caller whose matrix has neither calls no
+ * rode_hip_spmm_clear_rows() at all.  (Aligned slots of a row: its nonzeros plus
+ * row_offsets[r] % 4.)  No counterpart in the reference. */
+#define RODE_SPMM_OVERWRITE 16
 /* Launch only the block-segment kernel / only the residue kernel / only the kernels of a
  * hub plan, with every other decision (which rows a single wavefront sums whole, which rows
  * the hub kernels take) made as if all were launched: for measuring one kernel, and for
@@ -288,6 +298,12 @@ int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, co
                           const int* d_column_indices, const int* d_row_offsets, const int* d_row_indices1,
                           const int* d_row_indices2, const int* d_row_seg_st_offsets, const void* d_B, void* d_C,
                           const rode_hip_plans* plans, void* stream1, void* stream2);
+
+/* The longest row, in aligned slots, that rode_hip_spmm_planned(..., RODE_SPMM_WHOLE_LISTS |
+ * RODE_SPMM_OVERWRITE, m1, ..., plans, ...) stores with one work item; 0: none of the rows
+ * with 32 aligned slots or more (few block segments: every work item adds; a hub plan).
+ * plans may be NULL.  Host arithmetic, no GPU work. */
+int rode_hip_spmm_overwrite_limit(int m1, const rode_hip_plans* plans);
 
 /*
  * Prepares an uninitialised C[M x n] for one of the SpMM calls: zeroes exactly the rows

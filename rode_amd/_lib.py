@@ -43,6 +43,7 @@ SIGNATURES = {
     "rode_hip_csr_transpose_workspace_bytes": (c_size_t, [c_int]),
     "rode_hip_csr_transpose": (c_int, [c_int] * 3 + [c_void_p] * 6 + [c_size_t, c_void_p]),
     "rode_hip_permute_f32": (c_int, [c_int] + [c_void_p] * 4),
+    "rode_hip_spmm_overwrite_limit": (c_int, [c_int, c_void_p]),
     "rode_hip_attention_forward": (c_int, [c_int] * 3 + [c_void_p] * 6 + [ctypes.c_float] + [c_void_p] * 4),
     "rode_hip_attention_forward_batched": (c_int, [c_int] * 6 + [c_void_p] * 6 + [ctypes.c_float] + [c_void_p] * 5),
     "rode_hip_attention_backward_rows": (c_int, [c_int] * 6 + [c_void_p] * 9 + [ctypes.c_float] + [c_void_p] * 5),
@@ -58,7 +59,7 @@ class Plans(ctypes.Structure):
 
 
 DENSE_CODE = {"f32": 0, "f16": 1, "f64": 2}  # RODE_DENSE_* of include/rode_hip.h
-SPMM_WHOLE_LISTS, SPMM_ONLY_BLOCK, SPMM_ONLY_RESIDUE, SPMM_ONLY_HUB = 1, 2, 4, 8  # RODE_SPMM_* flags
+SPMM_WHOLE_LISTS, SPMM_ONLY_BLOCK, SPMM_ONLY_RESIDUE, SPMM_ONLY_HUB, SPMM_OVERWRITE = 1, 2, 4, 8, 16  # RODE_SPMM_* flags
 
 _lib = None
 

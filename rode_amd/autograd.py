@@ -26,7 +26,8 @@ def _sddmm(csr, values, lhs, rhs):
 def _spmm(csr, values, dense):
     return rode_sddmm_hip.spmm_forward(csr.block_indices, csr.residue_indices, csr.st_offsets, csr.m1, csr.m2,
                                        csr.row_offsets, csr.column_indices, values.contiguous(), csr.m, csr.n,
-                                       dense.contiguous(), plan=csr.plan, seg_length=csr.config["seg_length"])
+                                       dense.contiguous(), plan=csr.plan, seg_length=csr.config["seg_length"],
+                                       every_row_stored=csr.spmm_stores_every_row())
 
 
 class SddmmFunction(torch.autograd.Function):

@@ -239,11 +239,14 @@ int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, co
                           const rode_hip_plans* plans, void* stream1, void* stream2)
 {
     (void)k;
-    constexpr int kKnown = RODE_SPMM_WHOLE_LISTS | RODE_SPMM_ONLY_BLOCK | RODE_SPMM_ONLY_RESIDUE | RODE_SPMM_ONLY_HUB;
+    constexpr int kKnown = RODE_SPMM_WHOLE_LISTS | RODE_SPMM_ONLY_BLOCK | RODE_SPMM_ONLY_RESIDUE | RODE_SPMM_ONLY_HUB |
+                           RODE_SPMM_OVERWRITE;
     static_assert(RODE_SPMM_WHOLE_LISTS == rode::kSpmmWholeLists && RODE_SPMM_ONLY_BLOCK == rode::kSpmmOnlyBlock &&
-                      RODE_SPMM_ONLY_RESIDUE == rode::kSpmmOnlyResidue && RODE_SPMM_ONLY_HUB == rode::kSpmmOnlyHub,
+                      RODE_SPMM_ONLY_RESIDUE == rode::kSpmmOnlyResidue && RODE_SPMM_ONLY_HUB == rode::kSpmmOnlyHub &&
+                      RODE_SPMM_OVERWRITE == rode::kSpmmOverwrite,
                   "header and library disagree");
     if (m1 < 0 || m2 < 0 || (flags & ~kKnown)) return hipErrorInvalidValue;
+    if ((flags & RODE_SPMM_OVERWRITE) && !(flags & RODE_SPMM_WHOLE_LISTS)) return hipErrorInvalidValue; // (one owner per row needs whole lists)
     const int only = flags & rode::kOnlyMask;
     if (only & (only - 1)) return hipErrorInvalidValue; // at most one ONLY bit
     if (m1 == 0 && m2 == 0) return hipSuccess;
@@ -268,6 +271,12 @@ int rode_hip_spmm_planned(int dtype, int flags, int m1, int m2, int k, int n, co
                                          static_cast<const double*>(d_B), static_cast<double*>(d_C), flags, plan, s1, s2);
     default: return hipErrorInvalidValue;
     }
+}
+
+int rode_hip_spmm_overwrite_limit(int m1, const rode_hip_plans* plans)
+{
+    const bool hub = plans && plans->hub && plans->hub_counts && plans->hub_counts[3] != 0 && plans->hub_counts[0] > 0;
+    return m1 < 0 ? 0 : rode::spmm_overwrite_limit(m1, hub);
 }
 
 int rode_hip_spmm_f32(int m1, int m2, int k, int n, const float* d_values, const int* d_column_indices,

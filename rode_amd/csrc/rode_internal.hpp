@@ -23,7 +23,7 @@ template <typename T> struct SpmmAcc { using type = float; };
 template <> struct SpmmAcc<double> { using type = double; };
 
 // flags: the RODE_SPMM_* bits of the C ABI
-constexpr int kSpmmWholeLists = 1, kSpmmOnlyBlock = 2, kSpmmOnlyResidue = 4, kSpmmOnlyHub = 8;
+constexpr int kSpmmWholeLists = 1, kSpmmOnlyBlock = 2, kSpmmOnlyResidue = 4, kSpmmOnlyHub = 8, kSpmmOverwrite = 16;
 constexpr int kOnlyMask = kSpmmOnlyBlock | kSpmmOnlyResidue | kSpmmOnlyHub;
 
 // A locality plan (rode_plan.hip): device array, and optionally a host copy of its four
@@ -82,6 +82,8 @@ hipError_t window_plan_launch(int m2, int dense_rows, const int* residue_rows, c
 hipError_t window_plan_rows_launch(int m2, const int* residue_rows, const int* row_ptr, const int* col, const int* plan,
                                    void* rows, hipStream_t stream);
 
+// (rode_spmm.hip) which rows an SpMM call under kSpmmOverwrite stores instead of adding to
+int spmm_overwrite_limit(int m1, bool hub_plan);
 template <typename T>
 hipError_t spmm_launch(int m1, int m2, int n, const int* block_rows, const int* residue_rows, const int* st_off,
                        const int* row_ptr, const int* col, const typename SpmmAcc<T>::type* val, const T* B,

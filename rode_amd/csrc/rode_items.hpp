@@ -47,6 +47,7 @@ struct RowOwners {
     int hub_min_len = 0;              // > 0: rows of that aligned length or more belong to the hub kernels
     const RowGroup* groups = nullptr; // the groups of a group plan, or null
     int n_groups = 0;
+    bool overwrite = false;           // SpMM: a row with a single work item is stored, not added to C
 };
 __device__ __forceinline__ bool owned_elsewhere(const RowOwners& o, int row, int aligned_len)
 {
@@ -71,6 +72,7 @@ __device__ __forceinline__ P* of_head(P* first, size_t stride)
 // belong to the previous row (unaligned start) and must not contribute.
 struct BlockItem {
     int row, base, mask, cnt;
+    bool whole = false; // the work item is its row's only one (SpMM: a row summed whole)
 };
 
 // Consecutive segments of one row whose starts fall into the same window of MERGE slots
@@ -100,6 +102,7 @@ __device__ __forceinline__ bool merged_leader(int MERGE, int seg, int m1, int la
     it.mask = start & (kVecLen - 1);
     it.base = start - it.mask;
     it.cnt = end - it.base;
+    it.whole = false;
     return true;
 }
 
@@ -140,6 +143,7 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
         it.mask = row_start & (kVecLen - 1);
         it.base = row_start - it.mask;
         it.cnt = row_end - it.base;
+        it.whole = true;
         return true;
     }
     if (owned_slots != 0)
@@ -150,6 +154,7 @@ __device__ __forceinline__ bool spmm_block_item(int seg, int m1, int owned_slots
     it.mask = start & (kVecLen - 1);
     it.base = start - it.mask;
     it.cnt = (end - start + it.mask) / kBlockItems * kBlockItems;
+    it.whole = false;
     return true;
 }
 
@@ -289,6 +294,7 @@ __device__ __forceinline__ BlockItem chunk_item(const ChunkScan& c, int i)
         it.mask = row_start & (kVecLen - 1);
         it.base = row_base;
         it.cnt = row_end - row_base;
+        it.whole = true;
         return it;
     }
     // end of the row's block part, or the start of the next leader if that comes first

@@ -50,6 +50,7 @@ constexpr int kOwnedMinSegments = 1024;
 // Without the promise the block kernel may still merge the short segments of a row that
 // the list it was given holds, when there are this many of them.
 constexpr int kMergeMinSegments = 16384;
+
 // Up to this many workgroups, and when both kernels go to the same stream, the two lists
 // are processed by one launch (spmm_pair_kernel).  Above it the residue kernel runs on its
 // own: it needs a quarter of the block kernel's registers and keeps twice the waves per CU.
@@ -133,7 +134,10 @@ __device__ __forceinline__ void spmm_sum_slots(int base, int mask, int cnt, int 
 // (bid of nblocks: the workgroup's position in the part of the grid that works on block segments)
 // WALK: 0 one wave per segment only, 1 chunks only (chunk_hint > 1), 2 either, found out here.
 // (Kernels of their own, so that the code of one way does not cost the other registers.)
-template <typename T, int TN, bool EDGE, int WALK>
+// STORE: a row's only work item stores its sum instead of adding it (owners.overwrite; a
+// kernel of its own as well: as a run-time branch it slowed the fp16 kernel of width 128
+// that never takes it from 0.97 to 1.13 ms on the power-law benchmark).
+template <typename T, int TN, bool EDGE, int WALK, bool STORE>
 __device__ __forceinline__ void
 spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int chunk_hint, RowOwners owners,
                 const int* __restrict__ block_rows,
@@ -166,9 +170,16 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int chunk_
         const T* b_lane = B + tile + (col_ok ? ls * VEC : 0);
         constexpr int EPG = VEC / G > 0 ? VEC / G : 1; // elements each lane group adds to C
         A row_total[VEC];
-        int pending = -1; // the row that row_total belongs to
+        int pending = -1;           // the row that row_total belongs to
+        bool pending_whole = false; // ... is that row's one work item
         auto flush = [&]() {
             A* c_lane = C + (size_t)pending * n + tile + ls * VEC;
+            if (STORE && pending_whole) { // (the same in every lane)
+#pragma unroll
+                for (int x = 0; x < VEC; ++x)
+                    if (group == x / EPG && col_ok) c_lane[x] = row_total[x];
+                return;
+            }
 #pragma unroll
             for (int x = 0; x < VEC; ++x)
                 if (group == x / EPG && col_ok) atomicAdd(c_lane + x, row_total[x]);
@@ -184,6 +195,7 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int chunk_
                 if (it.row != pending) {
                     if (pending >= 0) flush();
                     pending = it.row;
+                    pending_whole = it.whole;
 #pragma unroll
                     for (int x = 0; x < VEC; ++x) row_total[x] = total[x];
                 } else {
@@ -252,6 +264,12 @@ spmm_block_body(int bid, int nblocks, int m1, int n, int owned_slots, int chunk_
         if (!first_of_run) return;
     }
     A* c_lane = C + (size_t)row * n + tile + ls * VEC;
+    if (STORE && it.whole) { // the row's only work item (the same in every lane): nothing to add to
+#pragma unroll
+        for (int x = 0; x < VEC; ++x)
+            if (group == x / EPG && col_ok) c_lane[x] = total[x];
+        return;
+    }
 #pragma unroll
     for (int x = 0; x < VEC; ++x)
         if (group == x / EPG && col_ok) atomicAdd(c_lane + x, total[x]);
@@ -327,7 +345,7 @@ spmm_residue_body(int bid, int nblocks, int m2, int n, int owned_slots, RowOwner
     }
 }
 
-template <typename T, int TN, bool EDGE, int WALK>
+template <typename T, int TN, bool EDGE, int WALK, bool STORE>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_block_kernel(int m1, int n, int owned_slots, int chunk_hint, RowOwners owners, const int* __restrict__ block_rows,
                   const int* __restrict__ st_off,
@@ -335,7 +353,7 @@ spmm_block_kernel(int m1, int n, int owned_slots, int chunk_hint, RowOwners owne
                   const typename DenseVec<T>::Acc* __restrict__ val, const T* __restrict__ B,
                   typename DenseVec<T>::Acc* __restrict__ C)
 {
-    spmm_block_body<T, TN, EDGE, WALK>(blockIdx.x, gridDim.x, m1, n, owned_slots, chunk_hint, owners, block_rows, st_off,
+    spmm_block_body<T, TN, EDGE, WALK, STORE>(blockIdx.x, gridDim.x, m1, n, owned_slots, chunk_hint, owners, block_rows, st_off,
                                        row_ptr, col, val, B, C);
 }
 
@@ -353,7 +371,7 @@ spmm_residue_kernel(int m2, int n, int owned_slots, RowOwners owners, const int*
 // Both lists in one launch: the first g1 workgroups of a grid row work on block segments,
 // the others on residue rows.  For matrices so small that a launch costs as much as its
 // kernel (a kernel of a few microseconds); the two parts then also fill the GPU together.
-template <typename T, int TN, bool EDGE>
+template <typename T, int TN, bool EDGE, bool STORE>
 __global__ void __launch_bounds__(kWgThreads)
 spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, int chunk_hint, RowOwners owners,
                  const int* __restrict__ block_rows,
@@ -362,7 +380,7 @@ spmm_pair_kernel(int g1, int m1, int m2, int n, int owned_slots, int chunk_hint,
                  const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C, const int* __restrict__ plan)
 {
     if ((int)blockIdx.x < g1)
-        spmm_block_body<T, TN, EDGE, 2>(blockIdx.x, g1, m1, n, owned_slots, 0, owners, block_rows, st_off, row_ptr, col, val,
+        spmm_block_body<T, TN, EDGE, 2, STORE>(blockIdx.x, g1, m1, n, owned_slots, 0, owners, block_rows, st_off, row_ptr, col, val,
                                         B, C);
     else
         spmm_residue_body<T, TN, EDGE>(blockIdx.x - g1, gridDim.x - g1, m2, n, max(owned_slots, 0), owners, residue_rows,
@@ -381,7 +399,7 @@ template <typename T, int TN, bool EDGE, int WPG>
 __global__ void __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, const int* __restrict__ row_ptr,
                   const int* __restrict__ col, const typename DenseVec<T>::Acc* __restrict__ val,
-                  const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C)
+                  const T* __restrict__ B, typename DenseVec<T>::Acc* __restrict__ C, bool overwrite)
 {
     using S = SpmmShape<T, TN>;
     using A = typename S::Acc;
@@ -517,7 +535,7 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
             if (group == 0 && col_ok) {
                 A* c_lane = C + (size_t)(row0 + r) * n + tile + ls * VEC;
 #pragma unroll
-                for (int x = 0; x < VEC; ++x) c_lane[x] += acc[r][x]; // (long rows are accumulated into C by contract)
+                for (int x = 0; x < VEC; ++x) c_lane[x] = overwrite ? acc[r][x] : c_lane[x] + acc[r][x]; // (added by contract, unless told to store)
             }
         }
     } else {
@@ -546,7 +564,7 @@ spmm_group_kernel(int n, int n_groups, const RowGroup* __restrict__ groups, cons
                     A total = outside[x];
 #pragma unroll
                     for (int v = 0; v < WPG; ++v) total += sums[v][r][ls * VEC + x];
-                    c_lane[x] += total; // (long rows are accumulated into C by contract)
+                    c_lane[x] = overwrite ? total : c_lane[x] + total; // (added by contract, unless told to store)
                 }
             }
         }
@@ -702,6 +720,9 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
         owners.groups = reinterpret_cast<const RowGroup*>(plan.groups + kGroupHeaderInts);
         owners.n_groups = plan.group_counts[0];
     }
+    // rows with a single work item are stored instead of added (spmm_overwrite_limit says which)
+    const bool overwrite = (flags & kSpmmOverwrite) != 0;
+    owners.overwrite = overwrite && spmm_overwrite_limit(m1, hub_plan) > 0;
     const int only = flags & kOnlyMask; // one kernel family of the call (timing each on its own)
     const bool hubs = hub_plan && (only == 0 || only == kSpmmOnlyHub);
     const bool grouped = group_plan && (only == 0 || only == kSpmmOnlyHub); // (timed with the hub kernels)
@@ -725,21 +746,21 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
     hipError_t e = hipSuccess;
     if (block && residue && standard_residue && s1 == s2 && (long long)(g1 + g2) * tiles <= kPairMaxWorkgroups) {
         dim3 grid(g1 + g2, tiles);
-        spmm_pair_kernel<T, TN, EDGE><<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, chunk_hint, owners, block_rows,
-                                                                   residue_rows, st_off, row_ptr, col, val, B, C, plan.dev);
+        auto kernel = owners.overwrite ? spmm_pair_kernel<T, TN, EDGE, true> : spmm_pair_kernel<T, TN, EDGE, false>;
+        kernel<<<grid, kWgThreads, 0, s1>>>(g1, m1, m2, n, block_owned, chunk_hint, owners, block_rows, residue_rows, st_off,
+                                            row_ptr, col, val, B, C, plan.dev);
         e = hipGetLastError();
     } else {
         if (block) {
             dim3 grid(g1, tiles);
+            auto kernel = spmm_block_kernel<T, TN, EDGE, 2, false>;
             if (chunk_hint == 1)
-                spmm_block_kernel<T, TN, EDGE, 0><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows,
-                                                                               st_off, row_ptr, col, val, B, C);
+                kernel = owners.overwrite ? spmm_block_kernel<T, TN, EDGE, 0, true> : spmm_block_kernel<T, TN, EDGE, 0, false>;
             else if (chunk_hint > 1)
-                spmm_block_kernel<T, TN, EDGE, 1><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows,
-                                                                               st_off, row_ptr, col, val, B, C);
-            else
-                spmm_block_kernel<T, TN, EDGE, 2><<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows,
-                                                                               st_off, row_ptr, col, val, B, C);
+                kernel = owners.overwrite ? spmm_block_kernel<T, TN, EDGE, 1, true> : spmm_block_kernel<T, TN, EDGE, 1, false>;
+            else if (owners.overwrite)
+                kernel = spmm_block_kernel<T, TN, EDGE, 2, true>;
+            kernel<<<grid, kWgThreads, 0, s1>>>(m1, n, block_owned, chunk_hint, owners, block_rows, st_off, row_ptr, col, val, B, C);
             e = hipGetLastError();
         }
         if (residue && standard_residue) {
@@ -769,11 +790,11 @@ hipError_t launch(int m1, int m2, int n, const int* block_rows, const int* resid
             const int wgs = (owners.n_groups + kWavesPerWg - 1) / kWavesPerWg;
             dim3 grid((wgs + kXcds - 1) / kXcds * kXcds, tiles);
             spmm_group_kernel<T, TN, EDGE, 1><<<grid, kWgThreads, 0, s1>>>(n, owners.n_groups, owners.groups, row_ptr, col,
-                                                                           val, B, C);
+                                                                           val, B, C, overwrite);
         } else {
             dim3 grid((owners.n_groups + kXcds - 1) / kXcds * kXcds, tiles);
             spmm_group_kernel<T, TN, EDGE, kWavesPerWg><<<grid, kWgThreads, 0, s1>>>(n, owners.n_groups, owners.groups, row_ptr,
-                                                                                     col, val, B, C);
+                                                                                     col, val, B, C, overwrite);
         }
         e = hipGetLastError();
     }
@@ -796,6 +817,12 @@ hipError_t launch_edge(int m1, int m2, int n, const int* block_rows, const int* 
 }
 
 } // namespace
+
+// The longest row (in aligned slots) that an SpMM call with m1 block segments, the whole-lists
+// promise and kSpmmOverwrite stores with a single work item instead of adding to it; 0: none
+// of the rows that have block segments (rows of fewer than 32 aligned slots are always
+// stored, rows of kept groups of a group plan under kSpmmOverwrite as well).
+int spmm_overwrite_limit(int m1, bool hub_plan) { return m1 >= kOwnedMinSegments && !hub_plan ? kOwnedRowSlots : 0; }
 
 // n: any positive multiple of the 128-bit vector width (4 fp32, 8 fp16, 2 fp64).  The
 // dense row is cut into tiles of 32, 64 or 128 columns (at most 32 lanes per tile row);

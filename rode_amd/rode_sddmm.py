@@ -182,6 +182,30 @@ class RoDeCSR:
             self._shared[key] = plans
         return plans
 
+    def spmm_stores_every_row(self):
+        """Whether an SpMM on this matrix leaves no row of C to be cleared beforehand: every row
+        has slots (rows without any are never written) and a single work item, which then stores
+        its row instead of adding to it (``RODE_SPMM_OVERWRITE``).  Worked out once per pattern
+        from the row lengths and ``rode_hip_spmm_overwrite_limit``."""
+        cached = self._shared.get("spmm_stores_every_row")
+        if cached is None:
+            cached = False
+            if self.m > 0 and self.nnz > 0:
+                start = self.row_offsets_cpu[:-1]
+                aligned = (self.row_offsets_cpu[1:] - start) + (start & 3)  # slots as the kernels count them
+                shortest, longest = int(aligned.min()), int(aligned.max())
+                if shortest > 0:
+                    plan = self.plan
+                    if isinstance(plan, rode_sddmm_hip.GroupPlan) and plan.usable and plan.counts[2] == 0:
+                        cached = True  # every row is in a kept group: one wave (or workgroup) owns it
+                    else:
+                        import ctypes
+                        from . import _lib
+                        limit = _lib.load().rode_hip_spmm_overwrite_limit(self.m1, ctypes.byref(self.call_plans()))
+                        cached = longest < 32 or longest <= limit
+            self._shared["spmm_stores_every_row"] = cached
+        return cached
+
     def with_values(self, values):
         """The same pattern and decomposition with other values (no preprocessing is
         repeated): how the output of one op becomes the sparse operand of the next,

@@ -392,7 +392,8 @@ def sddmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offset
 
 
 def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets, column_indices, values, m, k,
-                 dense_matrix, out=None, whole_lists=True, plan=None, seg_length=0, checked_lists=False, plans=None):
+                 dense_matrix, out=None, whole_lists=True, plan=None, seg_length=0, checked_lists=False, plans=None,
+                 every_row_stored=False):
     """C = A_csr @ dense_matrix through ``rode_hip_spmm_f32`` / ``_f16``
     (host API ``RoDe_SpMM/RoDeSpmm.h:4-8``).  ``dense_matrix`` is (k, n) with n a
     multiple of 4 (8 for fp16, 2 for fp64), fp32 / fp16 (fp32 ``values``) or fp64 (fp64 ``values``); the
@@ -402,7 +403,10 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
     complete decomposition (always true for a ``RoDeCSR``); pass False for a slice.
     ``plan``: a ``WindowPlan`` made from these very lists, a ``HubPlan`` of this pattern
     (used only with ``whole_lists``), or None.  ``checked_lists`` / ``plans``: as for
-    ``sddmm_forward`` (``plans``: of (plan, this width and element size, whole_lists, seg_length))."""
+    ``sddmm_forward`` (``plans``: of (plan, this width and element size, whole_lists, seg_length)).
+    ``every_row_stored``: with ``out`` None and ``whole_lists``, the caller has checked
+    (``rode_hip_spmm_overwrite_limit``) that every row of the matrix has slots and a single
+    work item: the kernels then store their rows (``RODE_SPMM_OVERWRITE``) and nothing is cleared."""
     if not checked_lists:
         for t, name in ((block_indices, "block_indices"), (residue_indices, "residue_indices"),
                         (st_offsets, "st_offsets"), (row_offsets, "row_offsets"), (column_indices, "column_indices"),
@@ -429,10 +433,13 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
             return torch.zeros((m, n), dtype=out_dtype, device=values.device)
         # only the rows the kernels add to (or skip) need clearing, the others are overwritten
         out = torch.empty((m, n), dtype=out_dtype, device=values.device)
+        every_row_stored = every_row_stored and whole_lists
         with _on_device(values.device):
-            _lib.check(lib.rode_hip_spmm_clear_rows(m, n, out.element_size(), row_offsets.data_ptr(), out.data_ptr(),
-                                                    _stream_handle(values.device)), "rode_hip_spmm_clear_rows")
+            if not every_row_stored:
+                _lib.check(lib.rode_hip_spmm_clear_rows(m, n, out.element_size(), row_offsets.data_ptr(), out.data_ptr(),
+                                                        _stream_handle(values.device)), "rode_hip_spmm_clear_rows")
     else:
+        every_row_stored = False  # (the caller's C is added to, as the kernels' contract says)
         _check_input(out, "out")
         _check(out.dtype == out_dtype and tuple(out.shape) == (m, n), f"out must be {out_dtype} of shape (m, n)")
     if m1 == 0 and m2 == 0:
@@ -442,7 +449,8 @@ def spmm_forward(block_indices, residue_indices, st_offsets, m1, m2, row_offsets
         s = _stream_handle(values.device)
         if plans is None:
             plans = plans_struct(plan, n, out.element_size(), whole_lists, seg_length=seg_length)
-        code = lib.rode_hip_spmm_planned(dtype, _lib.SPMM_WHOLE_LISTS if whole_lists else 0, m1, m2, k, n,
+        flags = (_lib.SPMM_WHOLE_LISTS if whole_lists else 0) | (_lib.SPMM_OVERWRITE if every_row_stored else 0)
+        code = lib.rode_hip_spmm_planned(dtype, flags, m1, m2, k, n,
                                          values.data_ptr(), column_indices.data_ptr(), row_offsets.data_ptr(),
                                          block_indices.data_ptr(), residue_indices.data_ptr(), st_offsets.data_ptr(),
                                          dense_matrix.data_ptr(), out.data_ptr(), ctypes.byref(plans), s, s)

@@ -32,4 +32,5 @@ def rode_spmm(sparse_matrix, dense, out=None, values=None):
         sparse_matrix.m1, sparse_matrix.m2, sparse_matrix.row_offsets, sparse_matrix.column_indices,
         sparse_matrix.values, sparse_matrix.m, sparse_matrix.n, dense.contiguous(), out, plan=sparse_matrix.plan,
         seg_length=sparse_matrix.config["seg_length"], checked_lists=True,
-        plans=sparse_matrix.call_plans(dense.shape[1], 4))
+        plans=sparse_matrix.call_plans(dense.shape[1], 4),
+        every_row_stored=out is None and sparse_matrix.spmm_stores_every_row())

@@ -497,3 +497,96 @@ def test_measurement_flags_launch_one_kernel_of_the_pair():
                                 csr.row_offsets.data_ptr(), csr.block_indices.data_ptr(),
                                 csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(), B.data_ptr(),
                                 both.data_ptr(), None, None) != 0
+
+
+def _spmm_overwrite(csr, B, C, flags):
+    import ctypes
+    from rode_amd import _lib, rode_sddmm_hip
+    lib = _lib.load()
+    plans = rode_sddmm_hip.plans_struct(csr.plan, B.shape[1], 4, True, seg_length=csr.config["seg_length"])
+    s = torch.cuda.current_stream().cuda_stream
+    code = lib.rode_hip_spmm_planned(_lib.DENSE_CODE["f16" if B.dtype == torch.float16 else "f32"], flags, csr.m1, csr.m2, csr.n,
+                                     B.shape[1], csr.values.data_ptr(), csr.column_indices.data_ptr(), csr.row_offsets.data_ptr(),
+                                     csr.block_indices.data_ptr(), csr.residue_indices.data_ptr(), csr.st_offsets.data_ptr(),
+                                     B.data_ptr(), C.data_ptr(), ctypes.byref(plans), s, s)
+    torch.cuda.synchronize()
+    return code
+
+
+@pytest.mark.parametrize("case", ["one_segment_rows", "short_rows_only", "segments_of_32", "every_row_in_a_group", "half"])
+def test_overwrite_stores_rows_that_have_one_owner(case):
+    """RODE_SPMM_OVERWRITE: C = A B into a C full of NaN, on matrices whose every row has slots
+    and a single work item (rows summed whole by one wave, rows of fewer than 32 slots, rows of
+    kept groups); ``RoDeCSR.spmm_stores_every_row`` says so and ``rode_spmm`` then clears nothing."""
+    import oracle
+    from gpu_common import DEV, TOL_F16, TOL_F32, make_csr, round_half
+    from helpers import spmm_row_l1_error
+    from rode_amd import _lib, rode_sddmm_hip, rode_spmm
+    rng = np.random.default_rng(len(case))
+    width, half, seg, locality = 64, case == "half", None, False
+    if case in ("one_segment_rows", "half"):
+        m, n = 6000, 3000
+        lens = rng.integers(1, 900, m)     # aligned lengths up to 903 slots: whole rows (m1 >= 1024 segments)
+    elif case == "short_rows_only":
+        m, n = 5000, 3000
+        lens = rng.integers(1, 28, m)      # residue rows only
+    elif case == "segments_of_32":
+        m, n, seg = 3000, 3000, 32
+        lens = rng.integers(200, 1000, m)  # >= 16384 segments of 32 slots: a wave walks a chunk of them
+    else:
+        m, n, locality = 2000, 2400, True
+        lens = None
+    if lens is not None:
+        rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        col = np.concatenate([np.sort(rng.choice(n, size=l, replace=False)) for l in lens]).astype(np.int32)
+    else:
+        rows = [np.arange(r, r + 300, dtype=np.int32) for r in range(m)]  # a window that moves one column per row
+        rp = np.concatenate([[0], np.cumsum([len(c) for c in rows])]).astype(np.int32)
+        col = np.concatenate(rows)
+    val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
+    csr = make_csr(rp, col, val, m, n, width, seg, locality=locality)
+    if case == "every_row_in_a_group":
+        assert isinstance(csr.plan, rode_sddmm_hip.GroupPlan) and csr.plan.counts[2] == 0
+    if case == "segments_of_32":
+        assert csr.m1 >= 16384
+    assert csr.spmm_stores_every_row()
+    B = rng.standard_normal((n, width)).astype(np.float32)
+    dB = torch.from_numpy(B).to(DEV, torch.float16 if half else torch.float32)
+    C = torch.full((m, width), float("nan"), device=DEV)
+    assert _spmm_overwrite(csr, dB, C, _lib.SPMM_WHOLE_LISTS | _lib.SPMM_OVERWRITE) == 0
+    ref = oracle.spmm_f64(rp, col, val, round_half(B) if half else B)
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all(), "a row was added to, or left alone"
+    assert spmm_row_l1_error(got, ref) <= (TOL_F16 if half else TOL_F32)
+    again = rode_spmm(csr, dB).cpu().numpy()  # the op: an uninitialised C and no clearing
+    assert spmm_row_l1_error(again, ref) <= (TOL_F16 if half else TOL_F32)
+
+
+def test_overwrite_leaves_other_rows_to_the_callers_clearing():
+    """Rows of several work items are still added to and rows without slots still untouched under
+    RODE_SPMM_OVERWRITE (C holds 7 on entry); the limit function says which rows are which, and
+    the flag needs the whole-lists promise."""
+    import oracle
+    from gpu_common import DEV, make_csr
+    from rode_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(77)
+    m, n, width = 4000, 5000, 32
+    lens = rng.integers(1, 600, m)
+    lens[10], lens[11], lens[12] = 3000, 0, 1025   # several work items; no slots; one slot too many
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(n, size=l, replace=False)) for l in lens]).astype(np.int32)
+    val = rng.uniform(-1, 1, rp[-1]).astype(np.float32)
+    csr = make_csr(rp, col, val, m, n, width, locality=False)
+    assert not csr.spmm_stores_every_row()
+    limit = lib.rode_hip_spmm_overwrite_limit(csr.m1, None)
+    assert limit == 1024 and lib.rode_hip_spmm_overwrite_limit(1023, None) == 0
+    B = rng.standard_normal((n, width)).astype(np.float32)
+    dB = torch.from_numpy(B).to(DEV)
+    C = torch.full((m, width), 7.0, device=DEV)
+    assert _spmm_overwrite(csr, dB, C, _lib.SPMM_WHOLE_LISTS | _lib.SPMM_OVERWRITE) == 0
+    aligned = lens + rp[:-1] % 4
+    added = (aligned > limit) | (aligned == 0)
+    want = oracle.spmm_f64(rp, col, val, B) + np.where(added[:, None], 7.0, 0.0)
+    assert np.abs(C.cpu().numpy() - want).max() <= 1e-4 * max(1.0, np.abs(want).max())
+    assert _spmm_overwrite(csr, dB, C, _lib.SPMM_OVERWRITE) != 0   # not without the whole-lists promise
