@@ -523,7 +523,10 @@ def main():
         cnt, t_spmm, t_sddmm, c_ref, o_ref = cpu_ops(rows, 1)
         threads = oracle.num_threads()
         _, mt_spmm, mt_sddmm, _, _ = cpu_ops(rows, threads)
-        # the same rows from the GPU run, as a parity gate of this very benchmark
+        # the same rows from the GPU run, as a parity gate of this very benchmark (into a C and an
+        # `out` full of NaN: a row or an element that the step leaves alone, or adds to, shows)
+        C.fill_(float("nan"))
+        out.fill_(float("nan"))
         step()
         torch.cuda.synchronize()
         c_gpu, o_gpu = C[:rows].cpu().numpy(), out[:cnt].cpu().numpy()
@@ -587,9 +590,9 @@ def main():
         failures = []
         if not bit_exact:
             failures.append("preprocessing differs from the CPU routine")
-        if spmm_err > tol:
+        if not spmm_err <= tol:
             failures.append(f"SpMM row-L1 error {spmm_err:.3g} > {tol}")
-        if sddmm_err > tol:
+        if not sddmm_err <= tol:
             failures.append(f"SDDMM row-L1 error {sddmm_err:.3g} > {tol} on rows with condition <= 100")
         # (on those rows both errors are one draw each of rounding noise of size condition x eps,
         # in different summation orders, and the maximum is over a handful of rows: the ratio is
@@ -597,7 +600,7 @@ def main():
         if gpu_err_bad > max(10.0 * cpu_err_bad, tol):
             failures.append(f"SDDMM error {gpu_err_bad:.3g} on ill-conditioned rows exceeds ten times the reference CPU "
                             f"loop's {cpu_err_bad:.3g}")
-        if sddmm_strict > (2e-6 if args.dtype == "f32" else 2e-3):
+        if not sddmm_strict <= (2e-6 if args.dtype == "f32" else 2e-3):
             failures.append(f"SDDMM per-element error {sddmm_strict:.3g} of the summed terms' magnitude")
         if args.dtype == "f32" and ref_rule_errors:
             failures.append(f"{ref_rule_errors} outputs fail the reference tests' rule")
